@@ -1,0 +1,48 @@
+// C entry points of the kernel library.  Every function takes the HIP stream
+// to launch on, returns 0 on success and nonzero after leaving a message for
+// pa_last_error().  `dtype` codes: 0 = float32, 1 = bfloat16.  All pointers
+// are device pointers unless said otherwise; nothing here allocates.
+#pragma once
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* pa_last_error();
+int pa_device_arch(char* out, int cap);
+int pa_num_compute_units();
+
+// out[t, :] = table[ids[t], :]
+int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, void* out, int tokens, int hidden,
+                    int vocab);
+// RMSNorm of x (+ residual, which then receives the sum) with a 32-bit weight;
+// with `rows`, output row r comes from input row rows[r] and the residual is left alone.
+int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out, const int* rows,
+               int nrows, int hidden, float eps);
+// out[t, c] = silu(gate_up[t, c]) * gate_up[t, inter + c]
+int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter);
+int pa_gather_rows(void* stream, int dtype, const void* x, const int* rows, void* out, int nrows, int width);
+int pa_add_bias(void* stream, int dtype, void* y, const float* b, int tokens, int width);
+int pa_to_f32(void* stream, int dtype, const void* x, float* out, long total);
+
+// qkv [tokens, (nh + 2 nkv) * hd] -> q_out [tokens, nh, hd] (normed, rotated) and, where slots[t] >= 0,
+// K (normed, rotated) and V into caches laid out [page, nkv, page_size, hd]; slot = page * page_size + offset.
+int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_weight, const float* k_weight,
+                      const float* cos_table, const float* sin_table, const int* positions, const int* slots,
+                      void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int hd, int rot,
+                      int page_size, float eps);
+
+// C[m, n] = A[m, k] W[n, k]^T (+ bias[n]), true 32-bit arithmetic.
+int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, const void* w, const float* bias, void* c,
+                  int m, int n, int k, long lda, long ldw, long ldc);
+
+// Paged causal attention, one query token per (seq_of_token[t], positions[t]); window 0 = all keys.
+int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
+                    const int* block_table, int table_stride, const int* seq_of_token, const int* positions, void* out,
+                    int tokens, int nh, int nkv, int hd, int page_size, int window, float scale);
+
+// out[r] = index of the largest of logits[r, :], the lowest index among equals.
+int pa_argmax(void* stream, const float* logits, int* out, int rows, int vocab);
+
+#ifdef __cplusplus
+}
+#endif

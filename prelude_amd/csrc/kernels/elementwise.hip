@@ -1,0 +1,174 @@
+// Row-wise kernels: embedding gather, RMSNorm with and without the residual
+// add, SiLU*mul, row gather, bias add and the cast to 32-bit logits.
+//
+// Counterparts in the reference (formulas only; the launch shapes are ours):
+//   rmsnorm / add_rmsnorm  crates/prelude-cuda/src/kernels/kernels_src/normalization/rmsnorm.cu:12-355
+//   silu_mul               crates/prelude-cuda/src/kernels/kernels_src/elementwise/silu_mul.cu:7-43
+//   embedding, row gather  crates/prelude-core/src/models/commons/embedding.rs:29-36,
+//                          crates/prelude-core/src/models/commons/mod.rs:227-243
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+// ---- embedding gather ------------------------------------------------------
+// One block per token; 16-byte copies when the row width allows.
+template <typename T>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                    T* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  // The host refuses ids outside the vocabulary before any launch; the clamp
+  // only keeps a stray id from reading outside the table.
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* src = table + (size_t)id * hidden;
+  T* dst = out + (size_t)t * hidden;
+  constexpr int kVec = 16 / sizeof(T);
+  if (hidden % kVec == 0) {
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    uint4* d4 = reinterpret_cast<uint4*>(dst);
+    for (int i = threadIdx.x; i < hidden / kVec; i += blockDim.x) d4[i] = s4[i];
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  }
+}
+
+// ---- RMSNorm, optionally fused with the residual add --------------------
+//   s = x (+ residual)                         in 32-bit
+//   residual <- round(s)                       (only when `residual` is given and `rows` is not)
+//   out = round(s * rsqrt(mean(s^2) + eps) * w)   from the unrounded s
+// With `rows`, output row r is computed from input row rows[r] and nothing
+// is written back to the residual: the final norm of only the wanted rows.
+template <typename T>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, T* residual, const float* __restrict__ w,
+                               T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  const T* xr = x + src * hidden;
+  T* rr = residual ? residual + src * hidden : nullptr;
+  T* orow = out + (size_t)r * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float s = to_f32(xr[i]);
+    if (rr) s += to_f32(rr[i]);
+    ss += s * s;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float s = to_f32(xr[i]);
+    if (rr) s += to_f32(rr[i]);
+    if (rr && !rows) rr[i] = from_f32<T>(s);
+    orow[i] = from_f32<T>(s * inv * w[i]);
+  }
+}
+
+// ---- SiLU(gate) * up over a merged [T, 2I] input -------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / inter, c = i % inter;
+  const float g = to_f32(gate_up[t * 2 * inter + c]);
+  const float u = to_f32(gate_up[t * 2 * inter + inter + c]);
+  out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+// ---- row gather ------------------------------------------------------------
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ x, const int* __restrict__ rows, T* __restrict__ out,
+                                   int width) {
+  const T* src = x + (size_t)rows[blockIdx.x] * width;
+  T* dst = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = src[i];
+}
+
+// ---- y[t, n] += b[n] -------------------------------------------------------
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ b, int width, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  y[i] = from_f32<T>(to_f32(y[i]) + b[i % width]);
+}
+
+template <typename T>
+__global__ void to_f32_kernel(const T* __restrict__ x, float* __restrict__ out, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) out[i] = to_f32(x[i]);
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+#define PA_DISPATCH(dtype, ...)                                      \
+  do {                                                               \
+    if ((dtype) == kF32) {                                           \
+      using T = float;                                               \
+      __VA_ARGS__;                                                   \
+    } else if ((dtype) == kBF16) {                                   \
+      using T = bf16;                                                \
+      __VA_ARGS__;                                                   \
+    } else {                                                         \
+      return pa::fail("unknown element type code %d", (int)(dtype)); \
+    }                                                                \
+  } while (0)
+
+extern "C" int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, void* out, int tokens,
+                               int hidden, int vocab) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes tokens=%d hidden=%d vocab=%d", tokens,
+             hidden, vocab);
+  PA_DISPATCH(dtype, hipLaunchKernelGGL(embed_gather_kernel<T>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, ids,
+                                        (const T*)table, (T*)out, hidden, vocab));
+  return check_launch("embed_gather");
+}
+
+extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out,
+                          const int* rows, int nrows, int hidden, float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && hidden > 0, "rmsnorm: bad sizes rows=%d hidden=%d", nrows, hidden);
+  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+  PA_DISPATCH(dtype, hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(nrows), dim3(threads), 0, (hipStream_t)stream,
+                                        (const T*)x, (T*)residual, w, (T*)out, rows, hidden, eps));
+  return check_launch("rmsnorm");
+}
+
+extern "C" int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && inter > 0, "silu_mul: bad sizes tokens=%d inter=%d", tokens, inter);
+  const size_t total = (size_t)tokens * inter;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  PA_DISPATCH(dtype, hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                                        (const T*)gate_up, (T*)out, inter, total));
+  return check_launch("silu_mul");
+}
+
+extern "C" int pa_gather_rows(void* stream, int dtype, const void* x, const int* rows, void* out, int nrows,
+                              int width) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && width > 0, "gather_rows: bad sizes rows=%d width=%d", nrows, width);
+  PA_DISPATCH(dtype, hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(nrows), dim3(256), 0, (hipStream_t)stream,
+                                        (const T*)x, rows, (T*)out, width));
+  return check_launch("gather_rows");
+}
+
+extern "C" int pa_add_bias(void* stream, int dtype, void* y, const float* b, int tokens, int width) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && width > 0, "add_bias: bad sizes tokens=%d width=%d", tokens, width);
+  const size_t total = (size_t)tokens * width;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  PA_DISPATCH(dtype, hipLaunchKernelGGL(add_bias_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (T*)y, b,
+                                        width, total));
+  return check_launch("add_bias");
+}
+
+extern "C" int pa_to_f32(void* stream, int dtype, const void* x, float* out, long total) {
+  if (total == 0) return 0;
+  PA_REQUIRE(total > 0, "to_f32: bad size %ld", total);
+  const unsigned blocks = (unsigned)(((size_t)total + 255) / 256);
+  PA_DISPATCH(dtype, hipLaunchKernelGGL(to_f32_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                                        (const T*)x, out, (size_t)total));
+  return check_launch("to_f32");
+}

@@ -1,0 +1,142 @@
+// Per-head RMSNorm of Q and K, rotary position encoding, and the write of K
+// and V into the paged cache, in one launch over a merged QKV activation.
+//
+// Formula: crates/prelude-cuda/src/kernels/kernels_src/rope/qknorm_rope.cu:20-91
+// (norm over head_dim in 32-bit, then rotate-half, one rounding at the end) and
+// crates/prelude-cuda/src/kernels/kernels_src/kvcache/scatter_kv_cache.cu:19-81,
+// knorm_rope_kv_write.cu:17-113 (K is normed and rotated on its way into the
+// cache; V is copied).  Differences that are ours: the norm weights and the
+// cos/sin tables are 32-bit in every mode, the rotary width may be smaller
+// than the head (the rest passes through after the norm), the norm may be
+// absent, and the cache is laid out [page, kv_head, offset, head_dim].
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+constexpr int kQkWaves = 4;
+constexpr int kMaxHeadDim = 256;
+
+// One wavefront per (token, head) over the nh + 2*nkv heads of a token's row.
+template <typename T>
+__global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __restrict__ q_weight,
+                                      const float* __restrict__ k_weight, const float* __restrict__ cos_table,
+                                      const float* __restrict__ sin_table, const int* __restrict__ positions,
+                                      const int* __restrict__ slots, T* __restrict__ q_out,
+                                      T* __restrict__ k_cache, T* __restrict__ v_cache, int tokens, int nh, int nkv,
+                                      int hd, int rot, int page_size, float eps) {
+  __shared__ float normed[kQkWaves][kMaxHeadDim];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int heads = nh + 2 * nkv;
+  const long long unit = (long long)blockIdx.x * kQkWaves + wave;
+  const bool active = unit < (long long)tokens * heads;
+  const int t = active ? (int)(unit / heads) : 0;
+  const int h = active ? (int)(unit % heads) : 0;
+  const T* src = qkv + ((size_t)t * heads + h) * hd;
+
+  // Where this head goes.
+  T* dst = nullptr;
+  const float* weight = nullptr;
+  bool rotate = false;
+  if (active) {
+    if (h < nh) {
+      dst = q_out + ((size_t)t * nh + h) * hd;
+      weight = q_weight;
+      rotate = true;
+    } else {
+      const long long slot = slots ? (long long)slots[t] : -1;
+      if (slot >= 0) {
+        const long long page = slot / page_size, off = slot % page_size;
+        const bool is_k = h < nh + nkv;
+        const int kvh = is_k ? h - nh : h - nh - nkv;
+        T* base = is_k ? k_cache : v_cache;
+        dst = base + (((size_t)page * nkv + kvh) * page_size + off) * hd;
+        weight = is_k ? k_weight : nullptr;
+        rotate = is_k;
+      }
+    }
+  }
+  const bool is_v = active && h >= nh + nkv;
+
+  float x[kMaxHeadDim / kWave];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
+    const int i = lane + e * kWave;
+    x[e] = (active && i < hd) ? to_f32(src[i]) : 0.f;
+    ss += x[e] * x[e];
+  }
+  if (is_v) {  // plain copy
+    if (dst) {
+#pragma unroll
+      for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
+        const int i = lane + e * kWave;
+        if (i < hd) dst[i] = src[i];
+      }
+    }
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / (float)hd + eps);
+#pragma unroll
+  for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
+    const int i = lane + e * kWave;
+    if (i < hd) {
+      if (!is_v && weight) x[e] = x[e] * inv * weight[i];
+      normed[wave][i] = x[e];
+    }
+  }
+  __syncthreads();
+  if (!active || is_v || !dst) return;
+  const int half = rot / 2;
+  const int pos = rot > 0 ? positions[t] : 0;
+  const float* c = cos_table + (size_t)pos * half;
+  const float* s = sin_table + (size_t)pos * half;
+#pragma unroll
+  for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
+    const int i = lane + e * kWave;
+    if (i >= hd) continue;
+    float r = x[e];
+    if (rotate && i < rot) {
+      if (i < half) {
+        r = x[e] * c[i] - normed[wave][i + half] * s[i];
+      } else {
+        const int j = i - half;
+        r = normed[wave][j] * s[j] + x[e] * c[j];
+      }
+    }
+    dst[i] = from_f32<T>(r);
+  }
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_weight,
+                                 const float* k_weight, const float* cos_table, const float* sin_table,
+                                 const int* positions, const int* slots, void* q_out, void* k_cache,
+                                 void* v_cache, int tokens, int nh, int nkv, int hd, int rot, int page_size,
+                                 float eps) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && nh > 0 && nkv >= 0 && page_size > 0, "qknorm_rope_kv: bad sizes tokens=%d nh=%d nkv=%d page=%d",
+             tokens, nh, nkv, page_size);
+  PA_REQUIRE(hd > 0 && hd <= kMaxHeadDim, "qknorm_rope_kv: head_dim %d is outside 1..%d", hd, kMaxHeadDim);
+  PA_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "qknorm_rope_kv: rotary width %d must be even and at most head_dim %d",
+             rot, hd);
+  PA_REQUIRE(rot == 0 || (cos_table && sin_table && positions), "qknorm_rope_kv: rotary tables or positions missing");
+  const long long units = (long long)tokens * (nh + 2 * nkv);
+  const unsigned blocks = (unsigned)((units + kQkWaves - 1) / kQkWaves);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == kF32) {
+    hipLaunchKernelGGL(qknorm_rope_kv_kernel<float>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const float*)qkv,
+                       q_weight, k_weight, cos_table, sin_table, positions, slots, (float*)q_out, (float*)k_cache,
+                       (float*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps);
+  } else if (dtype == kBF16) {
+    hipLaunchKernelGGL(qknorm_rope_kv_kernel<bf16>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const bf16*)qkv,
+                       q_weight, k_weight, cos_table, sin_table, positions, slots, (bf16*)q_out, (bf16*)k_cache,
+                       (bf16*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps);
+  } else {
+    return pa::fail("qknorm_rope_kv: unknown element type code %d", dtype);
+  }
+  return check_launch("qknorm_rope_kv");
+}

@@ -1,0 +1,25 @@
+"""Arrangements of parts into one layer.
+
+``prenorm``: norm -> mixer -> (+residual) norm -> feed-forward, with the
+residual carried beside the hidden state and each add deferred into the next
+norm (crates/prelude-core/src/models/qwen3.rs:486-502,
+crates/prelude-core/src/models/commons/linear.rs:471-488).
+"""
+from __future__ import annotations
+
+from .base import Block, register_part
+
+
+@register_part("block", "prenorm")
+class PreNormBlock(Block):
+    SLOTS = {"input_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm", "ffn": "ffn"}
+
+    def __init__(self, input_norm, mixer, post_mixer_norm, ffn):
+        self.input_norm, self.mixer, self.post_mixer_norm, self.ffn = input_norm, mixer, post_mixer_norm, ffn
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        residual, h = self.input_norm.forward_residual(hidden, residual)
+        h = self.mixer.forward(h, step, cache, write_cache)
+        residual, h = self.post_mixer_norm.forward_residual(h, residual)
+        h = self.ffn.forward(h)
+        return h, residual
