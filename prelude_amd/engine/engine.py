@@ -1,0 +1,252 @@
+"""The model with its cache on one GPU, and the one step function everything drives.
+
+``Engine.step`` takes a batch of (request, its next tokens, the places whose
+logits are wanted): portions of prompts beside single decoded tokens, cut
+anywhere.  It runs exactly the tokens it is given, as one packed batch, from
+the cache earlier steps left, and returns the logits at the wanted places.
+The reference's counterpart is ``batch_mixed_paged``
+(crates/prelude-core/src/engine/model_runner/paged_mixed.rs:13-335) over
+``StepRequest`` (crates/prelude-core/src/engine/executor.rs:96-115), which
+always returns one row per request.
+"""
+from __future__ import annotations
+
+import dataclasses
+import os
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import (CacheError, OutOfPages, PageTables, allocate_storage, bytes_per_token, plan_groups)
+from ..config.engine_config import EngineConfig
+from ..config.model_config import read_config_json
+from ..config.registry import resolve_architecture
+from ..models.causal_lm import CausalLM
+from ..weights.loader import load_into
+from .batch import GroupStep, StepBatch
+
+
+class StepError(ValueError):
+    pass
+
+
+@dataclasses.dataclass
+class StepEntry:
+    """One request's share of a step."""
+    id: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()     # indices into ``tokens`` whose logits are wanted
+
+
+class _Staging:
+    """Pinned host buffers for the step's index arrays, used in turn so that a
+    buffer is rewritten only after the copy that read it has finished."""
+
+    def __init__(self, depth: int = 3):
+        self._bufs: List[Optional[torch.Tensor]] = [None] * depth
+        self._events: List[Optional[torch.cuda.Event]] = [None] * depth
+        self._i = 0
+
+    def get(self, n: int) -> tuple:
+        i = self._i
+        self._i = (i + 1) % len(self._bufs)
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        b = self._bufs[i]
+        if b is None or b.numel() < n:
+            b = torch.empty(max(4096, 2 * n), dtype=torch.int32, pin_memory=True)
+            self._bufs[i] = b
+        return i, b
+
+    def sent(self, i: int) -> None:
+        ev = torch.cuda.Event()
+        ev.record()
+        self._events[i] = ev
+
+
+class Engine:
+    def __init__(self, model: CausalLM, config: EngineConfig, raw_config: Optional[dict] = None):
+        """``model`` must be loaded (``weights.load_into``) on ``config.device``."""
+        if model.device is None:
+            raise StepError("the model has no weights loaded")
+        self.model = model
+        self.config = config
+        self.raw_config = raw_config or {}
+        self.device = model.device
+        self.dtype = model.dtype
+        self.vocab_size = model.spec.vocab_size
+        self.max_positions = model.spec.max_positions
+        self.page_size = int(config.page_size)
+        specs = [c.spec for c in model.cache_slots]
+        self.group_specs, self._group_of_slot = plan_groups(specs)
+        tokens = self._decide_cache_tokens(specs)
+        pages = max(1, -(-tokens // self.page_size))
+        self.cache_tokens = pages * self.page_size
+        state_slots = config.max_state_slots if model.needs_state else 0
+        self.tables = PageTables(self.page_size, [(pages, g.window) for g in self.group_specs], state_slots)
+        self.caches = allocate_storage(specs, self._group_of_slot, [pages] * len(self.group_specs), self.page_size,
+                                       state_slots, self.dtype, self.device)
+        self._staging = _Staging()
+        self._live: Dict[int, int] = {}   # request id -> tokens fed so far
+
+    # ---- construction -------------------------------------------------------
+    @classmethod
+    def from_model_dir(cls, model_dir: str, config: Optional[EngineConfig] = None) -> "Engine":
+        """Reads config.json, picks the architecture from the registry, loads the safetensors."""
+        from .. import models  # noqa: F401  registers the built-in architectures
+        config = config or EngineConfig()
+        if not torch.cuda.is_available():
+            raise RuntimeError("prelude_amd needs a GPU: torch sees no HIP device, and there is no CPU path")
+        raw = read_config_json(model_dir)
+        arch = resolve_architecture(raw)
+        model = CausalLM(arch.build_spec(arch.parse_config(raw)))
+        device = torch.device(config.device)
+        torch.cuda.set_device(device)
+        load_into(model, model_dir, config.torch_dtype(), device)
+        return cls(model, config, raw)
+
+    def _decide_cache_tokens(self, specs) -> int:
+        if self.config.max_cache_tokens is not None:
+            return max(int(self.config.max_cache_tokens), self.page_size)
+        per_token = bytes_per_token(specs, self.dtype)
+        if per_token == 0:
+            return self.page_size
+        free, _total = torch.cuda.mem_get_info(self.device)
+        # room for one step's activations: a dozen hidden-sized rows, the widest projection, float32 logits rows
+        spec = self.model.spec
+        el = torch.empty((), dtype=self.dtype).element_size()
+        act = self.config.max_num_batched_tokens * spec.hidden_size * el * 48 + 256 * spec.vocab_size * 4 * 2
+        usable = int(free * self.config.gpu_memory_utilization) - act
+        tokens = max(usable // per_token, 16 * self.page_size)
+        return int(min(tokens, self.max_positions * max(1, self.config.max_running_requests)))
+
+    # ---- requests ---------------------------------------------------------------
+    def has(self, rid: int) -> bool:
+        return self.tables.has(rid)
+
+    def length(self, rid: int) -> int:
+        return self.tables.length(rid)
+
+    def release(self, rid: int) -> None:
+        """The request is over: its pages and its state slot go back."""
+        if self.tables.has(rid):
+            self.tables.close(rid)
+        self._live.pop(rid, None)
+
+    # ---- the step -----------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Opens unknown requests, takes pages, runs, and records the new lengths.
+
+        Returns float32 logits [sum(len(want)), vocab] in the order of the
+        entries and of each entry's ``want``.  Raises ``OutOfPages`` (with
+        nothing taken and nothing run) if the pools cannot hold the step.
+        """
+        self._validate(entries)
+        opened, reserved = [], []
+        try:
+            for e in entries:
+                if not self.tables.has(e.id):
+                    self.tables.open(e.id, self.model.needs_state)
+                    opened.append(e.id)
+                self.tables.reserve(e.id, self.tables.length(e.id) + len(e.tokens))
+                reserved.append(e.id)
+        except CacheError:
+            for rid in reserved:
+                self.tables.rollback(rid)
+            for rid in opened:
+                self.tables.close(rid)
+            raise
+        starts = [self.tables.length(e.id) for e in entries]
+        try:
+            logits = self.run(entries, starts)
+        except Exception:
+            for e in entries:
+                self.tables.rollback(e.id)
+            for rid in opened:
+                self.tables.close(rid)
+            raise
+        for e, s in zip(entries, starts):
+            self.tables.commit(e.id, s + len(e.tokens))
+        return logits
+
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.id in seen:
+                raise StepError(f"request {e.id} appears twice in one step")
+            seen.add(e.id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.id} brings no tokens")
+            a = np.asarray(e.tokens, dtype=np.int64)
+            if a.ndim != 1 or int(a.min()) < 0 or int(a.max()) >= self.vocab_size:
+                bad = [int(t) for t in a.reshape(-1) if not 0 <= int(t) < self.vocab_size][:1]
+                raise StepError(f"request {e.id}: token id {bad[0] if bad else a} is outside the vocabulary "
+                                f"of {self.vocab_size}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"request {e.id}: wanted place {w} is outside its {n} tokens")
+            have = self.tables.length(e.id) if self.tables.has(e.id) else 0
+            if have + n > self.max_positions:
+                raise StepError(f"request {e.id}: {have} + {n} tokens exceed max_position_embeddings "
+                                f"{self.max_positions}")
+
+    def build_batch(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> StepBatch:
+        """Index arrays of the step, built on the host in one pinned buffer and sent in one copy."""
+        n = len(entries)
+        counts = [len(e.tokens) for e in entries]
+        total = sum(counts)
+        ends = [s + c for s, c in zip(starts, counts)]
+        stride = max(1, -(-max(ends) // self.page_size))
+        wanted = sum(len(e.want) for e in entries)
+        layout = self.tables.step_layout(n, total, stride, wanted)
+        size = layout["_total"][1]
+        slot, pinned = self._staging.get(size)
+        host = pinned.numpy()
+        off, _ = layout["token_ids"]
+        woff, _ = layout["want_rows"]
+        t = 0
+        w = 0
+        for e, c in zip(entries, counts):
+            host[off + t: off + t + c] = e.tokens
+            for x in e.want:
+                host[woff + w] = t + int(x)
+                w += 1
+            t += c
+        self.tables.fill_step([e.id for e in entries], starts, counts, stride, host, layout)
+        soff, _ = layout["state_slots"]
+        foff, _ = layout["fresh"]
+        state_host = host[soff: soff + n].tolist()
+        fresh_host = host[foff: foff + n].tolist()
+        dev = torch.empty(size, dtype=torch.int32, device=self.device)
+        dev.copy_(pinned[:size], non_blocking=True)
+        self._staging.sent(slot)
+
+        def view(name):
+            o, s = layout[name]
+            return dev[o: o + s]
+
+        G = len(self.group_specs)
+        bt = view("block_tables").view(G, n, stride) if G else None
+        sl = view("slots").view(G, total) if G else None
+        kv = [GroupStep(bt[g], sl[g]) for g in range(G)]
+        return StepBatch(num_tokens=total, num_seqs=n, token_ids=view("token_ids"), positions=view("positions"),
+                         seq_of_token=view("seq_of_token"), cu_q=view("cu_q"), context_lens=view("context_lens"),
+                         state_slots=view("state_slots"), fresh=view("fresh"), want_rows=view("want_rows"), kv=kv,
+                         q_lens=counts, starts=list(starts), state_slots_host=state_host, fresh_host=fresh_host,
+                         max_q_len=max(counts), max_context_len=max(ends), page_size=self.page_size)
+
+    def run(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> torch.Tensor:
+        """Runs a step whose pages are already reserved (the scheduler's path)."""
+        batch = self.build_batch(entries, starts)
+        if self.model.needs_state:
+            fresh = [s for s, f in zip(batch.state_slots_host, batch.fresh_host) if f and s >= 0]
+            if fresh:
+                idx = torch.tensor(fresh, dtype=torch.int64, device=self.device)
+                for c in self.caches:
+                    if hasattr(c, "zero_slots"):
+                        c.zero_slots(idx)
+        return self.model.forward(batch, self.caches)

@@ -242,3 +242,12 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
     check(kernels().pa_argmax(_stream(), _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1]))
     return out
+
+
+def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int,
+              scale: float) -> torch.Tensor:
+    """Attention of one step over one cache group; picks the kernel for the sizes at hand.
+
+    ``group`` is the step's ``GroupStep`` of the cache group, ``step`` the ``StepBatch``.
+    """
+    return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
