@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
+
+The default run has the layer sizes of the Qwen3-4B shape (36 layers, hidden
+2560, 32 heads, 8 KV heads, head_dim 128, intermediate 9728, vocabulary
+151936, tied head) with random bfloat16 weights, a batch of 8 and a context of
+4,096 tokens: every request is prefilled through the engine's own step
+function, then K decode steps are timed (each step: build the batch, run the
+model from the paged cache, greedy argmax on the device, ids back to the host).
+One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is
+a 2,048-token prompt portion; ``roofline`` prices the decode step against HBM
+bandwidth; ``points`` holds batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "f32": 157.3e12}
+
+QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936, hidden_size=2560,
+                intermediate_size=9728, num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8,
+                head_dim=128, attention_bias=False, max_position_embeddings=40960, sliding_window=None,
+                max_window_layers=36, tie_word_embeddings=True, rope_theta=1000000.0, rms_norm_eps=1e-6,
+                use_sliding_window=False, hidden_act="silu", eos_token_id=151645)
+
+
+def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
+    """The engine's own model with weights drawn on the device (no 8 GB file is written)."""
+    import torch
+    from prelude_amd import models  # noqa: F401
+    from prelude_amd.config import EngineConfig, resolve_architecture
+    from prelude_amd.engine import Engine
+    from prelude_amd.models.causal_lm import CausalLM
+    from prelude_amd.parts.base import MATRIX, NORM
+
+    arch = resolve_architecture(raw)
+    model = CausalLM(arch.build_spec(arch.parse_config(raw)))
+    device = torch.device("cuda:0")
+    tdtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    gen = torch.Generator(device=device).manual_seed(seed)
+    cache = {}
+
+    def fetch(name, req):
+        if name not in cache:
+            t = torch.randn(req.shape, generator=gen, device=device, dtype=torch.float32)
+            t = (1.0 + 0.01 * t) if req.kind == NORM else 0.02 * t
+            cache[name] = t.to(tdtype if req.kind == MATRIX else torch.float32).contiguous()
+        return cache[name]
+
+    model.load(fetch, tdtype, device)
+    cache.clear()
+    cfg = EngineConfig(dtype=dtype, page_size=page_size, max_cache_tokens=cache_tokens, **cfg_overrides)
+    return Engine(model, cfg, raw)
+
+
+def weight_bytes(raw, el):
+    h, i, v = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
+    nh, nkv, hd, L = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"], raw["num_hidden_layers"]
+    per_layer = ((nh + 2 * nkv) * hd * h + nh * hd * h + 3 * i * h) * el + (2 * h + 2 * hd) * 4
+    head = v * h * el           # the head matrix is read whole; the embedding only gathers rows
+    return L * per_layer + head + h * 4, L * ((nh + 2 * nkv) * hd * h + nh * hd * h + 3 * i * h)
+
+
+def kv_bytes_per_token(raw, el):
+    return raw["num_hidden_layers"] * 2 * raw["num_key_value_heads"] * raw["head_dim"] * el
+
+
+def prefill_requests(engine, batch, length, chunk, vocab, seed):
+    import numpy as np
+    from prelude_amd.engine import StepEntry
+    rng = np.random.default_rng(seed)
+    prompts = [rng.integers(0, vocab, size=length).tolist() for _ in range(batch)]
+    for rid, p in enumerate(prompts):
+        for s in range(0, length, chunk):
+            engine.step([StepEntry(rid, p[s:s + chunk], [])])
+    return prompts
+
+
+def time_decode(engine, batch, steps, warmup, vocab):
+    """Greedy decode steps for `batch` live requests; returns seconds per step."""
+    import torch
+    from prelude_amd.engine import StepEntry
+    from prelude_amd.ops import kernels as K
+    last = [1] * batch
+
+    def one():
+        nonlocal last
+        logits = engine.step([StepEntry(r, [last[r]], [0]) for r in range(batch)])
+        last = K.argmax(logits).tolist()
+
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def decode_point(raw, dtype, batch, context, steps, warmup, layers_note):
+    import torch
+    total = steps + warmup
+    eng = build_engine(raw, dtype, cache_tokens=batch * (context + 64))
+    prefill_requests(eng, batch, context - total, 2048, raw["vocab_size"], seed=batch)
+    sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"])
+    del eng
+    torch.cuda.empty_cache()
+    return sec
+
+
+def time_prefill(raw, dtype, tokens, reps):
+    import numpy as np
+    import torch
+    from prelude_amd.engine import StepEntry
+    eng = build_engine(raw, dtype, cache_tokens=(reps + 2) * (tokens + 64))
+    rng = np.random.default_rng(7)
+    best = None
+    for r in range(reps + 1):
+        p = rng.integers(0, raw["vocab_size"], size=tokens).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.step([StepEntry(100 + r, p, [tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        eng.release(100 + r)
+        if r > 0:
+            best = dt if best is None else min(best, dt)
+    del eng
+    torch.cuda.empty_cache()
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus, flush=True)
+        return 2
+
+    import torch
+    raw = dict(QWEN3_4B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+        raw["max_window_layers"] = args.layers
+    el = 2 if args.dtype == "bfloat16" else 4
+    short = "bf16" if args.dtype == "bfloat16" else "f32"
+
+    sec = decode_point(raw, args.dtype, args.batch, args.context, args.steps, args.warmup, None)
+    value = args.batch / sec
+    wbytes, matmul_params = weight_bytes(raw, el)
+    step_bytes = wbytes + args.batch * args.context * kv_bytes_per_token(raw, el)
+    achieved = step_bytes / sec / 1e9
+
+    out = {
+        "metric": "decode tok/s @ batch 8, context 4096 (Qwen3-4B shape, bf16)" if args.batch == 8 else
+                  f"decode tok/s @ batch {args.batch}, context {args.context} (Qwen3-4B shape)",
+        "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic (random tokens, random-init weights)",
+        "config": {"model": "Qwen3-4B shape", "layers": raw["num_hidden_layers"], "layers_full": full_layers,
+                   "hidden": raw["hidden_size"], "heads": raw["num_attention_heads"],
+                   "kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
+                   "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"], "tied": True,
+                   "global_batch": args.batch, "seq_len": args.context, "page_size": 16, "parallelism": "none"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_prefill:
+        T = args.prefill_tokens
+        psec = time_prefill(raw, args.dtype, T, reps=3)
+        nh, hd, L = raw["num_attention_heads"], raw["head_dim"], raw["num_hidden_layers"]
+        flops = 2.0 * T * matmul_params + L * 2.0 * nh * hd * T * T + 2.0 * raw["vocab_size"] * raw["hidden_size"]
+        out["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
+                          "frac": round(flops / psec / MFMA_PEAK[short], 4)}
+    if not args.no_points:
+        pts = {}
+        for b in (1, 64):
+            s = decode_point(raw, args.dtype, b, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), None)
+            pts[f"decode_b{b}"] = round(b / s, 2)
+        out["points"] = pts
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -47,6 +47,7 @@ _KERNEL_API = {
     "pa_gemm_plain": (I, [P, I, I, P, P, P, P, I, I, I, c_long, c_long, c_long]),
     "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
     "pa_argmax": (I, [P, P, P, I, I]),
+    "pa_sample": (I, [P, P, P, P, P, P, P, I, I]),
 }
 
 _HOST_API = {

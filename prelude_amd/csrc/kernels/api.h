@@ -43,6 +43,11 @@ int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache,
 // out[r] = index of the largest of logits[r, :], the lowest index among equals.
 int pa_argmax(void* stream, const float* logits, int* out, int rows, int vocab);
 
+// Per row: temperature < 1e-7 -> argmax; else a draw from softmax(logits / T) kept to the top_k largest
+// (0 = all) and to the shortest descending prefix of mass top_p (>= 1 = all), at the uniform number uniform[r] in [0, 1).
+int pa_sample(void* stream, const float* logits, const float* temperature, const int* top_k, const float* top_p,
+              const float* uniform, int* out, int rows, int vocab);
+
 #ifdef __cplusplus
 }
 #endif

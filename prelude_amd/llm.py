@@ -1,0 +1,189 @@
+"""The Python entry point: ``LLM(model_dir).generate(prompts, ...)``.
+
+Modelled on the reference's ``InferenceEngine::generate`` / ``generate_batch``
+(crates/prelude-core/src/engine/mod.rs:75-132) and its request and result
+types (crates/prelude-core/src/types.rs:388-455): per request a prompt (text
+or token ids), ``max_tokens``, sampling options, stop token ids and a seed;
+per result the generated ids, why it finished (``stop`` | ``length`` | ``eos``),
+token counts and the four timings ``ttft_ms, prefill_ms, decode_ms, total_ms``.
+The loop is the reference's ``ar_loop`` (crates/prelude-core/src/engine/run/ar.rs:180-396)
+made synchronous: schedule, build the step, run it, sample, finish.
+"""
+from __future__ import annotations
+
+import dataclasses
+import os
+import time
+from typing import Dict, Iterable, List, Optional, Sequence, Union
+
+import torch
+
+from .config.engine_config import EngineConfig
+from .engine.engine import Engine, StepEntry
+from .engine.scheduler import Scheduler
+from .sampling.sampler import RequestSampler, SamplingParams, sample_rows
+
+DEFAULT_MAX_TOKENS = 4096   # crates/prelude-server/src/routes/generation_common.rs:9
+
+Prompt = Union[str, Sequence[int]]
+
+
+@dataclasses.dataclass
+class GenerationResult:
+    request_id: int
+    prompt_token_ids: List[int]
+    token_ids: List[int]
+    finish_reason: str                      # "stop" | "length" | "eos"
+    text: Optional[str] = None              # when a tokenizer is at hand
+    metrics: Dict[str, float] = dataclasses.field(default_factory=dict)
+    preemptions: int = 0
+
+    @property
+    def usage(self) -> Dict[str, int]:
+        n, m = len(self.prompt_token_ids), len(self.token_ids)
+        return {"prompt_tokens": n, "completion_tokens": m, "total_tokens": n + m}
+
+
+@dataclasses.dataclass
+class _Live:
+    rid: int
+    index: int
+    prompt: List[int]
+    tokens: List[int]            # prompt + generated
+    max_new: int
+    sampler: RequestSampler
+    stop_ids: frozenset
+    t_arrive: float
+    t_first: Optional[float] = None
+    finish_reason: Optional[str] = None
+
+
+class LLM:
+    def __init__(self, model: str, dtype: str = "bfloat16", config: Optional[EngineConfig] = None, **overrides):
+        """``model``: a folder with config.json and safetensors files.  Other
+        keyword arguments override fields of ``EngineConfig``."""
+        cfg = config or EngineConfig()
+        cfg.dtype = dtype if config is None else cfg.dtype
+        for k, v in overrides.items():
+            if not hasattr(cfg, k):
+                raise TypeError(f"unknown engine option {k!r}")
+            setattr(cfg, k, v)
+        self.config = cfg
+        self.model_dir = model
+        self.engine = Engine.from_model_dir(model, cfg)
+        spec = self.engine.model.spec
+        self.eos_token_ids = frozenset(spec.eos_token_ids)
+        self.max_positions = spec.max_positions
+        cap = cfg.decode_reservation_cap or self.max_positions
+        self.scheduler = Scheduler(self.engine.tables, cfg.max_num_batched_tokens, cfg.long_prefill_token_threshold,
+                                   cfg.max_running_requests, cfg.max_total_tokens, cap,
+                                   cfg.decode_priority_max_remaining_tokens, self.engine.model.needs_state)
+        self._next_id = 0
+        self._tokenizer = None
+        self.steps = 0
+
+    # ---- tokenizer (only when prompts are text) --------------------------------
+    def tokenizer(self):
+        if self._tokenizer is None:
+            path = os.path.join(self.model_dir, "tokenizer.json")
+            if not os.path.isfile(path):
+                raise ValueError(f"text prompts need {path}; pass token ids instead")
+            from tokenizers import Tokenizer
+            self._tokenizer = Tokenizer.from_file(path)
+        return self._tokenizer
+
+    def _to_ids(self, prompt: Prompt) -> List[int]:
+        if isinstance(prompt, str):
+            return list(self.tokenizer().encode(prompt).ids)
+        return [int(t) for t in prompt]
+
+    # ---- generation -----------------------------------------------------------------
+    def generate(self, prompts: Union[Prompt, Sequence[Prompt]], max_tokens: int = DEFAULT_MAX_TOKENS,
+                 temperature: float = 0.7, top_p: float = 1.0, top_k: Optional[int] = None,
+                 seed: Optional[int] = None, stop_token_ids: Iterable[int] = (),
+                 sampling_params: Optional[Sequence[SamplingParams]] = None) -> List[GenerationResult]:
+        """Runs all prompts to their end with continuous batching; results in the order of the prompts.
+
+        ``sampling_params`` gives each prompt options of its own and overrides
+        temperature/top_p/top_k/seed.  A request ends on an EOS id of the
+        model (``eos``), on one of ``stop_token_ids`` (``stop``), or after
+        ``max_tokens`` tokens, clamped to the positions the model has left (``length``).
+        """
+        single = isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int))
+        plist = [prompts] if single else list(prompts)
+        if sampling_params is not None and len(sampling_params) != len(plist):
+            raise ValueError("sampling_params must have one entry per prompt")
+        stop = frozenset(int(t) for t in stop_token_ids)
+        live: Dict[int, _Live] = {}
+        results: List[Optional[GenerationResult]] = [None] * len(plist)
+        now = time.perf_counter()
+        for i, p in enumerate(plist):
+            ids = self._to_ids(p)
+            if not ids:
+                raise ValueError(f"prompt {i} is empty")
+            bad = [t for t in ids if not 0 <= t < self.engine.vocab_size]
+            if bad:
+                raise ValueError(f"prompt {i}: token id {bad[0]} is outside the vocabulary")
+            # crates/prelude-core/src/engine/model_runner/generate.rs:23-26
+            max_new = min(int(max_tokens), self.max_positions - len(ids))
+            if max_new < 1:
+                raise ValueError(f"prompt {i} has {len(ids)} tokens; the model has positions for "
+                                 f"{self.max_positions} and none is left to generate")
+            sp = sampling_params[i] if sampling_params is not None else SamplingParams(temperature, top_p, top_k, seed)
+            rid = self._next_id
+            self._next_id += 1
+            self.scheduler.add_request(rid, len(ids), max_new)
+            live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop, now)
+
+        while live:
+            portions = self.scheduler.schedule()
+            if not portions:
+                raise RuntimeError("the scheduler has requests but nothing to run")
+            entries = [StepEntry(p.id, live[p.id].tokens[p.start:p.start + p.count], [p.count - 1] if p.samples else [])
+                       for p in portions]
+            try:
+                logits = self.engine.run(entries, [p.start for p in portions])
+            except Exception:
+                self.scheduler.step_cancelled()
+                raise
+            self.scheduler.step_done()
+            self.steps += 1
+            drawn = [live[p.id] for p in portions if p.samples]
+            toks = sample_rows(logits, [r.sampler for r in drawn])   # waits for the device
+            t = time.perf_counter()
+            for r, tok in zip(drawn, toks):
+                self.scheduler.on_token(r.rid)
+                r.tokens.append(int(tok))
+                if r.t_first is None:
+                    r.t_first = t
+                n_out = len(r.tokens) - len(r.prompt)
+                # order of checks: crates/prelude-core/src/engine/run/ar.rs:1525-1578
+                if tok in self.eos_token_ids:
+                    r.finish_reason = "eos"
+                elif tok in r.stop_ids:
+                    r.finish_reason = "stop"
+                elif n_out >= r.max_new:
+                    r.finish_reason = "length"
+                if r.finish_reason:
+                    info = self.scheduler.info(r.rid)
+                    self.scheduler.finish(r.rid)
+                    results[r.index] = self._result(r, t, info.preempt_count)
+                    del live[r.rid]
+        return results  # type: ignore[return-value]
+
+    def _result(self, r: _Live, t_end: float, preemptions: int) -> GenerationResult:
+        out = r.tokens[len(r.prompt):]
+        first = r.t_first if r.t_first is not None else t_end
+        metrics = {"ttft_ms": (first - r.t_arrive) * 1e3, "prefill_ms": (first - r.t_arrive) * 1e3,
+                   "decode_ms": (t_end - first) * 1e3, "total_ms": (t_end - r.t_arrive) * 1e3}
+        text = None
+        if self._tokenizer is not None:
+            text = self._tokenizer.decode(out)
+        return GenerationResult(r.rid, list(r.prompt), out, r.finish_reason or "length", text, metrics, preemptions)
+
+
+def generate(model: str, prompts, dtype: str = "bfloat16", **kwargs) -> List[GenerationResult]:
+    """One-shot convenience: load ``model`` and generate."""
+    engine_keys = {f.name for f in dataclasses.fields(EngineConfig)}
+    eng = {k: kwargs.pop(k) for k in list(kwargs) if k in engine_keys and k != "dtype"}
+    return LLM(model, dtype=dtype, **eng).generate(prompts, **kwargs)

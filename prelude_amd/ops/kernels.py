@@ -251,3 +251,26 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
     ``group`` is the step's ``GroupStep`` of the cache group, ``step`` the ``StepBatch``.
     """
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor) -> torch.Tensor:
+    """One token per row of float32 logits [R, V]; per-row float32 temperature / top_p / uniform and int32 top_k.
+
+    temperature < 1e-7: argmax.  Else a draw from softmax(logits / T) kept to the
+    top_k largest (0 = all) and the shortest descending prefix of mass top_p
+    (>= 1 = all), by inverse CDF in index order at uniform[r] in [0, 1).
+    """
+    _dev(logits, temperature, top_k, top_p, uniform)
+    _f32(logits, "logits")
+    _f32(temperature, "temperature")
+    _f32(top_p, "top_p")
+    _f32(uniform, "uniform")
+    _i32(top_k, "top_k")
+    r = logits.shape[0]
+    if logits.dim() != 2 or any(t.shape != (r,) for t in (temperature, top_k, top_p, uniform)):
+        raise NativeError("sample: per-row parameters do not match the rows of logits")
+    out = torch.empty((r,), dtype=torch.int32, device=logits.device)
+    check(kernels().pa_sample(_stream(), _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
+                              _ptr(out), r, logits.shape[1]))
+    return out

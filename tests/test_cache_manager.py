@@ -1,0 +1,197 @@
+"""The cache manager's bookkeeping (no GPU): no page lost, held twice or freed twice, under random orders of requests."""
+import random
+
+import numpy as np
+import pytest
+
+from prelude_amd.cache import CacheError, OutOfPages, PageTables
+
+
+def test_allocate_free_and_exhaustion():
+    # scenarios of crates/prelude-core/src/scheduler/components/cache/block_manager.rs:112-199
+    t = PageTables(16, [(4, 0)])
+    t.open(1)
+    t.reserve(1, 33)                       # 33 tokens -> 3 pages
+    assert t.free_pages(0) == 1 and len(t.table(1, 0)) == 3
+    t.commit(1, 33)
+    t.open(2)
+    with pytest.raises(OutOfPages):
+        t.reserve(2, 17)                   # needs 2, 1 free: nothing is taken
+    assert t.free_pages(0) == 1 and t.table(2, 0) == [] and t.audit() == ""
+    t.reserve(2, 16)
+    assert t.free_pages(0) == 0
+    t.close(1)
+    assert t.free_pages(0) == 3 and t.audit() == ""
+    with pytest.raises(CacheError):
+        t.close(1)                         # never freed twice silently
+    t.close(2)
+    assert t.free_pages(0) == 4 and t.num_requests() == 0
+
+
+def test_slot_formula():
+    # crates/prelude-core/src/scheduler/components/cache/block_manager.rs:151-158
+    table = [5, 10, 3]
+    assert [PageTables.slot(table, p, 16) for p in (0, 15, 16, 33)] == [80, 95, 160, 49]
+
+
+def test_pages_are_reused_first_in_first_out():
+    t = PageTables(8, [(3, 0)])
+    t.open(1); t.reserve(1, 24); t.commit(1, 24)
+    assert t.table(1, 0) == [0, 1, 2]
+    t.close(1)
+    t.open(2); t.reserve(2, 9); t.commit(2, 9)
+    assert t.table(2, 0) == [0, 1]
+    t.open(3); t.reserve(3, 1)
+    assert t.table(3, 0) == [2]
+
+
+def test_misuse_is_refused():
+    t = PageTables(8, [(8, 0)])
+    t.open(1)
+    with pytest.raises(CacheError, match="already live"):
+        t.open(1)
+    t.reserve(1, 5)
+    with pytest.raises(CacheError, match="in flight"):
+        t.reserve(1, 9)
+    with pytest.raises(CacheError):
+        t.commit(1, 4)
+    t.commit(1, 5)
+    with pytest.raises(CacheError, match="cannot extend"):
+        t.reserve(1, 5)
+    with pytest.raises(CacheError, match="not live"):
+        t.reserve(7, 5)
+    t.reserve(1, 20)
+    t.rollback(1)                          # the step did not run
+    assert t.length(1) == 5 and len(t.table(1, 0)) == 1 and t.free_pages(0) == 7 and t.audit() == ""
+
+
+def test_window_gives_pages_back_early():
+    t = PageTables(4, [(100, 0), (100, 6)])     # group 1 looks back over 6 keys
+    t.open(1)
+    pos = 0
+    for n in (5, 2, 9, 1, 1, 1, 7, 1):
+        t.reserve(1, pos + n)
+        # every key a query of this portion can see still has its page
+        table = t.table(1, 1)
+        first_key = max(0, pos - 6 + 1)
+        for key in range(first_key, pos + n):
+            assert table[key // 4] >= 0
+        # pages wholly before the first visible key are gone
+        for i, p in enumerate(table):
+            if (i + 1) * 4 <= first_key:
+                assert p == -1
+        assert all(p >= 0 for p in t.table(1, 0))
+        pos += n
+        t.commit(1, pos)
+        assert t.audit() == ""
+    assert t.live_pages(1, 0) == 7 and t.live_pages(1, 1) <= 3
+    assert t.free_pages(1) == 100 - t.live_pages(1, 1)
+    t.close(1)
+    assert t.free_pages(0) == 100 and t.free_pages(1) == 100
+
+
+def test_all_groups_or_none():
+    t = PageTables(4, [(10, 0), (2, 0)])
+    t.open(1)
+    with pytest.raises(OutOfPages):
+        t.reserve(1, 12)                   # group 1 has 2 pages, 3 needed
+    assert t.free_pages(0) == 10 and t.free_pages(1) == 2
+
+
+def test_state_slots():
+    t = PageTables(4, [(10, 0)], state_slots=2)
+    t.open(1, need_state=True)
+    t.open(2, need_state=True)
+    assert {t.state_slot(1), t.state_slot(2)} == {0, 1} and t.free_state_slots() == 0
+    with pytest.raises(CacheError, match="state slot"):
+        t.open(3, need_state=True)
+    t.open(4)                              # a request without state needs none
+    assert t.state_slot(4) == -1
+    t.close(1)
+    t.open(3, need_state=True)
+    assert t.free_state_slots() == 0 and t.audit() == ""
+
+
+def _fill(t, ids, starts, counts):
+    n, total = len(ids), sum(counts)
+    stride = max(-(-(s + c) // t.page_size) for s, c in zip(starts, counts))
+    layout = t.step_layout(n, total, stride, 0)
+    buf = np.full(layout["_total"][1], -7, dtype=np.int32)
+    t.fill_step(ids, starts, counts, stride, buf, layout)
+    get = lambda k: buf[layout[k][0]: layout[k][0] + layout[k][1]]
+    return get, stride
+
+
+def test_step_arrays():
+    t = PageTables(4, [(16, 0), (16, 5)], state_slots=4)
+    t.open(10, True); t.reserve(10, 6); t.commit(10, 6)
+    t.open(11, True); t.reserve(11, 3)
+    t.reserve(10, 7)
+    get, stride = _fill(t, [11, 10], [0, 6], [3, 1])
+    assert stride == 2
+    assert get("positions").tolist() == [0, 1, 2, 6] and get("seq_of_token").tolist() == [0, 0, 0, 1]
+    assert get("cu_q").tolist() == [0, 3, 4] and get("context_lens").tolist() == [3, 7]
+    assert get("fresh").tolist() == [1, 0]
+    assert get("state_slots").tolist() == [t.state_slot(11), t.state_slot(10)]
+    bt = get("block_tables").reshape(2, 2, 2)
+    assert bt[0, 0].tolist() == t.table(11, 0) + [-1] and bt[0, 1].tolist() == t.table(10, 0)
+    slots = get("slots").reshape(2, 4)
+    for g in range(2):
+        assert slots[g].tolist() == [PageTables.slot(t.table(11, g), p, 4) for p in range(3)] + \
+            [PageTables.slot(t.table(10, g), 6, 4)]
+    # position <-> (page, offset) is a bijection within a table
+    t.commit(11, 3); t.commit(10, 7)
+    t.reserve(10, 40)
+    get, _ = _fill(t, [10], [7], [33])
+    s0 = get("slots").reshape(2, 33)[0].tolist()
+    assert len(set(s0)) == 33
+    with pytest.raises(CacheError, match="does not continue"):
+        _fill(t, [10], [8], [32])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_lose_nothing(seed):
+    rng = random.Random(seed)
+    page = rng.choice([1, 4, 8, 16])
+    groups = [(rng.randint(6, 40), 0), (rng.randint(6, 40), rng.choice([3, 9, 20]))]
+    t = PageTables(page, groups, state_slots=3)
+    live = {}
+    nxt = 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 5:
+            need = rng.random() < 0.5 and t.free_state_slots() > 0
+            t.open(nxt, need)
+            live[nxt] = 0
+            nxt += 1
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 5, 13, 30])
+            before = [t.free_pages(g) for g in range(2)]
+            try:
+                t.reserve(rid, live[rid] + n)
+            except OutOfPages:
+                # nothing taken beyond what the window released
+                assert all(t.free_pages(g) >= before[g] for g in range(2))
+                assert t.reservable_len(rid) < live[rid] + n
+            else:
+                if rng.random() < 0.15:
+                    t.rollback(rid)
+                else:
+                    live[rid] += n
+                    t.commit(rid, live[rid])
+                    assert t.length(rid) == live[rid]
+        elif live:
+            rid = rng.choice(list(live))
+            t.close(rid)
+            del live[rid]
+        assert t.audit() == "", t.audit()
+        for g in range(2):
+            held = sum(t.live_pages(r, g) for r in live)
+            assert held + t.free_pages(g) == groups[g][0]
+            for r in live:   # full-attention group: exactly ceil(len / page) pages
+                if g == 0 and t.length(r) == live[r]:
+                    assert t.live_pages(r, 0) == -(-live[r] // page)
+    for rid in list(live):
+        t.close(rid)
+    assert [t.free_pages(g) for g in range(2)] == [g[0] for g in groups] and t.free_state_slots() == 3
