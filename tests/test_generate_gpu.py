@@ -1,0 +1,157 @@
+"""Generation through the Python entry point and the command line, against the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+from helpers import PAGE, model_folder
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def prompts_for(cfg, lengths, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, cfg["vocab_size"] - 3, (n,), generator=g).tolist() for n in lengths]
+
+
+def test_greedy_tiny_a(gpu):
+    """Tiny A: prompts of 5, 17 and 31 tokens, 16 greedy steps, float32."""
+    from prelude_amd import LLM
+    folder, cfg, w = model_folder("a")
+    prompts = prompts_for(cfg, [5, 17, 31], 0)
+    llm = LLM(folder, dtype="float32", page_size=PAGE["a"], max_cache_tokens=512)
+    outs = llm.generate(prompts, max_tokens=16, temperature=0.0)
+    for p, o in zip(prompts, outs):
+        want = pm.greedy(cfg, w, p, len(o.token_ids))
+        assert o.token_ids == want
+        assert o.finish_reason == ("eos" if o.token_ids[-1] == 255 else "length")
+        assert o.finish_reason == "eos" or len(o.token_ids) == 16
+        assert o.usage == {"prompt_tokens": len(p), "completion_tokens": len(o.token_ids), "total_tokens": len(p) + len(o.token_ids)}
+        assert set(o.metrics) == {"ttft_ms", "prefill_ms", "decode_ms", "total_ms"} and o.metrics["total_ms"] > 0
+    assert llm.engine.tables.audit() == "" and llm.engine.tables.num_requests() == 0
+
+
+def test_temperature_tiny_b(gpu):
+    """Tiny B: prompts of 1, 9, 40, 63 and 100 tokens, 24 steps at temperature 0.8, seeded: every token is the
+    plain draw from the plain logits at the request's own random number."""
+    from prelude_amd import LLM
+    from prelude_amd.sampling import RequestSampler, SamplingParams
+    folder, cfg, w = model_folder("b")
+    prompts = prompts_for(cfg, [1, 9, 40, 63, 100], 1)
+    llm = LLM(folder, dtype="float32", page_size=PAGE["b"], max_cache_tokens=1024, max_num_batched_tokens=64)
+    outs = llm.generate(prompts, max_tokens=24, temperature=0.8, seed=7)
+    again = llm.generate(prompts, max_tokens=24, temperature=0.8, seed=7)
+    assert [o.token_ids for o in outs] == [o.token_ids for o in again]                # same seed, same tokens
+    other = llm.generate(prompts, max_tokens=24, temperature=0.8, seed=8)
+    assert [o.token_ids for o in outs] != [o.token_ids for o in other]
+    checked = 0
+    for p, o in zip(prompts, outs):
+        rs = RequestSampler(SamplingParams(0.8, 1.0, None, 7))
+        seq = list(p)
+        for tok in o.token_ids:
+            u = rs.next_uniform()
+            prs = pm.sampling_probs(pm.forward(cfg, w, seq)[-1], 0.8)
+            cdf = torch.cumsum(prs, 0)
+            assert prs[tok] > 0
+            if float((cdf - u * float(cdf[-1])).abs().min()) > 1e-4:
+                assert tok == pm.draw(prs, u)
+                checked += 1
+            seq.append(tok)
+        assert len(o.token_ids) == 24 or o.token_ids[-1] in (507, 508)
+    assert checked > 60
+
+
+def test_top_k_top_p_and_stops(gpu):
+    from prelude_amd import LLM
+    folder, cfg, w = model_folder("b")
+    llm = LLM(folder, dtype="float32", page_size=16, max_cache_tokens=512)
+    p = prompts_for(cfg, [12], 2)[0]
+    greedy = llm.generate([p], max_tokens=10, temperature=0.0)[0].token_ids
+    assert llm.generate([p], max_tokens=10, temperature=1.0, top_k=1, seed=3)[0].token_ids == greedy   # top-1 is greedy
+    assert llm.generate([p], max_tokens=10, temperature=1.0, top_p=1e-6, seed=3)[0].token_ids == greedy
+    assert llm.generate([p], max_tokens=10, temperature=1e-9, seed=3)[0].token_ids == greedy        # T -> 0
+    stop = llm.generate([p], max_tokens=10, temperature=0.0, stop_token_ids=[greedy[3]])[0]
+    first = greedy.index(greedy[3])
+    assert stop.finish_reason == "stop" and stop.token_ids == greedy[:first + 1]                     # the stop token is kept
+    assert llm.generate(p, max_tokens=3, temperature=0.0)[0].finish_reason == "length"               # a single prompt
+    with pytest.raises(ValueError, match="empty"):
+        llm.generate([[]])
+    with pytest.raises(ValueError, match="vocabulary"):
+        llm.generate([[509]])
+    with pytest.raises(ValueError, match="positions"):
+        llm.generate([[1] * 256])
+    # max_tokens is clamped to the positions left (crates/prelude-core/src/engine/model_runner/generate.rs:23-26)
+    o = llm.generate([[1] * 250], max_tokens=100, temperature=0.0, stop_token_ids=[])[0]
+    assert len(o.token_ids) <= 6
+
+
+def test_eos_ends_a_request(gpu, tmp_path):
+    from prelude_amd import LLM
+    from prelude_amd.weights import write_safetensors
+    folder, cfg, w = model_folder("a")
+    p = prompts_for(cfg, [9], 3)[0]
+    greedy = pm.greedy(cfg, w, p, 6)
+    cfg2 = dict(cfg, eos_token_id=[greedy[2], 3])
+    (tmp_path / "config.json").write_text(json.dumps(cfg2))
+    write_safetensors(str(tmp_path / "model.safetensors"), w)
+    o = LLM(str(tmp_path), dtype="float32", page_size=8, max_cache_tokens=256).generate([p], max_tokens=6, temperature=0.0)[0]
+    first = greedy.index(greedy[2])
+    assert o.finish_reason == "eos" and o.token_ids == greedy[:first + 1]
+
+
+def test_running_out_of_pages_changes_no_token(gpu):
+    """A cache too small for all requests at once: some are evicted and recomputed, prompt and generated tokens
+    alike; the tokens are those of an ample cache."""
+    from prelude_amd import LLM
+    folder, cfg, w = model_folder("c")
+    prompts = prompts_for(cfg, [40, 70, 25, 90, 55, 33], 4)
+    ample = LLM(folder, dtype="float32", page_size=8, max_cache_tokens=4096).generate(prompts, max_tokens=40, temperature=0.0)
+    tight = LLM(folder, dtype="float32", page_size=8, max_cache_tokens=200, decode_reservation_cap=1,
+                max_num_batched_tokens=48)
+    outs = tight.generate(prompts, max_tokens=40, temperature=0.0)
+    assert [o.token_ids for o in outs] == [o.token_ids for o in ample]
+    assert tight.scheduler.preemptions > 0 and sum(o.preemptions for o in outs) == tight.scheduler.preemptions
+    assert tight.engine.tables.audit() == "" and tight.engine.tables.num_requests() == 0
+    for p, o in zip(prompts[:2], outs[:2]):
+        assert o.token_ids == pm.greedy(cfg, w, p, len(o.token_ids))
+
+
+def test_bfloat16_generation_runs(gpu):
+    from prelude_amd import LLM
+    folder, cfg, w = model_folder("b", "bfloat16")
+    prompts = prompts_for(cfg, [30, 5], 5)
+    outs = LLM(folder, dtype="bfloat16", page_size=16, max_cache_tokens=512).generate(prompts, max_tokens=12, temperature=0.0)
+    for p, o in zip(prompts, outs):
+        # every chosen token is the plain argmax or within bfloat16 rounding of it
+        seq = list(p)
+        for tok in o.token_ids:
+            lg = pm.forward(cfg, w, seq)[-1]
+            assert float(lg.max() - lg[tok]) < 0.06 * max(1.0, float(lg.abs().max()))
+            seq.append(tok)
+
+
+def test_command_line(gpu, tmp_path):
+    folder, cfg, w = model_folder("a")
+    p = prompts_for(cfg, [7], 6)[0]
+    cmd = [sys.executable, "-m", "prelude_amd", "--model", folder, "--dtype", "f32", "--prompt-ids",
+           ",".join(map(str, p)), "--max-tokens", "5", "--temperature", "0", "--page-size", "8", "--max-cache-tokens", "256"]
+    r = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rec = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rec["token_ids"] == pm.greedy(cfg, w, p, len(rec["token_ids"])) and rec["finish_reason"] in ("length", "eos")
+    assert rec["usage"]["prompt_tokens"] == 7
+    # --random-weights needs only a config.json
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    cmd = [os.path.join(ROOT, "bin", "prelude-amd"), "--model", str(tmp_path), "--random-weights", "--weights-seed", "3",
+           "--prompt-len", "9", "--prompt-len", "4", "--max-tokens", "4", "--temperature", "0.8", "--seed", "1",
+           "--page-size", "8", "--max-cache-tokens", "256"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    recs = [json.loads(l) for l in r.stdout.strip().splitlines()]
+    assert len(recs) == 2 and all(1 <= len(x["token_ids"]) <= 4 for x in recs)

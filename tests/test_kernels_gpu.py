@@ -1,0 +1,330 @@
+"""Each kernel alone against its plain reference, at other sizes than the tiny models use."""
+import math
+
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+DT = [torch.float32, torch.bfloat16]
+
+
+def K():
+    from prelude_amd.ops import kernels
+    return kernels
+
+
+def tol(dtype, ref, f32=2e-6, bf16=1e-2):
+    return (f32 if dtype == torch.float32 else bf16) * max(1.0, float(ref.abs().max()))
+
+
+def close(got, ref, dtype, **kw):
+    err = float((got.double().cpu() - ref.double().cpu()).abs().max())
+    assert err <= tol(dtype, ref, **kw), f"max error {err:.3e} > {tol(dtype, ref, **kw):.3e}"
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(*shape, generator=g)).to(dtype)
+
+
+# ---- embedding, gather ----------------------------------------------------------
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("vocab,hidden", [(509, 96), (1000, 2560), (37, 7)])
+def test_embed_gather(gpu, dtype, vocab, hidden):
+    table = rnd(vocab, hidden, dtype=dtype)
+    ids = torch.tensor([0, vocab - 1, 3, 3, vocab // 2], dtype=torch.int32)
+    out = K().embed_gather(ids.to(gpu), table.to(gpu))
+    assert torch.equal(out.cpu(), table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_gather_rows(gpu, dtype):
+    x = rnd(40, 130, dtype=dtype)
+    rows = torch.tensor([39, 0, 7, 7], dtype=torch.int32)
+    assert torch.equal(K().gather_rows(x.to(gpu), rows.to(gpu)).cpu(), x[rows.long()])
+
+
+# ---- norms --------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows,hidden,eps", [(5, 2560, 1e-6), (3, 100, 1e-5), (2, 7, 3e-6), (9, 4096, 1e-6), (1, 513, 1e-6)])
+def test_rmsnorm(gpu, dtype, rows, hidden, eps):
+    x = rnd(rows, hidden, dtype=dtype, scale=3.0)
+    w = 1.0 + 0.1 * rnd(hidden, seed=1)
+    ref = pm.rms_norm(x.double(), w.double(), eps)
+    close(K().rmsnorm(x.to(gpu), w.to(gpu), eps), ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows,hidden", [(6, 2560), (4, 96), (3, 1000)])
+def test_add_rmsnorm(gpu, dtype, rows, hidden):
+    # crates/prelude-core/tests/modules.rs:275-314: the sum is returned, the norm is of the unrounded sum
+    x, res = rnd(rows, hidden, dtype=dtype), rnd(rows, hidden, dtype=dtype, seed=2, scale=4.0)
+    w = 1.0 + 0.1 * rnd(hidden, seed=1)
+    s = x.double() + res.double()
+    r_dev = res.to(gpu).clone()
+    out = K().rmsnorm(x.to(gpu), w.to(gpu), 1e-6, residual=r_dev)
+    close(out, pm.rms_norm(s, w.double(), 1e-6), dtype)
+    assert torch.equal(r_dev.cpu(), s.to(dtype))             # the residual holds the sum, rounded once
+    # rows variant: compact output, residual untouched
+    rows_idx = torch.tensor([rows - 1, 0], dtype=torch.int32)
+    r2 = res.to(gpu).clone()
+    out2 = K().rmsnorm(x.to(gpu), w.to(gpu), 1e-6, residual=r2, rows=rows_idx.to(gpu))
+    close(out2, pm.rms_norm(s[rows_idx.long()], w.double(), 1e-6), dtype)
+    assert torch.equal(r2.cpu(), res)
+
+
+def test_rmsnorm_reference_vector(gpu):
+    x = torch.tensor([[3.0, 4.0]])
+    out = K().rmsnorm(x.to(gpu), torch.ones(2).to(gpu), 1e-6).cpu()
+    assert torch.allclose(out, x / math.sqrt(12.5 + 1e-6), atol=1e-6)
+
+
+# ---- SiLU * up ----------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("tokens,inter", [(3, 9728), (5, 160), (2, 7)])
+def test_silu_mul(gpu, dtype, tokens, inter):
+    gu = rnd(tokens, 2 * inter, dtype=dtype, scale=3.0)
+    ref = pm.silu(gu[:, :inter].double()) * gu[:, inter:].double()
+    close(K().silu_mul(gu.to(gpu)), ref, dtype)
+
+
+def test_silu_mul_reference_vector(gpu):
+    g = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5])
+    u = torch.tensor([1.0, 2.0, 3.0, 0.5, 1.0, 4.0])
+    out = K().silu_mul(torch.cat([g, u]).reshape(1, 12).to(gpu)).cpu()[0]
+    assert torch.allclose(out, torch.nn.functional.silu(g) * u, atol=1e-6) and float(out[0]) == 0.0
+
+
+# ---- matrix product ---------------------------------------------------------------------------
+@pytest.mark.parametrize("m,n,k", [(1, 509, 96), (33, 70, 45), (64, 64, 16), (130, 257, 160), (7, 2560, 2560)])
+def test_gemm_plain_f32(gpu, m, n, k):
+    x, w, b = rnd(m, k), rnd(n, k, seed=1), rnd(n, seed=2)
+    ref = x.double() @ w.double().T + b.double()
+    out = K().gemm_plain(x.to(gpu), w.to(gpu), b.to(gpu))
+    close(out, ref, torch.float32, f32=2e-6 * math.sqrt(k))
+    # a row's result does not depend on the other rows of the batch
+    one = K().gemm_plain(x[m // 2: m // 2 + 1].to(gpu), w.to(gpu), b.to(gpu))
+    assert torch.equal(one[0], out[m // 2])
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 509, 96), (8, 2560, 4096), (40, 331, 80), (300, 192, 96), (64, 6144, 2560)])
+def test_linear_bf16(gpu, m, n, k):
+    x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
+    ref = x.double() @ w.double().T
+    close(K().linear(x.to(gpu), w.to(gpu)), ref, torch.bfloat16)
+    close(K().linear(x.to(gpu), w.to(gpu), b.to(gpu)), ref + b.double(), torch.bfloat16)
+    out32 = K().linear(x.to(gpu), w.to(gpu), out_dtype=torch.float32)
+    assert out32.dtype == torch.float32
+    close(out32, ref, torch.bfloat16)
+    close(K().gemm_plain(x.to(gpu), w.to(gpu), out_dtype=torch.float32), ref, torch.float32, f32=1e-5)
+
+
+# ---- QK norm + RoPE + cache write ---------------------------------------------------------------
+def qk_reference(qkv, qw, kw, cos, sin, pos, nh, nkv, hd, rot, eps):
+    t = qkv.shape[0]
+    x = qkv.double().reshape(t, nh + 2 * nkv, hd)
+    q, k, v = x[:, :nh], x[:, nh:nh + nkv], x[:, nh + nkv:]
+    if qw is not None:
+        q = pm.rms_norm(q, qw.double(), eps)
+    if kw is not None:
+        k = pm.rms_norm(k, kw.double(), eps)
+    if rot:
+        c, s = cos.double()[pos.long()], sin.double()[pos.long()]
+        q = torch.cat([pm.apply_rope(q[..., :rot], c, s), q[..., rot:]], -1)
+        k = torch.cat([pm.apply_rope(k[..., :rot], c, s), k[..., rot:]], -1)
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkv,hd,rot,norm", [(32, 8, 128, 128, True), (6, 1, 32, 32, True), (5, 5, 48, 48, True),
+                                                 (4, 2, 256, 256, True), (3, 1, 80, 32, True), (2, 2, 16, 16, False),
+                                                 (7, 1, 112, 0, True), (4, 4, 64, 64, True)])
+def test_qknorm_rope_kv(gpu, dtype, nh, nkv, hd, rot, norm):
+    t, page, pages, eps = 11, 4, 9, 1e-5
+    qkv = rnd(t, (nh + 2 * nkv) * hd, dtype=dtype, scale=2.0)
+    qw = (1.0 + 0.2 * rnd(hd, seed=1)) if norm else None
+    kw = (1.0 + 0.2 * rnd(hd, seed=2)) if norm else None
+    pos = torch.tensor([0, 1, 2, 3, 17, 18, 99, 5, 6, 7, 255], dtype=torch.int32)
+    cos = sin = None
+    if rot:
+        cos, sin = pm.rope_tables(rot, 256, 10000.0, torch.float32)
+    slot_list = [35, 3, 0, 7, 8, 12, -1, 20, 21, 22, 30]                  # one token is not cached
+    slots = torch.tensor(slot_list, dtype=torch.int32)
+    kc = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype)
+    vc = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype)
+    dev = lambda x: None if x is None else x.to(gpu)
+    kcd, vcd = kc.to(gpu), vc.to(gpu)
+    q = K().qknorm_rope_kv(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), dev(pos), dev(slots), kcd, vcd, nh, nkv, hd,
+                           rot, eps)
+    rq, rk, rv = qk_reference(qkv, qw, kw, cos, sin, pos, nh, nkv, hd, rot, eps)
+    close(q, rq, dtype)
+    touched = torch.zeros(pages, page, dtype=torch.bool)
+    for i, s in enumerate(slot_list):
+        if s < 0:
+            continue
+        touched[s // page, s % page] = True
+        close(kcd[s // page, :, s % page], rk[i], dtype)
+        assert torch.equal(vcd[s // page, :, s % page].cpu().double(), rv[i].to(dtype).double())   # V is a copy
+    assert bool((kcd.cpu()[~touched[:, None, :].expand(pages, nkv, page)] == 7.0).all())             # nothing else written
+    # queries only (a layer that reads another layer's cache)
+    qonly = qkv[:, : nh * hd].contiguous()
+    q2 = K().qknorm_rope_kv(dev(qonly), dev(qw), None, dev(cos), dev(sin), dev(pos), None, None, None, nh, 0, hd, rot, eps)
+    assert torch.equal(q2, q)
+
+
+def test_qknorm_rope_refuses_bad_sizes(gpu):
+    from prelude_amd._native import NativeError
+    qkv = torch.zeros(2, 3 * 272, device=gpu)
+    with pytest.raises(NativeError, match="head_dim"):
+        K().qknorm_rope_kv(qkv, None, None, None, None, torch.zeros(2, dtype=torch.int32, device=gpu), None, None, None,
+                           3, 0, 272, 0, 1e-6)
+
+
+# ---- attention over the paged cache --------------------------------------------------------------
+def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None):
+    """seqs: list of (context_len, q_len): the last q_len tokens of each context are this step's queries.
+    Pages are handed out in a scrambled order.  Returns (engine output, plain output)."""
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-c // page) for c, _ in seqs) + 3
+    perm = torch.randperm(total_pages, generator=torch.Generator().manual_seed(seed + 77)).tolist()
+    kc = torch.zeros(total_pages, nkv, page, hd)
+    vc = torch.zeros(total_pages, nkv, page, hd)
+    stride = max(-(-c // page) for c, _ in seqs)
+    table = torch.full((len(seqs), stride), -1, dtype=torch.int32)
+    qs, seq_of, pos, refs = [], [], [], []
+    for i, (ctx, ql) in enumerate(seqs):
+        k = torch.randn(ctx, nkv, hd, generator=g)
+        v = torch.randn(ctx, nkv, hd, generator=g)
+        q = torch.randn(ql, nh, hd, generator=g)
+        if scale_trick is not None:
+            scale_trick(i, q, k, v)
+        k, v, q = k.to(dtype).float(), v.to(dtype).float(), q.to(dtype).float()
+        for p in range(-(-ctx // page)):
+            phys = perm.pop()
+            table[i, p] = phys
+            n = min(page, ctx - p * page)
+            kc[phys, :, :n] = k[p * page: p * page + n].transpose(0, 1)
+            vc[phys, :, :n] = v[p * page: p * page + n].transpose(0, 1)
+        if window:   # pages wholly before the first visible key may be gone
+            first = max(0, (ctx - ql) - window + 1)
+            for p in range(first // page):
+                kc[table[i, p]] = float("nan")
+                vc[table[i, p]] = float("nan")
+                table[i, p] = -1
+        qs.append(q)
+        seq_of += [i] * ql
+        pos += list(range(ctx - ql, ctx))
+        refs.append(pm.attention(q.double(), k.double(), v.double(), 1.0 / math.sqrt(hd), window=window or None,
+                                 q_offset=ctx - ql))
+    q = torch.cat(qs).to(dtype)
+    out = K().attention_generic(q.to(gpu), kc.to(dtype).to(gpu), vc.to(dtype).to(gpu), table.to(gpu),
+                                torch.tensor(seq_of, dtype=torch.int32, device=gpu),
+                                torch.tensor(pos, dtype=torch.int32, device=gpu), window, 1.0 / math.sqrt(hd))
+    return out, torch.cat(refs)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 16, 8), (6, 1, 32, 16), (32, 8, 128, 16), (5, 5, 48, 1), (3, 1, 256, 64),
+                                            (8, 2, 80, 4), (2, 1, 112, 16)])
+def test_attention_mixed_batch(gpu, dtype, nh, nkv, hd, page):
+    seqs = [(70, 70), (130, 1), (33, 7), (1, 1), (64, 2), (257, 1)]
+    out, ref = paged_case(gpu, dtype, nh, nkv, hd, page, seqs, 0)
+    close(out, ref, dtype, f32=3e-6)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("window,page", [(24, 8), (1, 4), (64, 16), (65, 16), (7, 1)])
+def test_attention_window(gpu, dtype, window, page):
+    seqs = [(100, 100), (200, 1), (90, 30), (window, 1), (window + 1, 1)]
+    out, ref = paged_case(gpu, dtype, 6, 2, 48, page, seqs, window)
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, dtype, f32=3e-6)
+
+
+def test_attention_far_key_and_window_edge(gpu):
+    """Random keys would hide a key that is never read: one far key is made to stand out so that it
+    takes nearly all the weight, once inside the window's edge and once just outside."""
+    hd = 32
+
+    def trick(i, q, k, v):
+        q[:] = 0
+        q[:, :, 0] = 12.0
+        k[:, :, 0] = 0
+        k[3, :, 0] = 12.0 * math.sqrt(hd)        # key 3 of hundreds
+
+    out, ref = paged_case(gpu, torch.float32, 2, 1, hd, 16, [(300, 1), (300, 300)], 0, scale_trick=trick)
+    close(out, ref, torch.float32, f32=3e-6)
+    # window edge: the query at position 99 sees keys 80..99 with window 20
+    for hot, seen in ((80, True), (79, False)):
+        def trick2(i, q, k, v, hot=hot):
+            q[:] = 0
+            q[:, :, 0] = 12.0
+            k[:, :, 0] = 0
+            k[hot, :, 0] = 12.0 * math.sqrt(hd)
+            v[hot] = 100.0
+        out, ref = paged_case(gpu, torch.float32, 2, 1, hd, 16, [(100, 1)], 20, scale_trick=trick2)
+        close(out, ref, torch.float32, f32=3e-6)
+        assert (float(out.abs().max()) > 50.0) == seen
+
+
+def test_attention_is_independent_of_pages_and_batch(gpu):
+    a, _ = paged_case(gpu, torch.float32, 4, 2, 64, 16, [(150, 150)], 0, seed=5)
+    b, _ = paged_case(gpu, torch.float32, 4, 2, 64, 4, [(150, 150)], 0, seed=5)       # other page size, other pages
+    assert torch.equal(a, b)
+
+
+# ---- sampling ---------------------------------------------------------------------------------
+def test_argmax(gpu):
+    # crates/prelude-core/src/engine/sampling/logits_processor.rs:144-149 and ties to the lowest index
+    x = torch.tensor([[0.1, 0.2, 0.9, 0.3], [0.9, 0.2, 0.9, 0.3], [-1.0, -1.0, -1.0, -1.0]])
+    assert K().argmax(x.to(gpu)).tolist() == [2, 0, 0]
+    big = rnd(5, 151936)
+    big[1, 150000] = 50.0
+    big[2, 7] = big[2, 140001] = 60.0
+    assert K().argmax(big.to(gpu)).tolist() == torch.argmax(big, dim=-1).tolist()
+    assert K().argmax(big.to(gpu)).tolist()[2] == 7
+
+
+@pytest.mark.parametrize("vocab", [509, 151936])
+def test_sample_matches_the_plain_draw(gpu, vocab):
+    g = torch.Generator().manual_seed(3)
+    rows = 24
+    logits = 3.0 * torch.randn(rows, vocab, generator=g)
+    temps = [0.0, 0.8, 1.0, 0.3, 1.5, 0.8] * 4
+    topk = [0, 0, 5, 0, 50, 20] * 4
+    topp = [1.0, 1.0, 1.0, 0.9, 0.5, 0.95] * 4
+    u = torch.rand(rows, generator=g)
+    out = K().sample(logits.to(gpu), torch.tensor(temps).to(gpu), torch.tensor(topk, dtype=torch.int32).to(gpu),
+                     torch.tensor(topp).to(gpu), u.to(gpu)).tolist()
+    checked = 0
+    for r in range(rows):
+        if temps[r] < 1e-7:
+            assert out[r] == int(torch.argmax(logits[r]))
+            continue
+        prs = pm.sampling_probs(logits[r], temps[r], topk[r] or None, topp[r] if topp[r] < 1.0 else None)
+        assert prs[out[r]] > 0, f"row {r}: token {out[r]} is outside the kept set"
+        cdf = torch.cumsum(prs, 0)
+        target = float(u[r]) * float(cdf[-1])
+        # compare only where 32-bit summation cannot move the draw across a boundary
+        if float((cdf - target).abs().min()) > 1e-4 * float(cdf[-1]):
+            assert out[r] == pm.draw(prs, float(u[r])), f"row {r}"
+            checked += 1
+    assert checked >= rows // 2
+
+
+def test_sample_statistics_and_limits(gpu):
+    logits = torch.tensor([[2.0, 1.0, 0.5, -1.0, 0.0]]).repeat(4000, 1)
+    g = torch.Generator().manual_seed(0)
+    u = torch.rand(4000, generator=g)
+    z = lambda v, dt=torch.float32: torch.full((4000,), v, dtype=dt).to(gpu)
+    out = K().sample(logits.to(gpu), z(0.8), z(0, torch.int32), z(1.0), u.to(gpu)).cpu()
+    freq = torch.bincount(out.long(), minlength=5).double() / 4000
+    assert float((freq - torch.softmax(logits[0].double() / 0.8, -1)).abs().max()) < 0.03
+    out = K().sample(logits.to(gpu), z(1.0), z(2, torch.int32), z(1.0), u.to(gpu)).cpu()
+    assert set(out.tolist()) == {0, 1}                                       # top-2 stays in {0, 1}
+    out = K().sample(logits.to(gpu), z(1e-9), z(0, torch.int32), z(1.0), u.to(gpu)).cpu()
+    assert set(out.tolist()) == {0}                                          # T -> 0 is the argmax
+    out = K().sample(logits.to(gpu), z(1.0), z(0, torch.int32), z(0.4), u.to(gpu)).cpu()
+    assert set(out.tolist()) == {0}                                          # the first entry alone reaches p = 0.4

@@ -1,0 +1,215 @@
+"""Trace replay against the plain implementation: whole, last 32 decoded, changing portions, mixed with page reuse."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import PAGE, check, model_folder, reference_logits
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"a": 100, "b": 180, "c": 150}
+
+
+def runner(name, dtype, max_tokens):
+    from prelude_amd.trace import TraceRunner
+    folder, _, _ = model_folder(name)
+    return TraceRunner(folder, dtype, max_tokens, page_size=PAGE[name])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_whole_sequence(gpu, name, dtype):
+    toks, ref = reference_logits(name, 0, LENGTHS[name])
+    r = runner(name, dtype, 256)
+    got = r.step([{"id": "x", "tokens": toks, "want": list(range(len(toks)))}], ["x"])
+    check(got, ref, dtype, f"{name} whole")
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_last_32_tokens_one_by_one(gpu, name, dtype):
+    toks, ref = reference_logits(name, 1, LENGTHS[name])
+    n = len(toks) - 32
+    r = runner(name, dtype, 256)
+    outs = [r.step([{"id": 0, "tokens": toks[:n], "want": list(range(n))}])]
+    for i in range(n, len(toks)):
+        outs.append(r.step([{"id": 0, "tokens": [toks[i]], "want": [0]}]))
+    check(np.concatenate(outs), ref, dtype, f"{name} prefill + 32 decode")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_portions_of_changing_size(gpu, name, dtype):
+    toks, ref = reference_logits(name, 2, LENGTHS[name])
+    sizes = [7, 2, 13, 2, 1, 31, 2, 9, 16, 3, 8, 2]
+    r = runner(name, dtype, 256)
+    outs, i, k = [], 0, 0
+    while i < len(toks):
+        n = min(sizes[k % len(sizes)], len(toks) - i)
+        k += 1
+        outs.append(r.step([{"id": "p", "tokens": toks[i:i + n], "want": list(range(n))}]))
+        i += n
+    check(np.concatenate(outs), ref, dtype, f"{name} portions")
+
+
+def mixed_trace(name, lengths, max_live=4, seed=0):
+    """Steps over several requests: up to max_live at a time, portions of some beside single
+    tokens of others, some left out of a step; a request ends as soon as it is fed."""
+    rng = np.random.default_rng(seed)
+    seqs = [reference_logits(name, 10 + i, n) for i, n in enumerate(lengths)]
+    fed = [0] * len(seqs)
+    waiting = list(range(len(seqs)))
+    live, steps = [], []
+    mode = {}
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            r = waiting.pop(0)
+            live.append(r)
+            mode[r] = "portion"
+        entries, end = [], []
+        for r in list(live):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                                           # left out of this step
+            left = len(seqs[r][0]) - fed[r]
+            if mode[r] == "portion":
+                n = int(min(left, rng.choice([2, 3, 5, 11, 17, 40])))
+                if fed[r] + n >= len(seqs[r][0]) * 0.6:
+                    mode[r] = "decode"
+            else:
+                n = 1
+            entries.append({"id": f"r{r}", "tokens": seqs[r][0][fed[r]:fed[r] + n], "want": list(range(n)),
+                            "_r": r, "_at": fed[r]})
+            fed[r] += n
+            if fed[r] == len(seqs[r][0]):
+                end.append(f"r{r}")
+                live.remove(r)
+        if entries:
+            steps.append((entries, end))
+    return seqs, steps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_mixed_batches_with_page_reuse(gpu, name, dtype):
+    lengths = {"a": [70, 45, 100, 33, 64, 90, 20, 128, 77, 50, 110, 60],
+               "b": [130, 60, 200, 31, 90, 150, 64, 256, 100, 40, 180, 75],
+               "c": [120, 40, 300, 64, 90, 200, 33, 500, 150, 260, 70, 400]}[name]
+    seqs, steps = mixed_trace(name, lengths, seed=3)
+    # the pool holds the four largest requests, each rounded up to 64: later requests get used pages
+    pool = sum(sorted(-(-n // 64) * 64 for n in lengths)[-4:])
+    r = runner(name, dtype, pool)
+    pages_seen = set()
+    reused = False
+    got = [np.zeros((len(s[0]), s[1].shape[1])) for s in seqs]
+    for entries, end in steps:
+        out = r.step([{k: v for k, v in e.items() if not k.startswith("_")} for e in entries], [])
+        row = 0
+        for e in entries:
+            n = len(e["tokens"])
+            got[e["_r"]][e["_at"]:e["_at"] + n] = out[row:row + n]
+            row += n
+            table = set(p for p in r.engine.tables.table(r._ids[e["id"]], 0) if p >= 0)
+            if e["_at"] == 0 and table & pages_seen:
+                reused = True
+            pages_seen |= table
+        r.step([], end)
+        assert r.engine.tables.audit() == ""
+    assert reused, "the trace never reused a page; make the pool smaller"
+    for i, (toks, ref) in enumerate(seqs):
+        check(got[i], ref, dtype, f"{name} mixed, request {i}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(gpu, dtype):
+    toks, ref = reference_logits("c", 5, 400)
+    r = runner("c", dtype, 448)
+    outs = [r.step([{"id": 0, "tokens": toks[:6], "want": list(range(6))}])]
+    for i in range(6, 400):
+        outs.append(r.step([{"id": 0, "tokens": [toks[i]], "want": [0]}]))
+    check(np.concatenate(outs), ref, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_first_tokens(gpu, name, dtype):
+    toks, ref = reference_logits(name, 6, 4)
+    r = runner(name, dtype, 64)
+    for n in (1, 2, 3, 4):
+        got = r.step([{"id": n, "tokens": toks[:n], "want": list(range(n))}], [n])
+        check(got, ref[:n], dtype, f"{name} first {n}")
+    outs = [r.step([{"id": "d", "tokens": [toks[i]], "want": [0]}]) for i in range(4)]   # from the very first token
+    check(np.concatenate(outs), ref, dtype, f"{name} decode from token 0")
+
+
+def test_wanted_places_only(gpu):
+    toks, ref = reference_logits("b", 7, 50)
+    r = runner("b", "float32", 128)
+    assert r.step([{"id": 0, "tokens": toks[:20], "want": []}]) is None
+    got = r.step([{"id": 0, "tokens": toks[20:50], "want": [29, 0, 7]}, {"id": 1, "tokens": toks[:5], "want": [4]}])
+    check(got[:3], ref[[49, 20, 27]], "float32", "wanted rows in the order asked")
+    check(got[3:], ref[[4]], "float32", "second request")
+
+
+def test_bfloat16_storage_is_used_as_stored(gpu):
+    """A folder stored in bfloat16, run in float32: the engine widens exactly, so it matches the plain
+    implementation on the rounded weights to float32 accuracy."""
+    from prelude_amd.trace import TraceRunner
+    folder, _, _ = model_folder("a", "bfloat16")
+    toks, ref = reference_logits("a", 8, 60, "bfloat16")
+    r = TraceRunner(folder, "float32", 128, page_size=8)
+    got = r.step([{"id": 0, "tokens": toks, "want": list(range(60))}])
+    check(got, ref, "float32", "bf16-stored weights in the 32-bit path")
+
+
+def test_errors_leave_the_cache_intact(gpu):
+    from prelude_amd.cache import OutOfPages
+    from prelude_amd.engine import StepError
+    toks, _ = reference_logits("a", 9, 100)
+    r = runner("a", "float32", 64)
+    r.step([{"id": 0, "tokens": toks[:40], "want": []}])
+    with pytest.raises(OutOfPages):
+        r.step([{"id": 1, "tokens": toks[:40], "want": []}])
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 1
+    with pytest.raises(StepError, match="vocabulary"):
+        r.step([{"id": 0, "tokens": [5, 256], "want": []}])
+    with pytest.raises(StepError, match="wanted place"):
+        r.step([{"id": 0, "tokens": [5], "want": [1]}])
+    with pytest.raises(StepError, match="max_position_embeddings"):
+        r.step([{"id": 0, "tokens": toks[:89], "want": []}])
+    assert r.engine.length(0) == 40
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_program(gpu, dtype, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and `done <step>` lines out."""
+    folder, cfg, _ = model_folder("b")
+    toks, ref = reference_logits("b", 0, 180)
+    toks2, ref2 = reference_logits("b", 1, 180)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks[:50], "want": [0, 49]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks[50:52], "want": []},
+                                {"id": "b", "tokens": toks2[:30], "want": [29]}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks[52:53], "want": [0]},
+                                {"id": "b", "tokens": toks2[30:31], "want": [0]}], "end": ["a"]},
+        {"step": 5, "entries": [{"id": "b", "tokens": toks2[31:40], "want": [8]}], "end": ["b"]},
+    ]
+    out = tmp_path / "out"
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+                        "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 5"]
+    v = cfg["vocab_size"]
+    load = lambda s: np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(-1, v)
+    check(load(0), ref[[0, 49]], dtype, "step 0")
+    check(load(1), ref2[[29]], dtype, "step 1")
+    check(load(2), torch.stack([ref[52], ref2[30]]), dtype, "step 2")
+    check(load(5), ref2[[39]], dtype, "step 5")
+    assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "2.f32", "5.f32"]

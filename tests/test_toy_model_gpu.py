@@ -1,0 +1,199 @@
+"""Generality of the parts: a toy mixer with state of its own and a toy architecture, both defined here, are
+registered, built, loaded from a folder the random-weights mode writes, and stepped -- without a change to the
+framework's files.  The toy model also names a layer twice in its run order and lets a run read another run's cache.
+It is no model of anyone's: a decaying sum as mixer, beside the framework's attention in the other layer.
+"""
+import dataclasses
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+
+
+def register_toy():
+    from prelude_amd.config.registry import Architecture, register_architecture
+    from prelude_amd.models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
+    from prelude_amd.ops import kernels as K
+    from prelude_amd.parts import MATRIX, Mixer, StateSpec, TensorReq, register_part
+
+    @register_part("mixer", "toy_decay")
+    class ToyDecay(Mixer):
+        """s_t = decay * s_{t-1} + x_t per request; y_t = W s_t.  The state s lives in a slot of the cache manager."""
+
+        def __init__(self, hidden_size, decay):
+            self.hidden_size, self.decay = hidden_size, decay
+            self.w = None
+
+        def cache_spec(self):
+            return StateSpec((("s", (self.hidden_size,), torch.float32),))
+
+        def tensors(self):
+            return {"proj.weight": TensorReq((self.hidden_size, self.hidden_size), MATRIX)}
+
+        def load(self, tensors, dtype, device):
+            self.w = tensors["proj.weight"]
+
+        def forward(self, x, step, cache, write_cache=True):
+            s_all = cache.tensors["s"]
+            out = torch.empty_like(x)
+            t = 0
+            for i, n in enumerate(step.q_lens):            # a request's portion is processed in order
+                slot = step.state_slots_host[i]
+                s = s_all[slot].clone()
+                for j in range(n):
+                    s = self.decay * s + x[t + j].float()
+                    out[t + j] = s.to(x.dtype)
+                s_all[slot] = s
+                t += n
+            return K.linear(out, self.w)
+
+    @dataclasses.dataclass
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        inter: int
+        heads: int
+        head_dim: int
+        decay: float
+        eps: float
+        max_positions: int
+
+    def parse(raw):
+        return ToyConfig(**{f.name: raw[f.name] for f in dataclasses.fields(ToyConfig)})
+
+    def spec(c):
+        norm = lambda name: PartSpec("rms_norm", dict(size=c.hidden_size, eps=c.eps), {"weight": name})
+        ffn = lambda p: PartSpec("gated_mlp", dict(hidden_size=c.hidden_size, intermediate_size=c.inter),
+                                 {f"{x}_proj.weight": f"{p}.ffn.{x}" for x in ("gate", "up", "down")})
+        toy = LayerSpec("prenorm", {"input_norm": norm("l0.n1"), "post_mixer_norm": norm("l0.n2"), "ffn": ffn("l0"),
+                                    "mixer": PartSpec("toy_decay", dict(hidden_size=c.hidden_size, decay=c.decay),
+                                                      {"proj.weight": "l0.mix.proj"})})
+        attn = LayerSpec("prenorm", {"input_norm": norm("l1.n1"), "post_mixer_norm": norm("l1.n2"), "ffn": ffn("l1"),
+                                     "mixer": PartSpec("gqa_attention", dict(
+                                         hidden_size=c.hidden_size, num_heads=c.heads, num_kv_heads=1,
+                                         head_dim=c.head_dim, norm_eps=c.eps, qk_norm=False, position="rope"),
+                                         {f"{x}_proj.weight": f"l1.attn.{x}" for x in "qkvo"})})
+        # layer 0 twice (two states per request), and the last run reads the keys and values run 1 wrote
+        order = [RunSpec(0), RunSpec(1), RunSpec(0), RunSpec(1, reads_cache_of=1)]
+        return ModelSpec("ToyForCausalLM", c.vocab_size, c.hidden_size, c.max_positions, (0,),
+                         PartSpec("token_embedding", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "emb"}),
+                         [toy, attn], order, norm("final"),
+                         PartSpec("linear_head", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "emb"}),
+                         {"rope": PartSpec("rope", dict(rotary_dim=c.head_dim, max_positions=c.max_positions, theta=100.0))})
+
+    register_architecture(Architecture("toy", ("Toy",), ("toy",), parse, spec))
+
+
+RAW = dict(architectures=["ToyForCausalLM"], vocab_size=97, hidden_size=48, inter=80, heads=3, head_dim=16, decay=0.7,
+           eps=1e-5, max_positions=128)
+
+
+def plain_toy(w, toks):
+    """The toy model for a whole sequence, in float64, from plain_model's functions."""
+    w = {k: v.double() for k, v in w.items()}
+    n = len(toks)
+    cos, sin = pm.rope_tables(16, 128, 100.0)
+    x = w["emb"][toks]
+
+    def toy(x, p):
+        h = pm.rms_norm(x, w[p + ".n1"], 1e-5)
+        s = torch.zeros(48, dtype=torch.float64)
+        ys = []
+        for t in range(n):
+            s = 0.7 * s + h[t]
+            ys.append(s.float().double())     # the state is kept in 32-bit
+        x = x + torch.stack(ys) @ w[p + ".mix.proj"].T
+        return x + pm.swiglu(pm.rms_norm(x, w[p + ".n2"], 1e-5), w[p + ".ffn.gate"], w[p + ".ffn.up"], w[p + ".ffn.down"])
+
+    def attn(x, p, kv=None):
+        h = pm.rms_norm(x, w[p + ".n1"], 1e-5)
+        q = pm.apply_rope((h @ w[p + ".attn.q"].T).reshape(n, 3, 16), cos[:n], sin[:n])
+        if kv is None:
+            k = pm.apply_rope((h @ w[p + ".attn.k"].T).reshape(n, 1, 16), cos[:n], sin[:n])
+            kv = (k, (h @ w[p + ".attn.v"].T).reshape(n, 1, 16))
+        o = pm.attention(q, kv[0], kv[1], 0.25)
+        x = x + o.reshape(n, 48) @ w[p + ".attn.o"].T
+        x = x + pm.swiglu(pm.rms_norm(x, w[p + ".n2"], 1e-5), w[p + ".ffn.gate"], w[p + ".ffn.up"], w[p + ".ffn.down"])
+        return x, kv
+
+    x = toy(x, "l0")
+    x, kv = attn(x, "l1")
+    x = toy(x, "l0")
+    x, _ = attn(x, "l1", kv)
+    return pm.rms_norm(x, w["final"], 1e-5) @ w["emb"].T
+
+
+def test_toy_model_is_built_and_stepped(gpu, tmp_path):
+    register_toy()
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    from prelude_amd.weights import WeightFiles, write_random_model
+    folder = write_random_model(RAW, str(tmp_path / "toy"), seed=4, std=0.2, norm_std=0.1, dtype=torch.float32)
+    files = WeightFiles(folder)
+    w = {n: files.tensor(n).clone() for n in files.names()}
+    assert set(w) == {"emb", "final"} | {f"l{i}.n{j}" for i in (0, 1) for j in (1, 2)} | {"l0.mix.proj"} | \
+        {f"l{i}.ffn.{x}" for i in (0, 1) for x in ("gate", "up", "down")} | {f"l1.attn.{x}" for x in "qkvo"}
+    eng = Engine.from_model_dir(folder, EngineConfig(dtype="float32", page_size=8, max_cache_tokens=128, max_state_slots=2))
+    m = eng.model
+    assert m.needs_state and len(m.cache_slots) == 3 and m.run_cache == [0, 1, 2, 1]      # two states, one KV cache
+    g = torch.Generator().manual_seed(0)
+    seqs = [torch.randint(0, 97, (n,), generator=g).tolist() for n in (50, 31, 44)]
+    refs = [plain_toy(w, s) for s in seqs]
+
+    def close(got, ref):
+        assert float((got.double().cpu() - ref).abs().max()) < 2e-5 * max(1.0, float(ref.abs().max()))
+
+    # whole
+    close(eng.step([StepEntry(0, seqs[0], list(range(50)))]), refs[0])
+    eng.release(0)
+    # two requests in portions, mixed in one batch: state is carried across portions and kept apart per request
+    got = {1: [], 2: []}
+    cuts = {1: [7, 2, 20, 1, 1], 2: [3, 11, 1, 5, 24]}
+    at = {1: 0, 2: 0}
+    for k in range(5):
+        entries = []
+        for rid in (1, 2):
+            n = cuts[rid][k]
+            entries.append(StepEntry(rid, seqs[rid][at[rid]:at[rid] + n], list(range(n))))
+            at[rid] += n
+        out = eng.step(entries)
+        got[1].append(out[:cuts[1][k]])
+        got[2].append(out[cuts[1][k]:])
+    close(torch.cat(got[1]), refs[1][:31])
+    close(torch.cat(got[2]), refs[2][:44])
+    # both slots are taken: a third request cannot open; after a release its slot starts from zero again
+    from prelude_amd.cache import CacheError
+    with pytest.raises(CacheError, match="state slot"):
+        eng.step([StepEntry(3, seqs[0][:4], [3])])
+    assert eng.tables.audit() == ""
+    eng.release(1)
+    close(eng.step([StepEntry(3, seqs[0], list(range(50)))]), refs[0])
+    eng.release(2)
+    eng.release(3)
+    assert eng.tables.audit() == "" and eng.tables.free_state_slots() == 2
+
+
+def test_toy_model_generates_through_the_entry_point(gpu, tmp_path):
+    register_toy()
+    from prelude_amd import LLM
+    from prelude_amd.weights import WeightFiles, write_random_model
+    folder = write_random_model(RAW, str(tmp_path / "toy"), seed=5, std=0.2, norm_std=0.1, dtype=torch.float32)
+    files = WeightFiles(folder)
+    w = {n: files.tensor(n).clone() for n in files.names()}
+    llm = LLM(folder, dtype="float32", page_size=8, max_cache_tokens=256, max_state_slots=2, max_num_batched_tokens=16)
+    prompts = [[5, 6, 7, 8, 9] * 5, [11, 12, 13], [20] * 30]           # three requests over two state slots
+    outs = llm.generate(prompts, max_tokens=6, temperature=0.0)
+    for p, o in zip(prompts, outs):
+        seq = list(p)
+        for tok in o.token_ids:
+            assert tok == int(torch.argmax(plain_toy(w, seq)[-1]))
+            seq.append(tok)
+        assert o.finish_reason in ("length", "eos")
+    assert llm.engine.tables.audit() == "" and llm.engine.tables.free_state_slots() == 2
