@@ -8,10 +8,13 @@ them.  Beside the pages there is a pool of slots for per-request state of
 fixed size (crates/prelude-core/src/scheduler/components/cache/deltanet_pool.rs:54-173),
 one slot per live request when the model has a mixer that keeps such state.
 
-Layout of a group's pages on the device, per cache slot: K and V each
-``[pages, kv_heads, page_size, head_dim]`` -- one (page, head) tile is
-contiguous, so a wavefront streaming a head's keys reads whole lines
-(the reference keeps ``[pages, page_size, kv_heads, head_dim]``,
+Layout of a group's pages on the device, per cache slot: K
+``[pages, kv_heads, page_size, head_dim]`` and V transposed
+``[pages, kv_heads, head_dim, page_size]`` -- one (page, head) tile is
+contiguous, so a wavefront streaming a head's keys reads whole lines, and
+both tiles can be loaded straight into matrix-core operands: the contraction
+index (head_dim for Q.K, keys for P.V) is the contiguous one in each
+(the reference keeps ``[pages, page_size, kv_heads, head_dim]`` for both,
 crates/prelude-core/src/scheduler/components/cache/manager.rs:286-329).
 """
 from __future__ import annotations
@@ -151,6 +154,7 @@ class PageTables:
         G = len(self.groups)
         sizes = [("token_ids", total), ("positions", total), ("seq_of_token", total), ("cu_q", n + 1),
                  ("context_lens", n), ("state_slots", n), ("fresh", n), ("want_rows", wanted),
+                 ("decode_seqs", n), ("prefill_seqs", n),
                  ("block_tables", G * n * stride), ("slots", G * total)]
         out, off = {}, 0
         for name, sz in sizes:
@@ -181,7 +185,7 @@ class PageTables:
 class KVLayerCache:
     """What an attention-like mixer gets: its pages and the group whose tables index them."""
     k: torch.Tensor   # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor   # [pages, kv_heads, head_dim, page_size]
     group: int
 
 
@@ -221,9 +225,9 @@ def allocate_storage(cache_specs: Sequence[object], of_slot: Sequence[Optional[i
     out: List[object] = []
     for cs, g in zip(cache_specs, of_slot):
         if isinstance(cs, KVCacheSpec):
-            shape = (pages_per_group[g], cs.num_kv_heads, page_size, cs.head_dim)
-            out.append(KVLayerCache(torch.zeros(shape, dtype=dtype, device=device),
-                                    torch.zeros(shape, dtype=dtype, device=device), g))
+            n = pages_per_group[g]
+            out.append(KVLayerCache(torch.zeros((n, cs.num_kv_heads, page_size, cs.head_dim), dtype=dtype, device=device),
+                                    torch.zeros((n, cs.num_kv_heads, cs.head_dim, page_size), dtype=dtype, device=device), g))
         elif isinstance(cs, StateSpec):
             out.append(StateLayerCache({name: torch.zeros((state_slots, *shape), dtype=dt, device=device)
                                         for name, shape, dt in cs.tensors}))

@@ -18,14 +18,15 @@ int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, 
 // with `rows`, output row r comes from input row rows[r] and the residual is left alone.
 int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out, const int* rows,
                int nrows, int hidden, float eps);
-// out[t, c] = silu(gate_up[t, c]) * gate_up[t, inter + c]
+// out[t, c] = silu(gate_up[t, 2c]) * gate_up[t, 2c + 1]   (columns alternate gate_j, up_j)
 int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter);
 int pa_gather_rows(void* stream, int dtype, const void* x, const int* rows, void* out, int nrows, int width);
 int pa_add_bias(void* stream, int dtype, void* y, const float* b, int tokens, int width);
 int pa_to_f32(void* stream, int dtype, const void* x, float* out, long total);
 
 // qkv [tokens, (nh + 2 nkv) * hd] -> q_out [tokens, nh, hd] (normed, rotated) and, where slots[t] >= 0,
-// K (normed, rotated) and V into caches laid out [page, nkv, page_size, hd]; slot = page * page_size + offset.
+// K (normed, rotated) into a cache laid out [page, nkv, page_size, hd] and V into one laid out
+// [page, nkv, hd, page_size]; slot = page * page_size + offset.
 int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_weight, const float* k_weight,
                       const float* cos_table, const float* sin_table, const int* positions, const int* slots,
                       void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int hd, int rot,
@@ -35,10 +36,29 @@ int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_w
 int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, const void* w, const float* bias, void* c,
                   int m, int n, int k, long lda, long ldw, long ldc);
 
+// C[m, n] = X[m, k] W[n, k]^T for m <= 64 in bfloat16 (32-bit accumulation); out_dtype 0 = float32, 1 = bfloat16.
+// epilogue 0: (+ bias[n]); 1: C[m, n/2] = silu(gate) * up for a weight whose rows alternate gate_j, up_j.
+int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
+                   int m, int n, int k, long ldx, long ldc);
+
 // Paged causal attention, one query token per (seq_of_token[t], positions[t]); window 0 = all keys.
 int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
                     const int* block_table, int table_stride, const int* seq_of_token, const int* positions, void* out,
                     int tokens, int nh, int nkv, int hd, int page_size, int window, float scale);
+
+// Matrix-core attention in bfloat16 (K cache [page, nkv, page_size, hd], V cache [page, nkv, hd, page_size]).
+// seq_ids lists the sequences of the step a call handles; cu_q[s] is the first packed token row of sequence s,
+// context_lens[s] its tokens in the cache after the step.  Decode takes sequences that feed one token and cuts
+// each one's keys into splits of split_keys; workspace must hold pa_attn_decode_workspace(...) floats.
+int pa_attn_mfma_supports(int hd, int page_size);
+long pa_attn_decode_workspace(int nseq, int nh, int hd, int max_splits);
+int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                   float* workspace, int nseq, int nh, int nkv, int hd, int page_size, int window, float scale,
+                   int split_keys, int max_splits);
+int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                    int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window, float scale);
 
 // out[r] = index of the largest of logits[r, :], the lowest index among equals.
 int pa_argmax(void* stream, const float* logits, int* out, int rows, int vocab);

@@ -10,6 +10,8 @@
 // result for a token is bit-identical whether it arrives in a whole prompt,
 // in a portion, or as a single decode token, and whatever pages hold its keys.
 //
+// K pages are [page, kv_head, offset, head_dim], V pages [page, kv_head, head_dim, offset].
+//
 // Formula: crates/prelude-core/src/models/qwen3.rs:276-370 and
 // crates/prelude-core/src/ops/traits/attention.rs:10-99 (scores q.k * scale,
 // key c visible to the query at position p when c <= p and, with a window of
@@ -74,12 +76,12 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
       for (int j = j_lo; j <= j_hi; ++j) {
         const int cj = c0 + j;
         const int page = table[cj / page_size];
-        const T* vr = v_cache + (((size_t)page * nkv + kvh) * page_size + (cj % page_size)) * hd;
+        const T* vr = v_cache + ((size_t)page * nkv + kvh) * hd * page_size + (cj % page_size);
         const float pj = ps[wave][j];
 #pragma unroll
         for (int e = 0; e < kAttnMaxHd / kWave; ++e) {
           const int d = lane + e * kWave;
-          if (d < hd) o[e] = fmaf(pj, to_f32(vr[d]), o[e]);
+          if (d < hd) o[e] = fmaf(pj, to_f32(vr[(size_t)d * page_size]), o[e]);
         }
       }
     }

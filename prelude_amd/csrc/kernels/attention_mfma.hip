@@ -1,0 +1,472 @@
+// Paged causal attention on the matrix cores (bfloat16 in, 32-bit softmax and
+// accumulation), in two kernels that share their inner step:
+//
+//   attn_decode  -- one query token per sequence; the keys of a sequence are
+//                   cut into splits of a fixed number of keys, each workgroup
+//                   reduces one split, a second kernel merges the splits.
+//   attn_prefill -- portions of several tokens; a wavefront owns 16 tokens of
+//                   up to four query heads that share a KV head and walks the
+//                   keys they may see.
+//
+// Both compute S^T = K Q^T and O^T = V^T P^T with v_mfma_f32_16x16x32_bf16, so
+// that a query is a column (lane % 16) in the scores and in the output alike:
+// the running maximum, the sum and the rescaling stay in the lane, and the
+// probabilities leave the first product in exactly the register layout the
+// second one wants.  K pages are [page, kv_head, offset, head_dim] and V pages
+// [page, kv_head, head_dim, offset]: in both, the contraction index of the
+// product they feed is contiguous, so every operand is loaded from memory
+// straight into registers, with no staging in LDS and no barrier in the loop.
+//
+// Operand layout of v_mfma_f32_16x16x32_bf16 (lane l, g = l / 16, r = l % 16):
+//   A[16 x 32]: row r,    columns 8g .. 8g+7        B[32 x 16]: column r, rows 8g .. 8g+7
+//   C[16 x 16]: column r, rows 4g .. 4g+3
+// For 32 keys, two score tiles give lane (g, r) the keys {4g..4g+3} and
+// {16+4g..16+4g+3} of query r; packed in that order they are the B operand of
+// O^T = V^T P^T, whose A operand takes the same eight keys of one head_dim row
+// of V^T: two 8-byte loads.
+//
+// Reference counterparts: the FA4 / FlashInfer paged kernels the reference
+// calls (crates/prelude-cuda/src/attn/flash_v4.rs:125-277,
+// crates/prelude-cuda/src/attn/flashinfer.rs:737-797); formula as in
+// crates/prelude-core/src/ops/traits/attention.rs:10-99.
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float xor_max16_32(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  return fmaxf(v, __shfl_xor(v, 32, kWave));
+}
+__device__ __forceinline__ float xor_sum16_32(float v) {
+  v += __shfl_xor(v, 16, kWave);
+  return v + __shfl_xor(v, 32, kWave);
+}
+
+// What a wavefront keeps per head while it walks keys: per lane, query column r.
+template <int HD>
+struct HeadState {
+  static constexpr int OT = HD / 16;
+  float m = -INFINITY;  // running maximum of the scaled scores (log2 domain), equal in the four lanes of a column
+  float l = 0.f;        // this lane's share of the running sum
+  f32x4 o[OT];          // O^T tiles: head_dim rows 16 t + 4g + i, column r
+  __device__ HeadState() {
+#pragma unroll
+    for (int t = 0; t < OT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+};
+
+template <int HD>
+struct KFrag {
+  static constexpr int KS = (HD + 31) / 32;
+  bf16x8 k[2][KS];
+};
+
+struct KeyWalk {
+  const bf16* kc;
+  const bf16* vc;
+  const int* table;
+  int nkv, kvh, page_size;
+  int lo, hi;  // keys [lo, hi) exist and may be read
+};
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+  return z;
+}
+
+// K rows of keys key0 .. key0+31 as A operands.  Keys outside [lo, hi) are read
+// from the nearest key inside (their scores are masked by the caller).
+template <int HD>
+__device__ __forceinline__ void load_k(const KeyWalk& w, int key0, int g, int r, KFrag<HD>& f) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    int key = key0 + 16 * t + r;
+    key = key < w.lo ? w.lo : (key >= w.hi ? w.hi - 1 : key);
+    const int page = w.table[key / w.page_size];
+    const bf16* row = w.kc + (((size_t)page * w.nkv + w.kvh) * w.page_size + key % w.page_size) * HD + 8 * g;
+#pragma unroll
+    for (int s = 0; s < KFrag<HD>::KS; ++s) {
+      if (HD % 32 == 0 || 32 * s + 8 * g < HD) {
+        f.k[t][s] = *reinterpret_cast<const bf16x8*>(row + 32 * s);
+      } else {
+        f.k[t][s] = zero8();
+      }
+    }
+  }
+}
+
+// The eight keys of lane group g, for head_dim row `d`, as the A operand of O^T = V^T P^T.
+// A chunk of four keys never straddles a page (the page size is a multiple of 4).
+template <int HD>
+__device__ __forceinline__ bf16x8 load_v(const KeyWalk& w, int key0, int g, int d) {
+  union {
+    bf16x8 v;
+    short4_t h[2];
+  } u;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    int c = key0 + 16 * t + 4 * g;  // first key of the chunk
+    // a chunk wholly outside [lo, hi) is read from the chunk that holds the nearest key inside
+    if (c + 3 < w.lo) c = w.lo & ~3;
+    if (c >= w.hi) c = (w.hi - 1) & ~3;
+    const int page = w.table[c / w.page_size];
+    const bf16* p = w.vc + (((size_t)page * w.nkv + w.kvh) * HD + d) * w.page_size + c % w.page_size;
+    u.h[t] = *reinterpret_cast<const short4_t*>(p);
+  }
+  return u.v;
+}
+
+// One step over 32 keys for one head: scores, online softmax, output update.
+// `vis(key)` says whether this lane's query may see the key (and the key exists).
+template <int HD, typename Visible>
+__device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int r, const KFrag<HD>& kf,
+                                         const bf16x8* qf, float scale_log2e, HeadState<HD>& st, Visible vis) {
+  float s[8];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    f32x4 acc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KFrag<HD>::KS; ++ks) acc = mfma16(kf.k[t][ks], qf[ks], acc);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = key0 + 16 * t + 4 * g + i;
+      s[4 * t + i] = vis(key) ? acc[i] * scale_log2e : -INFINITY;
+    }
+  }
+  float mx = s[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+  mx = xor_max16_32(mx);
+  const float m_new = fmaxf(st.m, mx);
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a column that has seen no key yet
+  const float alpha = exp2f(st.m - m_safe);
+  bf16x8 pb;
+  float psum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float p = exp2f(s[i] - m_safe);
+    psum += p;
+    pb[i] = (bf16)p;
+  }
+  st.l = st.l * alpha + psum;
+  st.m = m_new;
+#pragma unroll
+  for (int t = 0; t < HeadState<HD>::OT; ++t) {
+    const bf16x8 va = load_v<HD>(w, key0, g, 16 * t + r);
+    f32x4 o = st.o[t];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] *= alpha;
+    st.o[t] = mfma16(va, pb, o);
+  }
+}
+
+// Q^T of 16 queries of one head as B operands: lane (g, r) holds query r, head_dim 32 ks + 8g .. +7.
+template <int HD>
+__device__ __forceinline__ void load_q(const bf16* qrow, bool valid, int g, bf16x8* qf) {
+#pragma unroll
+  for (int ks = 0; ks < (HD + 31) / 32; ++ks) {
+    if (valid && (HD % 32 == 0 || 32 * ks + 8 * g < HD)) {
+      qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * g);
+    } else {
+      qf[ks] = zero8();
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// decode: grid (splits, nkv * qtiles, sequences), 4 wavefronts, each taking every fourth step of 32 keys
+// ---------------------------------------------------------------------------
+constexpr int kDecodeWaves = 4;
+
+template <int HD>
+__global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_size, int window,
+    float scale_log2e, int split_keys, int max_splits) {
+  constexpr int OT = HD / 16;
+  __shared__ float lds_o[kDecodeWaves][16][HD + 1];
+  __shared__ float lds_ml[kDecodeWaves][16][2];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int group = nh / nkv;
+  const int qtiles = (group + 15) / 16;
+  const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
+  const int seq = seq_ids[blockIdx.z];
+  const int ctx = context_lens[seq];
+  const int pos = ctx - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first_split = lo / split_keys;
+  const int nsplit = (ctx + split_keys - 1) / split_keys - first_split;
+  if ((int)blockIdx.x >= nsplit) return;
+  const int sp = first_split + blockIdx.x;
+  const int k_begin = sp * split_keys > lo ? sp * split_keys : lo;
+  const int k_end = (sp + 1) * split_keys < ctx ? (sp + 1) * split_keys : ctx;
+
+  KeyWalk w{kc, vc, block_table + (size_t)seq * table_stride, nkv, kvh, page_size, lo, ctx};
+  const int head = kvh * group + qt * 16 + r;  // this lane's query head
+  const bool qvalid = qt * 16 + r < group;
+  const size_t token = cu_q[seq];
+  bf16x8 qf[(HD + 31) / 32];
+  load_q<HD>(q + (token * nh + (qvalid ? head : 0)) * HD, qvalid, g, qf);
+
+  HeadState<HD> st;
+  const int step0 = (sp * split_keys) / 32;  // splits start at multiples of 32 keys
+  const int steps = split_keys / 32;
+  for (int i = wave; i < steps; i += kDecodeWaves) {
+    const int key0 = (step0 + i) * 32;
+    if (key0 + 32 <= k_begin || key0 >= k_end) continue;
+    KFrag<HD> kf;
+    load_k<HD>(w, key0, g, r, kf);
+    attend32<HD>(w, key0, g, r, kf, qf, scale_log2e, st, [&](int key) { return key >= k_begin && key < k_end; });
+  }
+  // merge the four wavefronts through LDS
+  const float l_wave = xor_sum16_32(st.l);
+  if (g == 0) {
+    lds_ml[wave][r][0] = st.m;
+    lds_ml[wave][r][1] = l_wave;
+  }
+#pragma unroll
+  for (int t = 0; t < OT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_o[wave][r][16 * t + 4 * g + i] = st.o[t][i];
+  __syncthreads();
+  const int nq = group - qt * 16 < 16 ? group - qt * 16 : 16;
+  for (int e = threadIdx.x; e < nq * HD; e += blockDim.x) {
+    const int qi = e / HD, d = e % HD;
+    float mm = lds_ml[0][qi][0];
+#pragma unroll
+    for (int v = 1; v < kDecodeWaves; ++v) mm = fmaxf(mm, lds_ml[v][qi][0]);
+    float o = 0.f, l = 0.f;
+#pragma unroll
+    for (int v = 0; v < kDecodeWaves; ++v) {
+      const float f = lds_ml[v][qi][0] == -INFINITY ? 0.f : exp2f(lds_ml[v][qi][0] - mm);
+      o += lds_o[v][qi][d] * f;
+      l += lds_ml[v][qi][1] * f;
+    }
+    const int h = kvh * group + qt * 16 + qi;
+    if (nsplit == 1) {
+      out[(token * nh + h) * HD + d] = (bf16)(o / l);
+    } else {
+      const size_t slot = ((size_t)blockIdx.z * nh + h) * max_splits + blockIdx.x;
+      part_o[slot * HD + d] = o;
+      if (d == 0) {
+        part_ml[slot * 2] = mm;
+        part_ml[slot * 2 + 1] = l;
+      }
+    }
+  }
+}
+
+// Merges the splits of one (sequence, head): grid (nh, sequences).
+template <int HD>
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         const int* __restrict__ seq_ids, const int* __restrict__ cu_q,
+                                         const int* __restrict__ context_lens, bf16* __restrict__ out, int nh,
+                                         int window, int split_keys, int max_splits) {
+  const int h = blockIdx.x;
+  const int seq = seq_ids[blockIdx.y];
+  const int ctx = context_lens[seq];
+  const int pos = ctx - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int nsplit = (ctx + split_keys - 1) / split_keys - lo / split_keys;
+  if (nsplit == 1) return;  // written by the first kernel
+  const size_t base = ((size_t)blockIdx.y * nh + h) * max_splits;
+  float mm = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  float l = 0.f;
+  for (int s = 0; s < nsplit; ++s) l += part_ml[(base + s) * 2 + 1] * exp2f(part_ml[(base + s) * 2] - mm);
+  const size_t token = cu_q[seq];
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < nsplit; ++s) o += part_o[(base + s) * HD + d] * exp2f(part_ml[(base + s) * 2] - mm);
+    out[(token * nh + h) * HD + d] = (bf16)(o / l);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// prefill: grid (tiles of 64 tokens, nkv * head groups, sequences); a wavefront owns 16 tokens x GT heads
+// ---------------------------------------------------------------------------
+template <int HD, int GT>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
+    int page_size, int window, float scale_log2e) {
+  constexpr int OT = HD / 16;
+  constexpr int KS = (HD + 31) / 32;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int group = nh / nkv;
+  const int hgroups = group / GT;
+  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int seq = seq_ids[blockIdx.z];
+  const int row0 = cu_q[seq];
+  const int q_len = cu_q[seq + 1] - row0;
+  const int ctx = context_lens[seq];
+  const int t0 = blockIdx.x * 64 + wave * 16;  // first token of this wavefront's tile, within the portion
+  if (t0 >= q_len) return;
+  const int start = ctx - q_len;                // position of the portion's first token
+  const bool qvalid = t0 + r < q_len;
+  const int my_pos = start + t0 + r;            // this lane's query position
+  const int last_pos = start + (t0 + 15 < q_len ? t0 + 15 : q_len - 1);
+  const int first_pos = start + t0;
+  const int lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+  const int hi = last_pos + 1;
+  const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+
+  KeyWalk w{kc, vc, block_table + (size_t)seq * table_stride, nkv, kvh, page_size, lo, hi};
+  bf16x8 qf[GT][KS];
+  HeadState<HD> st[GT];
+  const int head0 = kvh * group + hg * GT;
+#pragma unroll
+  for (int j = 0; j < GT; ++j)
+    load_q<HD>(q + ((size_t)(row0 + (qvalid ? t0 + r : 0)) * nh + head0 + j) * HD, qvalid, g, qf[j]);
+
+  for (int key0 = (lo / 32) * 32; key0 < hi; key0 += 32) {
+    KFrag<HD> kf;
+    load_k<HD>(w, key0, g, r, kf);
+#pragma unroll
+    for (int j = 0; j < GT; ++j)
+      attend32<HD>(w, key0, g, r, kf, qf[j], scale_log2e, st[j],
+                   [&](int key) { return key >= my_lo && key <= my_pos; });
+  }
+  if (!qvalid) return;
+#pragma unroll
+  for (int j = 0; j < GT; ++j) {
+    const float inv = 1.0f / xor_sum16_32(st[j].l);
+    bf16* orow = out + ((size_t)(row0 + t0 + r) * nh + head0 + j) * HD;
+#pragma unroll
+    for (int t = 0; t < OT; ++t) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(st[j].o[t][i] * inv);
+      *reinterpret_cast<bf16x4*>(orow + 16 * t + 4 * g) = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+template <int HD>
+int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
+                  int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                  float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_size, int window, float scale,
+                  int split_keys, int max_splits) {
+  const int qtiles = (nh / nkv + 15) / 16;
+  dim3 grid(max_splits, nkv * qtiles, nseq);
+  hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(kDecodeWaves * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
+                     (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
+                     part_ml, nh, nkv, page_size, window, scale * kLog2e, split_keys, max_splits);
+  if (int rc = check_launch("attn_decode")) return rc;
+  if (max_splits > 1) {
+    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(HD < 64 ? 64 : HD), 0, st, part_o, part_ml,
+                       seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys, max_splits);
+    return check_launch("attn_decode_merge");
+  }
+  return 0;
+}
+
+template <int HD, int GT>
+int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
+                      int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                      int nseq, int max_q_len, int nh, int nkv, int page_size, int window, float scale) {
+  dim3 grid((max_q_len + 63) / 64, nkv * (nh / nkv / GT), nseq);
+  hipLaunchKernelGGL((attn_prefill_kernel<HD, GT>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kc,
+                     (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, nh, nkv,
+                     page_size, window, scale * kLog2e);
+  return check_launch("attn_prefill");
+}
+
+template <int HD>
+int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
+                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
+                   int max_q_len, int nh, int nkv, int page_size, int window, float scale) {
+  const int group = nh / nkv;
+#define PA_GT(GT)                                                                                                   \
+  return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
+                                   max_q_len, nh, nkv, page_size, window, scale)
+  if (group % 4 == 0) PA_GT(4);
+  if (group % 2 == 0) PA_GT(2);
+  PA_GT(1);
+#undef PA_GT
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+#define PA_HD_SWITCH(hd, CALL)                                                                              \
+  switch (hd) {                                                                                             \
+    case 16: CALL(16);                                                                                      \
+    case 32: CALL(32);                                                                                      \
+    case 48: CALL(48);                                                                                      \
+    case 64: CALL(64);                                                                                      \
+    case 96: CALL(96);                                                                                      \
+    case 128: CALL(128);                                                                                    \
+    default: return pa::fail("MFMA attention: head_dim %d is not one of 16, 32, 48, 64, 96, 128", hd);      \
+  }
+
+static int check_common(const char* what, int nseq, int nh, int nkv, int page_size, int table_stride, int window) {
+  PA_REQUIRE(nseq > 0 && nh > 0 && nkv > 0 && table_stride > 0, "%s: bad sizes sequences=%d nh=%d nkv=%d table_stride=%d",
+             what, nseq, nh, nkv, table_stride);
+  PA_REQUIRE(nh % nkv == 0, "%s: %d query heads are not a multiple of %d KV heads", what, nh, nkv);
+  PA_REQUIRE(page_size >= 4 && page_size % 4 == 0, "%s: page size %d is not a multiple of 4", what, page_size);
+  PA_REQUIRE(window >= 0, "%s: window %d is negative (0 means none)", what, window);
+  PA_REQUIRE(nseq <= 65535, "%s: %d sequences exceed the grid", what, nseq);
+  return 0;
+}
+
+// 1 if the MFMA kernels take this head_dim and page size, else 0 (the caller then uses the generic kernel).
+extern "C" int pa_attn_mfma_supports(int hd, int page_size) {
+  const bool hd_ok = hd == 16 || hd == 32 || hd == 48 || hd == 64 || hd == 96 || hd == 128;
+  return hd_ok && page_size >= 4 && page_size % 4 == 0;
+}
+
+// Workspace the decode kernel needs, in floats, for `nseq` sequences cut into at most `max_splits` splits.
+extern "C" long pa_attn_decode_workspace(int nseq, int nh, int hd, int max_splits) {
+  return max_splits <= 1 ? 0 : (long)nseq * nh * max_splits * (hd + 2);
+}
+
+extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                              int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                              void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
+                              int window, float scale, int split_keys, int max_splits) {
+  if (nseq == 0) return 0;
+  if (int rc = check_common("attn_decode", nseq, nh, nkv, page_size, table_stride, window)) return rc;
+  PA_REQUIRE(split_keys >= 32 && split_keys % 32 == 0, "attn_decode: split of %d keys is not a multiple of 32", split_keys);
+  PA_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attn_decode: %d splits", max_splits);
+  PA_REQUIRE(max_splits == 1 || workspace, "attn_decode: no workspace for %d splits", max_splits);
+  float* part_o = workspace;
+  float* part_ml = workspace ? workspace + (size_t)nseq * nh * max_splits * hd : nullptr;
+#define PA_CALL(HD)                                                                                                  \
+  return launch_decode<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
+                           out, part_o, part_ml, nseq, nh, nkv, page_size, window, scale, split_keys, max_splits)
+  PA_HD_SWITCH(hd, PA_CALL)
+#undef PA_CALL
+}
+
+extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                               int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                               void* out, int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window,
+                               float scale) {
+  if (nseq == 0) return 0;
+  if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
+  PA_REQUIRE(max_q_len >= 1, "attn_prefill: longest portion %d", max_q_len);
+#define PA_CALL(HD)                                                                                                   \
+  return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
+                            out, nseq, max_q_len, nh, nkv, page_size, window, scale)
+  PA_HD_SWITCH(hd, PA_CALL)
+#undef PA_CALL
+}

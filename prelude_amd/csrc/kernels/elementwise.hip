@@ -64,14 +64,13 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, T* residual, const float
   }
 }
 
-// ---- SiLU(gate) * up over a merged [T, 2I] input -------------------------
+// ---- SiLU(gate) * up over a merged [T, 2I] input whose columns alternate gate_j, up_j ----
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, size_t total) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
-  const size_t t = i / inter, c = i % inter;
-  const float g = to_f32(gate_up[t * 2 * inter + c]);
-  const float u = to_f32(gate_up[t * 2 * inter + inter + c]);
+  const float g = to_f32(gate_up[2 * i]);
+  const float u = to_f32(gate_up[2 * i + 1]);
   out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
 }
 

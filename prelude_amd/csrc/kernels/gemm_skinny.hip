@@ -1,0 +1,208 @@
+// C[M,N] = X[M,K] * W[N,K]^T (+ bias) for few rows (M <= 64) in bfloat16 with
+// 32-bit accumulation: the matrix product of decode steps, where every weight
+// is read once and the time is the time to stream W from HBM.
+//
+// A workgroup owns 16 rows of W (16 outputs per token) and all of K; its
+// wavefronts take the 64-wide k-steps in turn and are summed through LDS in
+// wavefront order.  Both operands go from memory straight into
+// v_mfma_f32_16x16x32_bf16 registers: W^T tile as A (row = output n), X^T as B
+// (column = token m), so a lane ends up with four consecutive n of one token.
+// Within a k-step a lane reads 32 contiguous bytes of its row (k0 + 16g .. +15):
+// the first half feeds one MFMA, the second half the next, and X is read with
+// the same pattern, so the order of k inside the step is the same on both
+// sides; a wavefront's loads cover whole 128-byte lines of 16 rows.
+//
+// What keeps HBM busy is bytes in flight, not the number of compute units at
+// work: a narrow weight (N = 2560 gives 160 tiles for 256 units) gets 16
+// wavefronts per workgroup, a wide one 4, so that some thousands of wavefronts
+// each have two k-steps of loads outstanding.  Nothing is split across
+// workgroups, so there is no workspace, no counter and no fence, and the
+// result of a row depends on the weight's shape alone.
+//
+// Epilogues: plain (bfloat16 or float32 out, optional bias), and SiLU(gate)*up
+// for a weight whose rows alternate gate_j, up_j: a lane's four outputs are two
+// (gate, up) pairs, and [M, N/2] is written with no [M, N] intermediate.
+//
+// Reference counterpart: the GEMM dispatch of crates/prelude-cuda/src/ops/gemm.rs:35-137
+// (library kernels there; 32-bit accumulation as there, :151, :365) and the
+// activation of crates/prelude-cuda/src/kernels/kernels_src/elementwise/silu_mul.cu:26-33.
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+constexpr int kSkinnyMaxM = 64;
+
+struct Frag {
+  bf16x8 lo, hi;
+};
+
+__device__ __forceinline__ Frag load_frag(const bf16* row, int k0, int k, bool ok) {
+  Frag f;
+  const bool lo_ok = ok && k0 + 8 <= k, hi_ok = ok && k0 + 16 <= k;
+  if (lo_ok) {
+    f.lo = *reinterpret_cast<const bf16x8*>(row + k0);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f.lo[i] = (bf16)0.f;
+  }
+  if (hi_ok) {
+    f.hi = *reinterpret_cast<const bf16x8*>(row + k0 + 8);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f.hi[i] = (bf16)0.f;
+  }
+  return f;
+}
+
+enum Epilogue : int { kPlain = 0, kSiluMul = 1 };
+
+template <int MT, int WAVES, typename TC, int EPI>
+__global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* __restrict__ x,
+                                                                   const bf16* __restrict__ w,
+                                                                   const float* __restrict__ bias,
+                                                                   TC* __restrict__ c, int m, int n, int k, long ldx,
+                                                                   long ldc) {
+  __shared__ float red[WAVES][MT][kWave][4];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int n0 = blockIdx.x * 16;
+  const int steps = (k + 63) / 64;
+
+  const bool n_ok = n0 + r < n;
+  const bf16* wrow = w + (size_t)(n_ok ? n0 + r : 0) * k + 16 * g;
+  const bf16* xrow[MT];
+  bool m_ok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    m_ok[t] = 16 * t + r < m;
+    xrow[t] = x + (size_t)(m_ok[t] ? 16 * t + r : 0) * ldx + 16 * g;
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // two k-steps in flight per wavefront: the next step's rows of W and X are asked for before this step's are used
+  const int kk = k - 16 * g;
+  int s = wave;
+  Frag wn = load_frag(wrow, s * 64, kk, n_ok && s < steps);
+  Frag xn[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) xn[t] = load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
+  for (; s < steps; s += WAVES) {
+    const Frag wc = wn;
+    Frag xc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xc[t] = xn[t];
+    const int next = s + WAVES;
+    wn = load_frag(wrow, next * 64, kk, n_ok && next < steps);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xn[t] = load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.lo, xc[t].lo, acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.hi, xc[t].hi, acc[t], 0, 0, 0);
+    }
+  }
+  // the wavefronts' shares, added in wavefront order by wavefront 0
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][t][lane][i] = acc[t][i];
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = red[0][t][lane][i];
+#pragma unroll
+      for (int u = 1; u < WAVES; ++u) v += red[u][t][lane][i];
+      acc[t][i] = v;
+    }
+  // epilogue: lane (g, r) writes four consecutive n of token 16t + r
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int mi = 16 * t + r;
+    if (mi >= m) continue;
+    const int nb = n0 + 4 * g;
+    if (EPI == kSiluMul) {
+      // rows alternate gate_j, up_j: outputs nb/2 and nb/2 + 1
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int nn = nb + 2 * j;
+        if (nn + 1 < n) {
+          const float gate = acc[t][2 * j], up = acc[t][2 * j + 1];
+          c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate / (1.0f + expf(-gate)) * up);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (nb + i < n) {
+          float v = acc[t][i];
+          if (bias) v += bias[nb + i];
+          c[(size_t)mi * ldc + nb + i] = from_f32<TC>(v);
+        }
+      }
+    }
+  }
+}
+
+// Wavefronts per workgroup for an [n, k] weight: aim at about 3000 wavefronts on the chip, each with at
+// least two k-steps.  Depends on the weight's shape only, never on the batch.
+static int skinny_waves(int n, int k) {
+  const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
+  int w = 4;
+  while (w < 16 && tiles * w < 3000 && steps / (2 * w) >= 2) w *= 2;
+  return w;
+}
+
+template <int MT, typename TC, int EPI>
+int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
+                  long ldx, long ldc) {
+  dim3 grid((n + 15) / 16);
+#define PA_W(WV)                                                                                               \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, TC, EPI>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
+                     (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc)
+  switch (skinny_waves(n, k)) {
+    case 16: PA_W(16); break;
+    case 8: PA_W(8); break;
+    default: PA_W(4); break;
+  }
+#undef PA_W
+  return check_launch("gemm_skinny");
+}
+
+template <typename TC, int EPI>
+int launch_skinny_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
+                     long ldx, long ldc) {
+  switch ((m + 15) / 16) {
+    case 1: return launch_skinny<1, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    case 2: return launch_skinny<2, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    case 3: return launch_skinny<3, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    default: return launch_skinny<4, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  }
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+// epilogue 0: C[m, n] (+ bias); 1: C[m, n/2] = silu(gate) * up over a weight whose rows alternate gate_j, up_j.
+extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w,
+                              const float* bias, void* c, int m, int n, int k, long ldx, long ldc) {
+  if (m == 0 || n == 0) return 0;
+  PA_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_skinny: bad sizes m=%d n=%d k=%d", m, n, k);
+  PA_REQUIRE(m <= kSkinnyMaxM, "gemm_skinny: %d rows exceed %d", m, kSkinnyMaxM);
+  PA_REQUIRE(k % 8 == 0 && ldx % 8 == 0, "gemm_skinny: k=%d and the row stride %ld must be multiples of 8", k, ldx);
+  PA_REQUIRE(ldx >= k, "gemm_skinny: row stride %ld is smaller than k=%d", ldx, k);
+  PA_REQUIRE(epilogue == kPlain || (n % 2 == 0 && !bias), "gemm_skinny: the SiLU*up epilogue needs an even n and no bias");
+  PA_REQUIRE(ldc >= (epilogue == kSiluMul ? n / 2 : n), "gemm_skinny: output row stride %ld is too small", ldc);
+  hipStream_t st = (hipStream_t)stream;
+  if (epilogue == kPlain && out_dtype == kBF16) return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  if (epilogue == kPlain && out_dtype == kF32) return launch_skinny_mt<float, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  if (epilogue == kSiluMul && out_dtype == kBF16)
+    return launch_skinny_mt<bf16, kSiluMul>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  return pa::fail("gemm_skinny: unsupported output type %d with epilogue %d", out_dtype, epilogue);
+}

@@ -8,7 +8,10 @@
 // cache; V is copied).  Differences that are ours: the norm weights and the
 // cos/sin tables are 32-bit in every mode, the rotary width may be smaller
 // than the head (the rest passes through after the norm), the norm may be
-// absent, and the cache is laid out [page, kv_head, offset, head_dim].
+// absent, and the caches are laid out K [page, kv_head, offset, head_dim] and
+// V [page, kv_head, head_dim, offset]: V transposed, so that the attention
+// kernels can feed both straight from memory into the matrix cores (keys are
+// the contraction index of P.V, and an MFMA operand wants it contiguous).
 #include "common.h"
 #include "api.h"
 
@@ -36,6 +39,7 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
 
   // Where this head goes.
   T* dst = nullptr;
+  long dst_stride = 1;  // distance between consecutive head_dim elements at the destination
   const float* weight = nullptr;
   bool rotate = false;
   if (active) {
@@ -49,8 +53,12 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
         const long long page = slot / page_size, off = slot % page_size;
         const bool is_k = h < nh + nkv;
         const int kvh = is_k ? h - nh : h - nh - nkv;
-        T* base = is_k ? k_cache : v_cache;
-        dst = base + (((size_t)page * nkv + kvh) * page_size + off) * hd;
+        if (is_k) {
+          dst = k_cache + (((size_t)page * nkv + kvh) * page_size + off) * hd;
+        } else {
+          dst = v_cache + ((size_t)page * nkv + kvh) * hd * page_size + off;
+          dst_stride = page_size;
+        }
         weight = is_k ? k_weight : nullptr;
         rotate = is_k;
       }
@@ -71,7 +79,7 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
 #pragma unroll
       for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
         const int i = lane + e * kWave;
-        if (i < hd) dst[i] = src[i];
+        if (i < hd) dst[(size_t)i * dst_stride] = src[i];
       }
     }
   }

@@ -40,6 +40,13 @@ class StepBatch:
     fresh_host: List[int] = dataclasses.field(default_factory=list)
     max_q_len: int = 0
     max_context_len: int = 0
+    # the step's sequences by kind, for kernels that treat single tokens and portions differently
+    decode_seqs: Optional[torch.Tensor] = None    # int32 [n_decode] indices of sequences feeding one token
+    prefill_seqs: Optional[torch.Tensor] = None   # int32 [n_prefill] indices of sequences feeding more
+    n_decode: int = 0
+    n_prefill: int = 0
+    max_prefill_q: int = 0       # longest portion among prefill_seqs
+    max_decode_context: int = 0  # longest context among decode_seqs
     page_size: int = 0
     graph: Optional[object] = None  # set while a step is being captured or replayed from fixed buffers
 

@@ -89,6 +89,12 @@ class Engine:
                                        state_slots, self.dtype, self.device)
         self._staging = _Staging()
         self._live: Dict[int, int] = {}   # request id -> tokens fed so far
+        # decode steps as HIP graphs: only for models whose layers keep nothing but pages (a mixer with
+        # state of its own may run host code per step), and only in the serving type
+        self._graphs = None
+        if config.hip_graph and not model.needs_state and self.dtype == torch.bfloat16:
+            from .graph import DecodeGraphs
+            self._graphs = DecodeGraphs(self, config.hip_graph_max_bs)
 
     # ---- construction -------------------------------------------------------
     @classmethod
@@ -168,6 +174,8 @@ class Engine:
             raise
         for e, s in zip(entries, starts):
             self.tables.commit(e.id, s + len(e.tokens))
+        if self._graphs is not None and self._graphs.owns(logits):
+            logits = logits.clone()   # the graph's own output tensor is overwritten by the next replay
         return logits
 
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -194,13 +202,22 @@ class Engine:
                 raise StepError(f"request {e.id}: {have} + {n} tokens exceed max_position_embeddings "
                                 f"{self.max_positions}")
 
-    def build_batch(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> StepBatch:
-        """Index arrays of the step, built on the host in one pinned buffer and sent in one copy."""
+    def build_batch(self, entries: Sequence[StepEntry], starts: Sequence[int], stride: Optional[int] = None,
+                    device_buffer: Optional[torch.Tensor] = None) -> StepBatch:
+        """Index arrays of the step, built on the host in one pinned buffer and sent in one copy.
+
+        ``stride`` widens the block tables beyond what the step needs and
+        ``device_buffer`` receives the arrays instead of a fresh tensor: a
+        captured graph reads its inputs from fixed addresses with a fixed layout.
+        """
         n = len(entries)
         counts = [len(e.tokens) for e in entries]
         total = sum(counts)
         ends = [s + c for s, c in zip(starts, counts)]
-        stride = max(1, -(-max(ends) // self.page_size))
+        need = max(1, -(-max(ends) // self.page_size))
+        stride = need if stride is None else stride
+        if stride < need:
+            raise StepError(f"block table stride {stride} is smaller than the {need} pages the step needs")
         wanted = sum(len(e.want) for e in entries)
         layout = self.tables.step_layout(n, total, stride, wanted)
         size = layout["_total"][1]
@@ -217,11 +234,22 @@ class Engine:
                 w += 1
             t += c
         self.tables.fill_step([e.id for e in entries], starts, counts, stride, host, layout)
+        dec = [i for i, c in enumerate(counts) if c == 1]
+        pre = [i for i, c in enumerate(counts) if c > 1]
+        doff, _ = layout["decode_seqs"]
+        poff, _ = layout["prefill_seqs"]
+        host[doff: doff + len(dec)] = dec
+        host[poff: poff + len(pre)] = pre
         soff, _ = layout["state_slots"]
         foff, _ = layout["fresh"]
         state_host = host[soff: soff + n].tolist()
         fresh_host = host[foff: foff + n].tolist()
-        dev = torch.empty(size, dtype=torch.int32, device=self.device)
+        if device_buffer is None:
+            dev = torch.empty(size, dtype=torch.int32, device=self.device)
+        else:
+            if device_buffer.numel() != size:
+                raise StepError(f"the fixed index buffer holds {device_buffer.numel()} words, the step needs {size}")
+            dev = device_buffer
         dev.copy_(pinned[:size], non_blocking=True)
         self._staging.sent(slot)
 
@@ -233,14 +261,27 @@ class Engine:
         bt = view("block_tables").view(G, n, stride) if G else None
         sl = view("slots").view(G, total) if G else None
         kv = [GroupStep(bt[g], sl[g]) for g in range(G)]
+        fixed = device_buffer is not None
         return StepBatch(num_tokens=total, num_seqs=n, token_ids=view("token_ids"), positions=view("positions"),
                          seq_of_token=view("seq_of_token"), cu_q=view("cu_q"), context_lens=view("context_lens"),
                          state_slots=view("state_slots"), fresh=view("fresh"), want_rows=view("want_rows"), kv=kv,
                          q_lens=counts, starts=list(starts), state_slots_host=state_host, fresh_host=fresh_host,
-                         max_q_len=max(counts), max_context_len=max(ends), page_size=self.page_size)
+                         max_q_len=max(counts), max_context_len=stride * self.page_size if fixed else max(ends),
+                         page_size=self.page_size,
+                         decode_seqs=view("decode_seqs")[:len(dec)], prefill_seqs=view("prefill_seqs")[:len(pre)],
+                         n_decode=len(dec), n_prefill=len(pre), max_prefill_q=max([counts[i] for i in pre], default=0),
+                         # with fixed buffers the launch shapes must not follow the data: bound by what the tables can hold
+                         max_decode_context=(stride * self.page_size if fixed else max([ends[i] for i in dec], default=0)))
 
     def run(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> torch.Tensor:
-        """Runs a step whose pages are already reserved (the scheduler's path)."""
+        """Runs a step whose pages are already reserved (the scheduler's path).
+
+        A step of single tokens whose logits are all wanted is replayed from a
+        captured HIP graph when graphs are on; the logits tensor it returns is
+        then the graph's own and is overwritten by the next such step.
+        """
+        if self._graphs is not None and self._graphs.eligible(entries):
+            return self._graphs.run(entries, starts)
         batch = self.build_batch(entries, starts)
         if self.model.needs_state:
             fresh = [s for s, f in zip(batch.state_slots_host, batch.fresh_host) if f and s >= 0]

@@ -90,7 +90,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optiona
 
 
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(gate) * up for gate_up [T, 2I] (gate columns first) -> [T, I]."""
+    """silu(gate) * up for gate_up [T, 2I] whose columns alternate gate_j, up_j -> [T, I]."""
     _dev(gate_up)
     if gate_up.dim() != 2 or gate_up.shape[1] % 2:
         raise NativeError(f"silu_mul: input {tuple(gate_up.shape)} is not [T, 2I]")
@@ -128,6 +128,17 @@ def to_f32(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def _check_caches(k_cache, v_cache, num_kv_heads, head_dim, dtype, what) -> None:
+    """K [pages, nkv, page, hd] and V [pages, nkv, hd, page] of the same pool."""
+    ok = (k_cache is not None and v_cache is not None and k_cache.dim() == 4 and v_cache.dim() == 4
+          and k_cache.shape[0] == v_cache.shape[0] and k_cache.shape[1] == v_cache.shape[1] == num_kv_heads
+          and k_cache.shape[3] == v_cache.shape[2] == head_dim and k_cache.shape[2] == v_cache.shape[3]
+          and k_cache.dtype == dtype and v_cache.dtype == dtype)
+    if not ok:
+        raise NativeError(f"{what}: caches must be K [pages, {num_kv_heads}, page, {head_dim}] and "
+                          f"V [pages, {num_kv_heads}, {head_dim}, page] of {dtype}")
+
+
 def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
                    cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                    slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
@@ -136,7 +147,7 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
 
     qkv [T, (nh + 2 nkv) * hd]; returns q [T, nh, hd].  With ``slots`` None
     nothing is written to the cache (then ``num_kv_heads`` may be 0 for a
-    Q-only input).  Caches are [pages, nkv, page_size, hd].
+    Q-only input).  K cache [pages, nkv, page_size, hd], V cache [pages, nkv, hd, page_size].
     """
     _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache)
     _i32(positions, "positions")
@@ -161,10 +172,7 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
         _i32(slots, "slots")
         if slots.shape != (t,):
             raise NativeError(f"qknorm_rope_kv: slots {tuple(slots.shape)} for {t} tokens")
-        if k_cache is None or v_cache is None or k_cache.shape != v_cache.shape or k_cache.dim() != 4 \
-                or k_cache.shape[1] != num_kv_heads or k_cache.shape[3] != head_dim \
-                or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
-            raise NativeError(f"qknorm_rope_kv: caches must be [pages, {num_kv_heads}, page, {head_dim}] of {qkv.dtype}")
+        _check_caches(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, "qknorm_rope_kv")
         page_size = k_cache.shape[2]
     q_out = torch.empty((t, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     check(kernels().pa_qknorm_rope_kv(_stream(), _code(qkv), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos),
@@ -192,15 +200,43 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
     return out
 
 
+SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel itself takes up to 64)
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False) -> torch.Tensor:
+    """x [M <= 64, K] @ w[N, K]^T in bfloat16 on the matrix cores, streaming w once.
+
+    With ``silu_mul_epilogue`` the rows of w alternate gate_j, up_j and the
+    result is silu(gate) * up, [M, N/2]."""
+    _dev(x, w, bias)
+    _f32(bias, "bias")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise NativeError(f"gemm_skinny: x {tuple(x.shape)} {x.dtype} / w {tuple(w.shape)} {w.dtype}")
+    m, k = x.shape
+    n = w.shape[0]
+    out_dtype = out_dtype or torch.bfloat16
+    if bias is not None and bias.shape != (n,):
+        raise NativeError(f"gemm_skinny: bias {tuple(bias.shape)} is not [{n}]")
+    cols = n // 2 if silu_mul_epilogue else n
+    out = torch.empty((m, cols), dtype=out_dtype, device=x.device)
+    check(kernels().pa_gemm_skinny(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w),
+                                   _ptr(bias), _ptr(out), m, n, k, k, cols))
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T (+ b), W [out, in].  float32: our own true 32-bit product.
-    bfloat16: the library product with 32-bit accumulation."""
+    bfloat16: up to 64 rows our weight-streaming kernel, above that the library
+    product; 32-bit accumulation in both."""
     if x.dtype == torch.float32:
         return gemm_plain(x, w, bias, out_dtype)
     _dev(x, w, bias)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise NativeError(f"linear: x {x.dtype} / w {w.dtype}")
+    if x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0:
+        return gemm_skinny(x, w, bias, out_dtype)
     y = torch.matmul(x, w.t())
     if bias is not None:
         add_bias_(y, bias)
@@ -209,21 +245,35 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
     return y
 
 
+def set_skinny_max_rows(n: int) -> None:
+    """Up to how many rows ``linear`` uses the weight-streaming kernel (for measurements)."""
+    global SKINNY_MAX_ROWS
+    SKINNY_MAX_ROWS = max(0, min(int(n), 64))
+
+
+def linear_silu_mul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) for a weight [2I, K] whose rows alternate gate_j, up_j."""
+    if x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0:
+        return gemm_skinny(x, w, silu_mul_epilogue=True)
+    return silu_mul(linear(x, w))
+
+
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       seq_of_token: torch.Tensor, positions: torch.Tensor, window: int, scale: float) -> torch.Tensor:
     """Paged causal attention, any mix of portions and decode tokens.
 
-    q [T, nh, hd]; caches [pages, nkv, page, hd]; block_table int32 [B, stride];
+    q [T, nh, hd]; K cache [pages, nkv, page, hd], V cache [pages, nkv, hd, page]; block_table int32 [B, stride];
     seq_of_token / positions int32 [T].  window 0 = all keys.
     """
     _dev(q, k_cache, v_cache, block_table, seq_of_token, positions)
     _i32(block_table, "block_table")
     _i32(seq_of_token, "seq_of_token")
     _i32(positions, "positions")
-    if q.dim() != 3 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[3] != q.shape[2] \
-            or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
-        raise NativeError(f"attention: q {tuple(q.shape)} {q.dtype} / cache {tuple(k_cache.shape)} {k_cache.dtype}")
+    if q.dim() != 3:
+        raise NativeError(f"attention: q {tuple(q.shape)} is not [T, heads, head_dim]")
     t, nh, hd = q.shape
+    _check_caches(k_cache, v_cache, k_cache.shape[1] if k_cache is not None and k_cache.dim() == 4 else -1, hd, q.dtype,
+                  "attention")
     if seq_of_token.shape != (t,) or positions.shape != (t,) or block_table.dim() != 2:
         raise NativeError("attention: index arrays do not match the number of tokens")
     out = torch.empty_like(q)
@@ -244,12 +294,66 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+DECODE_SPLIT_KEYS = 256   # keys per split of the decode kernel: fixed, so a token's result never depends on its batch
+
+
+def mfma_attention_supported(head_dim: int, page_size: int) -> bool:
+    return bool(kernels().pa_attn_mfma_supports(int(head_dim), int(page_size)))
+
+
+def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_context: int,
+                     window: int, scale: float) -> None:
+    """Matrix-core attention for the sequences ``seq_ids`` (each feeding one token); writes their rows of ``out``."""
+    _dev(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out)
+    t, nh, hd = q.shape
+    _check_caches(k_cache, v_cache, k_cache.shape[1], hd, torch.bfloat16, "attention_decode")
+    n = seq_ids.shape[0]
+    if n == 0:
+        return
+    span = min(max_context, window + DECODE_SPLIT_KEYS) if window else max_context
+    max_splits = max(1, -(-span // DECODE_SPLIT_KEYS) + (1 if window else 0))
+    words = kernels().pa_attn_decode_workspace(n, nh, hd, max_splits)
+    ws = torch.empty((max(words, 1),), dtype=torch.float32, device=q.device)
+    check(kernels().pa_attn_decode(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+                                   block_table.shape[1], _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out),
+                                   _ptr(ws), n, nh, k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale),
+                                   DECODE_SPLIT_KEYS, max_splits))
+
+
+def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_q_len: int,
+                      window: int, scale: float) -> None:
+    """Matrix-core attention for the sequences ``seq_ids`` (portions of several tokens); writes their rows of ``out``."""
+    _dev(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out)
+    t, nh, hd = q.shape
+    _check_caches(k_cache, v_cache, k_cache.shape[1], hd, torch.bfloat16, "attention_prefill")
+    n = seq_ids.shape[0]
+    if n == 0:
+        return
+    check(kernels().pa_attn_prefill(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+                                    block_table.shape[1], _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out), n,
+                                    int(max_q_len), nh, k_cache.shape[1], hd, k_cache.shape[2], int(window),
+                                    float(scale)))
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int,
               scale: float) -> torch.Tensor:
     """Attention of one step over one cache group; picks the kernel for the sizes at hand.
 
     ``group`` is the step's ``GroupStep`` of the cache group, ``step`` the ``StepBatch``.
+    bfloat16 with a head_dim and page size the matrix-core kernels take: single
+    tokens go to the split decode kernel, portions to the prefill kernel.
+    Everything else (float32, other sizes) goes to the generic kernel.
     """
+    if q.dtype == torch.bfloat16 and step.decode_seqs is not None \
+            and mfma_attention_supported(q.shape[2], k_cache.shape[2]):
+        out = torch.empty_like(q)
+        if step.n_decode:
+            attention_decode(q, k_cache, v_cache, group.block_table, step.decode_seqs, step.cu_q, step.context_lens,
+                             out, step.max_decode_context, window, scale)
+        if step.n_prefill:
+            attention_prefill(q, k_cache, v_cache, group.block_table, step.prefill_seqs, step.cu_q, step.context_lens,
+                              out, step.max_prefill_q, window, scale)
+        return out
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
 
 

@@ -2,8 +2,9 @@
 
 crates/prelude-core/src/models/qwen3.rs:383-448; silu(x) = x / (1 + e^-x) in
 32-bit (crates/prelude-cuda/src/kernels/kernels_src/elementwise/silu_mul.cu:26-33).
-Gate and up are one matrix [2I, H] here, gate rows first, so one product feeds
-the activation kernel.
+Gate and up are one matrix [2I, H] here with rows alternating gate_j, up_j:
+one product yields each (gate_j, up_j) pair side by side, so the activation
+is the epilogue of that product for few rows and a pairwise kernel otherwise.
 """
 from __future__ import annotations
 
@@ -28,8 +29,9 @@ class GatedMLP(FeedForward):
                 "down_proj.weight": TensorReq((h, i), MATRIX)}
 
     def load(self, tensors, dtype, device):
-        self.gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
+        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        self.gate_up = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
         self.down = tensors["down_proj.weight"]
 
     def forward(self, x):
-        return K.linear(K.silu_mul(K.linear(x, self.gate_up)), self.down)
+        return K.linear(K.linear_silu_mul(x, self.gate_up), self.down)

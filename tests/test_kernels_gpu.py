@@ -86,14 +86,14 @@ def test_rmsnorm_reference_vector(gpu):
 @pytest.mark.parametrize("tokens,inter", [(3, 9728), (5, 160), (2, 7)])
 def test_silu_mul(gpu, dtype, tokens, inter):
     gu = rnd(tokens, 2 * inter, dtype=dtype, scale=3.0)
-    ref = pm.silu(gu[:, :inter].double()) * gu[:, inter:].double()
+    ref = pm.silu(gu[:, 0::2].double()) * gu[:, 1::2].double()
     close(K().silu_mul(gu.to(gpu)), ref, dtype)
 
 
 def test_silu_mul_reference_vector(gpu):
     g = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5])
     u = torch.tensor([1.0, 2.0, 3.0, 0.5, 1.0, 4.0])
-    out = K().silu_mul(torch.cat([g, u]).reshape(1, 12).to(gpu)).cpu()[0]
+    out = K().silu_mul(torch.stack([g, u], dim=1).reshape(1, 12).to(gpu)).cpu()[0]
     assert torch.allclose(out, torch.nn.functional.silu(g) * u, atol=1e-6) and float(out[0]) == 0.0
 
 
@@ -119,6 +119,37 @@ def test_linear_bf16(gpu, m, n, k):
     assert out32.dtype == torch.float32
     close(out32, ref, torch.bfloat16)
     close(K().gemm_plain(x.to(gpu), w.to(gpu), out_dtype=torch.float32), ref, torch.float32, f32=1e-5)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 2560, 4096), (8, 6144, 2560), (8, 2560, 9728), (13, 509, 96), (16, 331, 80),
+                                   (17, 64, 64), (33, 192, 160), (64, 2560, 2560), (5, 19456, 2560), (2, 40, 8),
+                                   (3, 151936, 256)])
+def test_gemm_skinny(gpu, m, n, k):
+    x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
+    ref = x.double() @ w.double().T
+    xd, wd = x.to(gpu), w.to(gpu)
+    close(K().gemm_skinny(xd, wd, out_dtype=torch.float32), ref, torch.float32, f32=2e-5)
+    close(K().gemm_skinny(xd, wd), ref, torch.bfloat16)
+    close(K().gemm_skinny(xd, wd, b.to(gpu), out_dtype=torch.float32), ref + b.double(), torch.float32, f32=2e-5)
+    # a row's result does not depend on how many rows there are (same weight, same split of K)
+    full = K().gemm_skinny(xd, wd, out_dtype=torch.float32)
+    one = K().gemm_skinny(xd[m - 1:].contiguous(), wd, out_dtype=torch.float32)
+    assert torch.equal(one[0], full[m - 1])
+    if n % 2 == 0:
+        act = K().gemm_skinny(xd, wd, silu_mul_epilogue=True)
+        close(act, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
+        close(K().linear_silu_mul(xd, wd), pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
+
+
+def test_gemm_skinny_refuses(gpu):
+    from prelude_amd._native import NativeError
+    with pytest.raises(NativeError, match="exceed"):
+        K().gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=gpu), torch.zeros(16, 64, dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(NativeError, match="multiples of 8"):
+        K().gemm_skinny(torch.zeros(2, 12, dtype=torch.bfloat16, device=gpu), torch.zeros(16, 12, dtype=torch.bfloat16, device=gpu))
+    # what it refuses, linear() sends elsewhere
+    out = K().linear(torch.ones(2, 12, dtype=torch.bfloat16, device=gpu), torch.ones(16, 12, dtype=torch.bfloat16, device=gpu))
+    assert float(out.float().min()) == 12.0
 
 
 # ---- QK norm + RoPE + cache write ---------------------------------------------------------------
@@ -153,7 +184,7 @@ def test_qknorm_rope_kv(gpu, dtype, nh, nkv, hd, rot, norm):
     slot_list = [35, 3, 0, 7, 8, 12, -1, 20, 21, 22, 30]                  # one token is not cached
     slots = torch.tensor(slot_list, dtype=torch.int32)
     kc = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype)
-    vc = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype)
+    vc = torch.full((pages, nkv, hd, page), 7.0, dtype=dtype)
     dev = lambda x: None if x is None else x.to(gpu)
     kcd, vcd = kc.to(gpu), vc.to(gpu)
     q = K().qknorm_rope_kv(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), dev(pos), dev(slots), kcd, vcd, nh, nkv, hd,
@@ -166,8 +197,9 @@ def test_qknorm_rope_kv(gpu, dtype, nh, nkv, hd, rot, norm):
             continue
         touched[s // page, s % page] = True
         close(kcd[s // page, :, s % page], rk[i], dtype)
-        assert torch.equal(vcd[s // page, :, s % page].cpu().double(), rv[i].to(dtype).double())   # V is a copy
+        assert torch.equal(vcd[s // page, :, :, s % page].cpu().double(), rv[i].to(dtype).double())   # V is a copy
     assert bool((kcd.cpu()[~touched[:, None, :].expand(pages, nkv, page)] == 7.0).all())             # nothing else written
+    assert bool((vcd.cpu().transpose(2, 3)[~touched[:, None, :].expand(pages, nkv, page)] == 7.0).all())
     # queries only (a layer that reads another layer's cache)
     qonly = qkv[:, : nh * hd].contiguous()
     q2 = K().qknorm_rope_kv(dev(qonly), dev(qw), None, dev(cos), dev(sin), dev(pos), None, None, None, nh, 0, hd, rot, eps)
@@ -183,14 +215,14 @@ def test_qknorm_rope_refuses_bad_sizes(gpu):
 
 
 # ---- attention over the paged cache --------------------------------------------------------------
-def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None):
+def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None, kernel="generic"):
     """seqs: list of (context_len, q_len): the last q_len tokens of each context are this step's queries.
     Pages are handed out in a scrambled order.  Returns (engine output, plain output)."""
     g = torch.Generator().manual_seed(seed)
     total_pages = sum(-(-c // page) for c, _ in seqs) + 3
     perm = torch.randperm(total_pages, generator=torch.Generator().manual_seed(seed + 77)).tolist()
     kc = torch.zeros(total_pages, nkv, page, hd)
-    vc = torch.zeros(total_pages, nkv, page, hd)
+    vc = torch.zeros(total_pages, nkv, hd, page)
     stride = max(-(-c // page) for c, _ in seqs)
     table = torch.full((len(seqs), stride), -1, dtype=torch.int32)
     qs, seq_of, pos, refs = [], [], [], []
@@ -206,7 +238,7 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
             table[i, p] = phys
             n = min(page, ctx - p * page)
             kc[phys, :, :n] = k[p * page: p * page + n].transpose(0, 1)
-            vc[phys, :, :n] = v[p * page: p * page + n].transpose(0, 1)
+            vc[phys, :, :, :n] = v[p * page: p * page + n].permute(1, 2, 0)
         if window:   # pages wholly before the first visible key may be gone
             first = max(0, (ctx - ql) - window + 1)
             for p in range(first // page):
@@ -219,6 +251,21 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
         refs.append(pm.attention(q.double(), k.double(), v.double(), 1.0 / math.sqrt(hd), window=window or None,
                                  q_offset=ctx - ql))
     q = torch.cat(qs).to(dtype)
+    if kernel == "mfma":
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+        cu = [0]
+        for _, ql in seqs:
+            cu.append(cu[-1] + ql)
+        dec = [i for i, (_, ql) in enumerate(seqs) if ql == 1]
+        pre = [i for i, (_, ql) in enumerate(seqs) if ql > 1]
+        qd, kd, vd, td = q.to(gpu), kc.to(dtype).to(gpu), vc.to(dtype).to(gpu), table.to(gpu)
+        out = torch.full_like(qd, float("nan"))
+        ctxs = i32([c for c, _ in seqs])
+        K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, out, max([seqs[i][0] for i in dec], default=0),
+                             window, 1.0 / math.sqrt(hd))
+        K().attention_prefill(qd, kd, vd, td, i32(pre), i32(cu), ctxs, out, max([seqs[i][1] for i in pre], default=0),
+                              window, 1.0 / math.sqrt(hd))
+        return out, torch.cat(refs)
     out = K().attention_generic(q.to(gpu), kc.to(dtype).to(gpu), vc.to(dtype).to(gpu), table.to(gpu),
                                 torch.tensor(seq_of, dtype=torch.int32, device=gpu),
                                 torch.tensor(pos, dtype=torch.int32, device=gpu), window, 1.0 / math.sqrt(hd))
@@ -267,6 +314,67 @@ def test_attention_far_key_and_window_edge(gpu):
         out, ref = paged_case(gpu, torch.float32, 2, 1, hd, 16, [(100, 1)], 20, scale_trick=trick2)
         close(out, ref, torch.float32, f32=3e-6)
         assert (float(out.abs().max()) > 50.0) == seen
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 16, 8), (6, 1, 32, 16), (32, 8, 128, 16), (6, 2, 48, 4), (8, 8, 64, 64),
+                                            (24, 1, 96, 32), (16, 2, 128, 128), (3, 3, 64, 16)])
+def test_mfma_attention_mixed_batch(gpu, nh, nkv, hd, page):
+    seqs = [(70, 70), (130, 1), (33, 7), (1, 1), (64, 2), (700, 1), (257, 1), (300, 150), (16, 16), (513, 1)]
+    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, 0, kernel="mfma")
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.bfloat16)
+
+
+@pytest.mark.parametrize("window,page", [(24, 8), (4, 4), (64, 16), (65, 16), (300, 16), (256, 32)])
+def test_mfma_attention_window(gpu, window, page):
+    seqs = [(100, 100), (200, 1), (90, 30), (window, 1), (window + 1, 1), (700, 1), (600, 300), (512, 1), (513, 1)]
+    out, ref = paged_case(gpu, torch.bfloat16, 6, 2, 48, page, seqs, window, kernel="mfma")
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.bfloat16)
+
+
+def test_mfma_attention_far_key_and_edges(gpu):
+    hd = 64
+
+    def trick(i, q, k, v):
+        q[:] = 0
+        q[:, :, 0] = 12.0
+        k[:, :, 0] = 0
+        k[3, :, 0] = 12.0 * math.sqrt(hd)
+        v[3] = 50.0
+
+    out, ref = paged_case(gpu, torch.bfloat16, 4, 1, hd, 16, [(1000, 1), (600, 600)], 0, scale_trick=trick, kernel="mfma")
+    close(out, ref, torch.bfloat16)
+    assert float(out[0].float().abs().min()) > 40.0            # the far key is found from position 999
+    for hot, seen in ((80, True), (79, False)):
+        def trick2(i, q, k, v, hot=hot):
+            q[:] = 0
+            q[:, :, 0] = 12.0
+            k[:, :, 0] = 0
+            k[hot, :, 0] = 12.0 * math.sqrt(hd)
+            v[hot] = 100.0
+        for seqs in ([(100, 1)], [(100, 20)]):
+            out, ref = paged_case(gpu, torch.bfloat16, 2, 1, hd, 16, seqs, 20, scale_trick=trick2, kernel="mfma")
+            close(out, ref, torch.bfloat16)
+            assert (float(out[-1].float().abs().max()) > 50.0) == seen
+
+
+def test_mfma_attention_batch_and_page_independence(gpu):
+    one, _ = paged_case(gpu, torch.bfloat16, 8, 2, 128, 16, [(900, 1)], 0, seed=5, kernel="mfma")
+    many, _ = paged_case(gpu, torch.bfloat16, 8, 2, 128, 16, [(900, 1), (40, 1), (300, 30)], 0, seed=5, kernel="mfma")
+    assert torch.equal(one[0], many[0])                          # same sequence, other company
+    other, _ = paged_case(gpu, torch.bfloat16, 8, 2, 128, 64, [(900, 1)], 0, seed=5, kernel="mfma")
+    assert torch.equal(one, other)                               # other page size, other pages
+
+
+def test_mfma_attention_refuses_what_it_does_not_take(gpu):
+    from prelude_amd._native import NativeError
+    assert K().mfma_attention_supported(128, 16) and K().mfma_attention_supported(48, 8)
+    assert not K().mfma_attention_supported(80, 16) and not K().mfma_attention_supported(128, 1)
+    with pytest.raises(NativeError, match="head_dim"):
+        paged_case(gpu, torch.bfloat16, 2, 1, 80, 16, [(20, 1)], 0, kernel="mfma")
+    with pytest.raises(NativeError, match="page size"):
+        paged_case(gpu, torch.bfloat16, 2, 1, 64, 2, [(20, 1)], 0, kernel="mfma")
 
 
 def test_attention_is_independent_of_pages_and_batch(gpu):

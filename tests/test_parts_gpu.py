@@ -133,7 +133,7 @@ def test_attention_part(gpu, dtype, nh, nkv, hd, bias, window, qk_norm):
     tol = (3e-6 if dtype == torch.float32 else 3e-2) * max(1.0, float(ref.abs().max()))
     pages = [5, 2, 7, 0, 3]
     mk = lambda: KVLayerCache(torch.zeros(8, nkv, page, hd, dtype=dtype, device=gpu),
-                              torch.zeros(8, nkv, page, hd, dtype=dtype, device=gpu), 0)
+                              torch.zeros(8, nkv, hd, page, dtype=dtype, device=gpu), 0)
     cache = mk()
     out = a.forward(x.to(gpu), one_sequence_step(gpu, n, page, pages), cache)
     assert float((out.double().cpu() - ref).abs().max()) < tol

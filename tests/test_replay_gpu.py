@@ -213,3 +213,44 @@ def test_trace_run_program(gpu, dtype, tmp_path):
     check(load(2), torch.stack([ref[52], ref2[30]]), dtype, "step 2")
     check(load(5), ref2[[39]], dtype, "step 5")
     assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "2.f32", "5.f32"]
+
+
+def test_graph_replays_equal_eager_steps(gpu):
+    """Decode steps replayed from HIP graphs, with eager work (prompt portions, other batch sizes) between the
+    replays: every replay gives the logits of the eager step, bit for bit."""
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    folder, cfg, _ = model_folder("b")
+    seqs = [reference_logits("b", 20 + i, n)[0] for i, n in enumerate([150, 40, 90])]
+
+    def play(hip_graph):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=1024,
+                                                         hip_graph=hip_graph))
+        outs = []
+        at = [0, 0, 0]
+
+        def feed(parts):
+            entries = []
+            for r, n in parts:
+                entries.append(StepEntry(r, seqs[r][at[r]:at[r] + n], [n - 1]))
+                at[r] += n
+            outs.append(eng.step(entries).cpu())
+        feed([(0, 60)])
+        for _ in range(5):
+            feed([(0, 1)])                       # batch of one: first capture, then replays
+        feed([(1, 20), (0, 1)])                  # eager, mixed
+        for _ in range(4):
+            feed([(0, 1), (1, 1)])               # batch of two
+        feed([(2, 70)])
+        for _ in range(6):
+            feed([(0, 1), (1, 1), (2, 1)])
+        for _ in range(3):
+            feed([(0, 1)])                       # the first graph again, after the others
+        feed([(2, 1), (0, 1)])                   # other order of requests, same graph as batch of two
+        return eng, outs
+
+    eager_eng, eager = play(False)
+    graph_eng, graphed = play(True)
+    assert eager_eng._graphs is None and graph_eng._graphs.captures == 3 and graph_eng._graphs.replays == 19
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
