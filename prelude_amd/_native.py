@@ -51,7 +51,8 @@ _KERNEL_API = {
     "pa_attn_decode_workspace": (c_long, [I, I, I, I]),
     "pa_attn_decode": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I]),
     "pa_attn_prefill": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, F]),
-    "pa_argmax": (I, [P, P, P, I, I]),
+    "pa_argmax_scratch": (I, [I, I]),
+    "pa_argmax": (I, [P, P, P, P, I, I]),
     "pa_sample": (I, [P, P, P, P, P, P, P, I, I]),
 }
 

@@ -61,7 +61,9 @@ int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc,
                     int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window, float scale);
 
 // out[r] = index of the largest of logits[r, :], the lowest index among equals.
-int pa_argmax(void* stream, const float* logits, int* out, int rows, int vocab);
+// scratch: pa_argmax_scratch(rows, vocab) floats (none for narrow rows).
+int pa_argmax_scratch(int rows, int vocab);
+int pa_argmax(void* stream, const float* logits, int* out, float* scratch, int rows, int vocab);
 
 // Per row: temperature < 1e-7 -> argmax; else a draw from softmax(logits / T) kept to the top_k largest
 // (0 = all) and to the shortest descending prefix of mass top_p (>= 1 = all), at the uniform number uniform[r] in [0, 1).

@@ -270,12 +270,17 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   }
 }
 
-// Merges the splits of one (sequence, head): grid (nh, sequences).
+// Merges the splits of one (sequence, head): grid (nh, sequences), one wavefront.  Lanes first take a split
+// each (maximum and weights), then a head_dim column each; the sums run over the splits in order.
 template <int HD>
-__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         const int* __restrict__ seq_ids, const int* __restrict__ cu_q,
-                                         const int* __restrict__ context_lens, bf16* __restrict__ out, int nh,
-                                         int window, int split_keys, int max_splits) {
+__global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* __restrict__ part_o,
+                                                                  const float* __restrict__ part_ml,
+                                                                  const int* __restrict__ seq_ids,
+                                                                  const int* __restrict__ cu_q,
+                                                                  const int* __restrict__ context_lens,
+                                                                  bf16* __restrict__ out, int nh, int window,
+                                                                  int split_keys, int max_splits) {
+  __shared__ float weight[1024];
   const int h = blockIdx.x;
   const int seq = seq_ids[blockIdx.y];
   const int ctx = context_lens[seq];
@@ -283,16 +288,33 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int nsplit = (ctx + split_keys - 1) / split_keys - lo / split_keys;
   if (nsplit == 1) return;  // written by the first kernel
+  const int lane = threadIdx.x;
   const size_t base = ((size_t)blockIdx.y * nh + h) * max_splits;
   float mm = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  for (int s = lane; s < nsplit; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  mm = wave_max(mm);
   float l = 0.f;
-  for (int s = 0; s < nsplit; ++s) l += part_ml[(base + s) * 2 + 1] * exp2f(part_ml[(base + s) * 2] - mm);
+  for (int s0 = 0; s0 < nsplit; s0 += kWave) {   // in order of the splits
+    const int s = s0 + lane;
+    float f = 0.f, ls = 0.f;
+    if (s < nsplit) {
+      f = exp2f(part_ml[(base + s) * 2] - mm);
+      ls = part_ml[(base + s) * 2 + 1] * f;
+      if (s < 1024) weight[s] = f;
+    }
+    l += wave_sum(ls);
+  }
+  __syncthreads();
   const size_t token = cu_q[seq];
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+  const float inv = 1.0f / l;
+  for (int d = lane; d < HD; d += kWave) {
     float o = 0.f;
-    for (int s = 0; s < nsplit; ++s) o += part_o[(base + s) * HD + d] * exp2f(part_ml[(base + s) * 2] - mm);
-    out[(token * nh + h) * HD + d] = (bf16)(o / l);
+#pragma unroll 4
+    for (int s = 0; s < nsplit; ++s) {
+      const float f = s < 1024 ? weight[s] : exp2f(part_ml[(base + s) * 2] - mm);
+      o += part_o[(base + s) * HD + d] * f;
+    }
+    out[(token * nh + h) * HD + d] = (bf16)(o * inv);
   }
 }
 
@@ -371,7 +393,7 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
                      part_ml, nh, nkv, page_size, window, scale * kLog2e, split_keys, max_splits);
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
-    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(HD < 64 ? 64 : HD), 0, st, part_o, part_ml,
+    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(kWave), 0, st, part_o, part_ml,
                        seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys, max_splits);
     return check_launch("attn_decode_merge");
   }

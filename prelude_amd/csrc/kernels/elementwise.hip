@@ -64,6 +64,58 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, T* residual, const float
   }
 }
 
+// The same with 16-byte loads and every element held in registers between the
+// two passes: one read of x and the residual, one write of each output.
+// NV vectors per thread; the block has ceil(hidden / VEC / NV) threads rounded up to a wavefront.
+template <typename T, int NV>
+__global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const float* __restrict__ w,
+                                   T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+  constexpr int VEC = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(VEC)));
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  const vec_t* xr = reinterpret_cast<const vec_t*>(x + src * hidden);
+  vec_t* rr = residual ? reinterpret_cast<vec_t*>(residual + src * hidden) : nullptr;
+  vec_t* orow = reinterpret_cast<vec_t*>(out + (size_t)r * hidden);
+  const int nvec = hidden / VEC;
+  float s[NV][VEC];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = threadIdx.x + j * blockDim.x;
+    if (v < nvec) {
+      const vec_t xv = xr[v];
+      if (rr) {
+        const vec_t rv = rr[v];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s[j][e] = to_f32(xv[e]) + to_f32(rv[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s[j][e] = to_f32(xv[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) ss += s[j][e] * s[j][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = threadIdx.x + j * blockDim.x;
+    if (v < nvec) {
+      vec_t ov, sv;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        sv[e] = from_f32<T>(s[j][e]);
+        ov[e] = from_f32<T>(s[j][e] * inv * w[v * VEC + e]);
+      }
+      if (rr && !rows) rr[v] = sv;
+      orow[v] = ov;
+    }
+  }
+}
+
 // ---- SiLU(gate) * up over a merged [T, 2I] input whose columns alternate gate_j, up_j ----
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, size_t total) {
@@ -128,6 +180,25 @@ extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual
                           const int* rows, int nrows, int hidden, float eps) {
   if (nrows == 0) return 0;
   PA_REQUIRE(nrows > 0 && hidden > 0, "rmsnorm: bad sizes rows=%d hidden=%d", nrows, hidden);
+  const int vec = dtype == kF32 ? 4 : 8;
+  if (hidden % vec == 0 && hidden / vec <= 4 * 1024) {
+    const int nvec = hidden / vec;
+    const int nv = (nvec + 1023) / 1024;   // vectors per thread: 1, 2 or 4
+    const int per = nv == 3 ? 4 : nv;
+    const int threads = (((nvec + per - 1) / per) + 63) / 64 * 64;
+#define PA_RMS(NV)                                                                                                   \
+  PA_DISPATCH(dtype, hipLaunchKernelGGL((rmsnorm_vec_kernel<T, NV>), dim3(nrows), dim3(threads), 0, (hipStream_t)stream, \
+                                        (const T*)x, (T*)residual, w, (T*)out, rows, hidden, eps))
+    if (per == 1) {
+      PA_RMS(1);
+    } else if (per == 2) {
+      PA_RMS(2);
+    } else {
+      PA_RMS(4);
+    }
+#undef PA_RMS
+    return check_launch("rmsnorm");
+  }
   const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
   PA_DISPATCH(dtype, hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(nrows), dim3(threads), 0, (hipStream_t)stream,
                                         (const T*)x, (T*)residual, w, (T*)out, rows, hidden, eps));

@@ -116,6 +116,68 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
   }
 }
 
+// The same for head_dim 64, 128 or 256 rotated over its whole width: a lane owns EPL = head_dim / 64
+// contiguous elements, read and written as one vector; its rotation partner (element + head_dim / 2)
+// sits in lane ^ 32, so nothing goes through LDS.
+template <typename T, int EPL>
+__global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
+    const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table, const int* __restrict__ positions,
+    const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int tokens,
+    int nh, int nkv, int page_size, float eps) {
+  typedef T vec_t __attribute__((ext_vector_type(EPL)));
+  constexpr int hd = EPL * kWave;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int heads = nh + 2 * nkv;
+  const long long unit = (long long)blockIdx.x * kQkWaves + wave;
+  if (unit >= (long long)tokens * heads) return;
+  const int t = (int)(unit / heads), h = (int)(unit % heads);
+  const vec_t xv = *reinterpret_cast<const vec_t*>(qkv + ((size_t)t * heads + h) * hd + lane * EPL);
+  if (h >= nh + nkv) {  // V: a copy into the transposed page
+    const long long slot = slots ? (long long)slots[t] : -1;
+    if (slot < 0) return;
+    const long long page = slot / page_size, off = slot % page_size;
+    T* dst = v_cache + ((size_t)page * nkv + (h - nh - nkv)) * hd * page_size + off;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = xv[e];
+    return;
+  }
+  T* dst;
+  const float* weight;
+  if (h < nh) {
+    dst = q_out + ((size_t)t * nh + h) * hd;
+    weight = q_weight;
+  } else {
+    const long long slot = slots ? (long long)slots[t] : -1;
+    if (slot < 0) return;
+    const long long page = slot / page_size, off = slot % page_size;
+    dst = k_cache + (((size_t)page * nkv + (h - nh)) * page_size + off) * hd;
+    weight = k_weight;
+  }
+  float x[EPL];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    x[e] = to_f32(xv[e]);
+    ss += x[e] * x[e];
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / (float)hd + eps);
+  const int pos = positions[t];
+  const int j0 = (lane % 32) * EPL;  // index into the cos/sin row
+  const float* c = cos_table + (size_t)pos * (hd / 2) + j0;
+  const float* s = sin_table + (size_t)pos * (hd / 2) + j0;
+  vec_t ov;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    if (weight) x[e] = x[e] * inv * weight[lane * EPL + e];
+    const float partner = __shfl_xor(x[e], 32, kWave);
+    const float r = lane < 32 ? x[e] * c[e] - partner * s[e] : partner * s[e] + x[e] * c[e];
+    ov[e] = from_f32<T>(r);
+  }
+  *reinterpret_cast<vec_t*>(dst + lane * EPL) = ov;
+}
+
 }  // namespace pa
 
 using namespace pa;
@@ -135,6 +197,23 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
   const long long units = (long long)tokens * (nh + 2 * nkv);
   const unsigned blocks = (unsigned)((units + kQkWaves - 1) / kQkWaves);
   hipStream_t st = (hipStream_t)stream;
+  if (rot == hd && rot > 0 && (hd == 64 || hd == 128 || hd == 256) && (dtype == kF32 || dtype == kBF16)) {
+#define PA_WIDE(T, EPL)                                                                                             \
+  hipLaunchKernelGGL((qknorm_rope_kv_wide_kernel<T, EPL>), dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const T*)qkv, \
+                     q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)q_out, (T*)k_cache, (T*)v_cache, \
+                     tokens, nh, nkv, page_size, eps)
+    if (dtype == kF32) {
+      if (hd == 64) PA_WIDE(float, 1);
+      else if (hd == 128) PA_WIDE(float, 2);
+      else PA_WIDE(float, 4);
+    } else {
+      if (hd == 64) PA_WIDE(bf16, 1);
+      else if (hd == 128) PA_WIDE(bf16, 2);
+      else PA_WIDE(bf16, 4);
+    }
+#undef PA_WIDE
+    return check_launch("qknorm_rope_kv");
+  }
   if (dtype == kF32) {
     hipLaunchKernelGGL(qknorm_rope_kv_kernel<float>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const float*)qkv,
                        q_weight, k_weight, cos_table, sin_table, positions, slots, (float*)q_out, (float*)k_cache,

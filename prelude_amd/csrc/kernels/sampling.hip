@@ -57,6 +57,51 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
   }
 }
 
+// Wide rows: grid (rows, chunks) writes one candidate per chunk, a second launch picks among them.
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ cand_v,
+                                                          int* __restrict__ cand_i, int vocab, int chunk) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const float* row = logits + (size_t)blockIdx.x * vocab;
+  const int begin = blockIdx.y * chunk;
+  const int end = begin + chunk < vocab ? begin + chunk : vocab;
+  MaxIdx best{-INFINITY, 0x7fffffff};
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
+    const float v = row[i];
+    if (v > best.v || (v == best.v && i < best.i)) best = MaxIdx{v, i};
+  }
+#pragma unroll
+  for (int m = kWave / 2; m > 0; m >>= 1) {
+    MaxIdx o{__shfl_xor(best.v, m, kWave), __shfl_xor(best.i, m, kWave)};
+    best = better(best, o);
+  }
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (lane == 0) {
+    sv[wave] = best.v;
+    si[wave] = best.i;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) best = better(best, MaxIdx{sv[w], si[w]});
+    cand_v[blockIdx.x * gridDim.y + blockIdx.y] = best.v;
+    cand_i[blockIdx.x * gridDim.y + blockIdx.y] = best.i;
+  }
+}
+
+__global__ __launch_bounds__(kWave) void argmax_pick_kernel(const float* __restrict__ cand_v,
+                                                            const int* __restrict__ cand_i, int* __restrict__ out,
+                                                            int chunks) {
+  MaxIdx best{-INFINITY, 0x7fffffff};
+  for (int c = threadIdx.x; c < chunks; c += kWave)
+    best = better(best, MaxIdx{cand_v[blockIdx.x * chunks + c], cand_i[blockIdx.x * chunks + c]});
+#pragma unroll
+  for (int m = kWave / 2; m > 0; m >>= 1) {
+    MaxIdx o{__shfl_xor(best.v, m, kWave), __shfl_xor(best.i, m, kWave)};
+    best = better(best, o);
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best.i == 0x7fffffff ? 0 : best.i;
+}
+
 __device__ __forceinline__ unsigned order_key(float v) {
   const unsigned u = __float_as_uint(v);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
@@ -205,9 +250,26 @@ extern "C" int pa_sample(void* stream, const float* logits, const float* tempera
   return check_launch("sample");
 }
 
-extern "C" int pa_argmax(void* stream, const float* logits, int* out, int rows, int vocab) {
+// Floats of scratch pa_argmax needs for rows of this width (0: none).
+extern "C" int pa_argmax_scratch(int rows, int vocab) {
+  return vocab <= 8192 ? 0 : rows * ((vocab + 2047) / 2048) * 2;
+}
+
+extern "C" int pa_argmax(void* stream, const float* logits, int* out, float* scratch, int rows, int vocab) {
   if (rows == 0) return 0;
   PA_REQUIRE(rows > 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, out, vocab);
+  if (vocab <= 8192) {
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, out, vocab);
+    return check_launch("argmax");
+  }
+  PA_REQUIRE(scratch, "argmax: rows of %d need scratch", vocab);
+  const int chunks = (vocab + 2047) / 2048;
+  PA_REQUIRE(chunks <= 65535, "argmax: %d columns exceed the grid", vocab);
+  float* cand_v = scratch;
+  int* cand_i = reinterpret_cast<int*>(scratch + (size_t)rows * chunks);
+  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(rows, chunks), dim3(256), 0, (hipStream_t)stream, logits, cand_v, cand_i,
+                     vocab, 2048);
+  if (int rc = check_launch("argmax")) return rc;
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, (hipStream_t)stream, cand_v, cand_i, out, chunks);
   return check_launch("argmax");
 }

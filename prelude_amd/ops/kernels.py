@@ -290,7 +290,9 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     if logits.dim() != 2:
         raise NativeError(f"argmax: logits {tuple(logits.shape)}")
     out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-    check(kernels().pa_argmax(_stream(), _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1]))
+    words = kernels().pa_argmax_scratch(logits.shape[0], logits.shape[1])
+    scratch = torch.empty((words,), dtype=torch.float32, device=logits.device) if words else None
+    check(kernels().pa_argmax(_stream(), _ptr(logits), _ptr(out), _ptr(scratch), logits.shape[0], logits.shape[1]))
     return out
 
 

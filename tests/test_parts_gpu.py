@@ -141,7 +141,11 @@ def test_attention_part(gpu, dtype, nh, nkv, hd, bias, window, qk_norm):
     o1 = a.forward(x[:21].to(gpu), one_sequence_step(gpu, 21, page, pages), cache2)
     o2 = a.forward(x[21:].to(gpu), one_sequence_step(gpu, n - 21, page, pages, start=21), cache2)
     assert float((torch.cat([o1, o2]).double().cpu() - ref).abs().max()) < tol
-    assert torch.equal(cache.k, cache2.k) and torch.equal(cache.v, cache2.v)
+    if dtype == torch.float32:   # one product kernel whatever the number of rows: the same bits
+        assert torch.equal(cache.k, cache2.k) and torch.equal(cache.v, cache2.v)
+    else:                        # few rows and many rows take different product kernels: equal to rounding
+        assert float((cache.k.float() - cache2.k.float()).abs().max()) < 0.05
+        assert float((cache.v.float() - cache2.v.float()).abs().max()) < 0.05
     # reading a cache another run wrote: queries only
     o3 = a.forward(x[21:].to(gpu), one_sequence_step(gpu, n - 21, page, pages, start=21), cache, write_cache=False)
     assert float((o3.double().cpu() - ref[21:]).abs().max()) < tol
