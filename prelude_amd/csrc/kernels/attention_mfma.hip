@@ -16,6 +16,10 @@
 // [page, kv_head, head_dim, offset]: in both, the contraction index of the
 // product they feed is contiguous, so every operand is loaded from memory
 // straight into registers, with no staging in LDS and no barrier in the loop.
+// Heads that share a KV head share every K and V register: a step computes
+// all their scores first, then walks V once.  Comparisons with the mask are
+// made only in steps that touch the diagonal, a window's edge or the end, and
+// an output is rescaled only in steps where a running maximum moved.
 //
 // Operand layout of v_mfma_f32_16x16x32_bf16 (lane l, g = l / 16, r = l % 16):
 //   A[16 x 32]: row r,    columns 8g .. 8g+7        B[32 x 16]: column r, rows 8g .. 8g+7
@@ -31,6 +35,8 @@
 // crates/prelude-core/src/ops/traits/attention.rs:10-99.
 #include "common.h"
 #include "api.h"
+
+#include <stdlib.h>
 
 namespace pa {
 
@@ -55,7 +61,7 @@ __device__ __forceinline__ float xor_sum16_32(float v) {
 template <int HD>
 struct HeadState {
   static constexpr int OT = HD / 16;
-  float m = -INFINITY;  // running maximum of the scaled scores (log2 domain), equal in the four lanes of a column
+  float m = -INFINITY;  // running maximum of the raw scores, equal in the four lanes of a column
   float l = 0.f;        // this lane's share of the running sum
   f32x4 o[OT];          // O^T tiles: head_dim rows 16 t + 4g + i, column r
   __device__ HeadState() {
@@ -70,11 +76,12 @@ struct KFrag {
   bf16x8 k[2][KS];
 };
 
+// Where a sequence's keys are.  Page sizes are powers of two here, so a key's page and offset are a shift and a mask.
 struct KeyWalk {
   const bf16* kc;
   const bf16* vc;
   const int* table;
-  int nkv, kvh, page_size;
+  int nkv, kvh, page_shift, page_mask;
   int lo, hi;  // keys [lo, hi) exist and may be read
 };
 
@@ -93,8 +100,9 @@ __device__ __forceinline__ void load_k(const KeyWalk& w, int key0, int g, int r,
   for (int t = 0; t < 2; ++t) {
     int key = key0 + 16 * t + r;
     key = key < w.lo ? w.lo : (key >= w.hi ? w.hi - 1 : key);
-    const int page = w.table[key / w.page_size];
-    const bf16* row = w.kc + (((size_t)page * w.nkv + w.kvh) * w.page_size + key % w.page_size) * HD + 8 * g;
+    const int page = w.table[key >> w.page_shift];
+    const bf16* row =
+        w.kc + ((((size_t)page * w.nkv + w.kvh) << w.page_shift) + (key & w.page_mask)) * HD + 8 * g;
 #pragma unroll
     for (int s = 0; s < KFrag<HD>::KS; ++s) {
       if (HD % 32 == 0 || 32 * s + 8 * g < HD) {
@@ -106,32 +114,44 @@ __device__ __forceinline__ void load_k(const KeyWalk& w, int key0, int g, int r,
   }
 }
 
-// The eight keys of lane group g, for head_dim row `d`, as the A operand of O^T = V^T P^T.
-// A chunk of four keys never straddles a page (the page size is a multiple of 4).
+// Where lane group g finds its eight keys of a 32-key step in V^T: two chunks of four keys, each
+// inside one page (pages hold a multiple of four keys).  p[t] points at head_dim row 0; row d is d pages further.
+struct VChunks {
+  const bf16* p[2];
+};
+
 template <int HD>
-__device__ __forceinline__ bf16x8 load_v(const KeyWalk& w, int key0, int g, int d) {
-  union {
-    bf16x8 v;
-    short4_t h[2];
-  } u;
+__device__ __forceinline__ VChunks v_chunks(const KeyWalk& w, int key0, int g) {
+  VChunks v;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     int c = key0 + 16 * t + 4 * g;  // first key of the chunk
     // a chunk wholly outside [lo, hi) is read from the chunk that holds the nearest key inside
     if (c + 3 < w.lo) c = w.lo & ~3;
     if (c >= w.hi) c = (w.hi - 1) & ~3;
-    const int page = w.table[c / w.page_size];
-    const bf16* p = w.vc + (((size_t)page * w.nkv + w.kvh) * HD + d) * w.page_size + c % w.page_size;
-    u.h[t] = *reinterpret_cast<const short4_t*>(p);
+    const int page = w.table[c >> w.page_shift];
+    v.p[t] = w.vc + ((((size_t)page * w.nkv + w.kvh) * HD) << w.page_shift) + (c & w.page_mask);
   }
-  return u.v;
+  return v;
 }
 
-// One step over 32 keys for one head: scores, online softmax, output update.
+__device__ __forceinline__ bf16x8 load_v(const VChunks& v, int d, int page_shift) {
+  union {
+    bf16x8 v8;
+    short4_t h[2];
+  } u;
+  u.h[0] = *reinterpret_cast<const short4_t*>(v.p[0] + ((size_t)d << page_shift));
+  u.h[1] = *reinterpret_cast<const short4_t*>(v.p[1] + ((size_t)d << page_shift));
+  return u.v8;
+}
+
+// Scores of 32 keys against one head's 16 queries, then the online softmax: returns the probabilities packed
+// as the B operand of O^T = V^T P^T and the factor the head's output so far must be scaled by.
+// `masked` false: every key of the step is visible to every query (no comparisons).
 // `vis(key)` says whether this lane's query may see the key (and the key exists).
 template <int HD, typename Visible>
-__device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int r, const KFrag<HD>& kf,
-                                         const bf16x8* qf, float scale_log2e, HeadState<HD>& st, Visible vis) {
+__device__ __forceinline__ bf16x8 scores32(int key0, int g, const KFrag<HD>& kf, const bf16x8* qf, float c,
+                                           bool masked, HeadState<HD>& st, float& alpha, Visible vis) {
   float s[8];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -139,10 +159,14 @@ __device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int 
 #pragma unroll
     for (int ks = 0; ks < KFrag<HD>::KS; ++ks) acc = mfma16(kf.k[t][ks], qf[ks], acc);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = key0 + 16 * t + 4 * g + i;
-      s[4 * t + i] = vis(key) ? acc[i] * scale_log2e : -INFINITY;
-    }
+    for (int i = 0; i < 4; ++i) s[4 * t + i] = acc[i];
+  }
+  if (masked) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (!vis(key0 + 16 * t + 4 * g + i)) s[4 * t + i] = -INFINITY;
   }
   float mx = s[0];
 #pragma unroll
@@ -150,25 +174,19 @@ __device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int 
   mx = xor_max16_32(mx);
   const float m_new = fmaxf(st.m, mx);
   const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a column that has seen no key yet
-  const float alpha = exp2f(st.m - m_safe);
+  alpha = __builtin_amdgcn_exp2f((st.m - m_safe) * c);
+  const float shift = -m_safe * c;
   bf16x8 pb;
   float psum = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float p = exp2f(s[i] - m_safe);
+    const float p = __builtin_amdgcn_exp2f(fmaf(s[i], c, shift));  // 2^((s - m) c), c = scale * log2(e)
     psum += p;
     pb[i] = (bf16)p;
   }
   st.l = st.l * alpha + psum;
   st.m = m_new;
-#pragma unroll
-  for (int t = 0; t < HeadState<HD>::OT; ++t) {
-    const bf16x8 va = load_v<HD>(w, key0, g, 16 * t + r);
-    f32x4 o = st.o[t];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] *= alpha;
-    st.o[t] = mfma16(va, pb, o);
-  }
+  return pb;
 }
 
 // Q^T of 16 queries of one head as B operands: lane (g, r) holds query r, head_dim 32 ks + 8g .. +7.
@@ -184,19 +202,55 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool valid, int g, bf16
   }
 }
 
+// One step over 32 keys for GT heads that share the keys: the scores and softmax of every head first, then
+// each V^T tile (asked for at the start of the step, so it arrives under the scores) is used by all heads.
+// An output is rescaled only when some maximum moved.  `kf` holds the step's K rows, loaded a step ahead.
+template <int HD, int GT, typename Visible>
+__device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int r, const KFrag<HD>& kf,
+                                         const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked, HeadState<HD>* st,
+                                         Visible vis) {
+  constexpr int OT = HeadState<HD>::OT;
+  const VChunks vch = v_chunks<HD>(w, key0, g);
+  bf16x8 va[OT];
+#pragma unroll
+  for (int t = 0; t < OT; ++t) va[t] = load_v(vch, 16 * t + r, w.page_shift);
+  bf16x8 pb[GT];
+  float alpha[GT];
+  bool rescale[GT];
+#pragma unroll
+  for (int j = 0; j < GT; ++j) {
+    pb[j] = scores32<HD>(key0, g, kf, qf[j], c, masked, st[j], alpha[j], vis);
+    rescale[j] = __any(alpha[j] != 1.0f);
+  }
+#pragma unroll
+  for (int t = 0; t < OT; ++t) {
+#pragma unroll
+    for (int j = 0; j < GT; ++j) {
+      f32x4 o = st[j].o[t];
+      if (rescale[j]) {
+        asm volatile("" ::: "memory");  // keep this a branch: as selects it would cost a multiply per output every step
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] *= alpha[j];
+      }
+      st[j].o[t] = mfma16(va[t], pb[j], o);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // decode: grid (splits, nkv * qtiles, sequences), 4 wavefronts, each taking every fourth step of 32 keys
 // ---------------------------------------------------------------------------
 constexpr int kDecodeWaves = 4;
 
 template <int HD>
-__global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
+__global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_size, int window,
-    float scale_log2e, int split_keys, int max_splits) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_shift, int window, float c,
+    int split_keys, int max_splits) {
   constexpr int OT = HD / 16;
+  constexpr int KS = (HD + 31) / 32;
   __shared__ float lds_o[kDecodeWaves][16][HD + 1];
   __shared__ float lds_ml[kDecodeWaves][16][2];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -215,33 +269,35 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int k_begin = sp * split_keys > lo ? sp * split_keys : lo;
   const int k_end = (sp + 1) * split_keys < ctx ? (sp + 1) * split_keys : ctx;
 
-  KeyWalk w{kc, vc, block_table + (size_t)seq * table_stride, nkv, kvh, page_size, lo, ctx};
+  KeyWalk w{kc, vc, block_table + (size_t)seq * table_stride, nkv, kvh, page_shift, (1 << page_shift) - 1, lo, ctx};
   const int head = kvh * group + qt * 16 + r;  // this lane's query head
   const bool qvalid = qt * 16 + r < group;
   const size_t token = cu_q[seq];
-  bf16x8 qf[(HD + 31) / 32];
-  load_q<HD>(q + (token * nh + (qvalid ? head : 0)) * HD, qvalid, g, qf);
+  bf16x8 qf[1][KS];
+  load_q<HD>(q + (token * nh + (qvalid ? head : 0)) * HD, qvalid, g, qf[0]);
 
-  HeadState<HD> st;
+  HeadState<HD> st[1];
   const int step0 = (sp * split_keys) / 32;  // splits start at multiples of 32 keys
   const int steps = split_keys / 32;
+  // a wavefront has two steps at most here: many wavefronts per SIMD hide the latency, not a prefetch
   for (int i = wave; i < steps; i += kDecodeWaves) {
     const int key0 = (step0 + i) * 32;
     if (key0 + 32 <= k_begin || key0 >= k_end) continue;
     KFrag<HD> kf;
     load_k<HD>(w, key0, g, r, kf);
-    attend32<HD>(w, key0, g, r, kf, qf, scale_log2e, st, [&](int key) { return key >= k_begin && key < k_end; });
+    const bool masked = key0 < k_begin || key0 + 32 > k_end;
+    attend32<HD, 1>(w, key0, g, r, kf, qf, c, masked, st, [&](int key) { return key >= k_begin && key < k_end; });
   }
-  // merge the four wavefronts through LDS
-  const float l_wave = xor_sum16_32(st.l);
+  // merge the four wavefronts through LDS; maxima leave in the log2 domain (raw maximum times c)
+  const float l_wave = xor_sum16_32(st[0].l);
   if (g == 0) {
-    lds_ml[wave][r][0] = st.m;
+    lds_ml[wave][r][0] = st[0].m * c;
     lds_ml[wave][r][1] = l_wave;
   }
 #pragma unroll
   for (int t = 0; t < OT; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_o[wave][r][16 * t + 4 * g + i] = st.o[t][i];
+    for (int i = 0; i < 4; ++i) lds_o[wave][r][16 * t + 4 * g + i] = st[0].o[t][i];
   __syncthreads();
   const int nq = group - qt * 16 < 16 ? group - qt * 16 : 16;
   for (int e = threadIdx.x; e < nq * HD; e += blockDim.x) {
@@ -319,51 +375,44 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 }
 
 // ---------------------------------------------------------------------------
-// prefill: grid (tiles of 64 tokens, nkv * head groups, sequences); a wavefront owns 16 tokens x GT heads
+// prefill: grid (pairs of 64-token tiles, nkv * head groups, sequences); a wavefront owns 16 tokens x GT heads
 // ---------------------------------------------------------------------------
+// One wavefront's share of a 64-token tile: 16 tokens from t0, all keys they may see.
 template <int HD, int GT>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
-    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
-    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
-    int page_size, int window, float scale_log2e) {
+__device__ __forceinline__ void prefill_tile(const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* kc,
+                                             const bf16* vc, const int* table, int row0, int q_len, int ctx, int t0,
+                                             int nh, int nkv, int kvh, int head0, int page_shift, int window, float c,
+                                             int g, int r) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int g = lane / 16, r = lane % 16;
-  const int group = nh / nkv;
-  const int hgroups = group / GT;
-  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
-  const int seq = seq_ids[blockIdx.z];
-  const int row0 = cu_q[seq];
-  const int q_len = cu_q[seq + 1] - row0;
-  const int ctx = context_lens[seq];
-  const int t0 = blockIdx.x * 64 + wave * 16;  // first token of this wavefront's tile, within the portion
-  if (t0 >= q_len) return;
   const int start = ctx - q_len;                // position of the portion's first token
   const bool qvalid = t0 + r < q_len;
   const int my_pos = start + t0 + r;            // this lane's query position
-  const int last_pos = start + (t0 + 15 < q_len ? t0 + 15 : q_len - 1);
+  const int last_valid = t0 + 15 < q_len ? t0 + 15 : q_len - 1;
+  const int last_pos = start + last_valid;
   const int first_pos = start + t0;
   const int lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
   const int hi = last_pos + 1;
   const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+  // keys every valid query of the tile sees: from the last token's window start up to the first token's position
+  const int all_lo = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
+  const int all_hi = first_pos + 1;
 
-  KeyWalk w{kc, vc, block_table + (size_t)seq * table_stride, nkv, kvh, page_size, lo, hi};
+  KeyWalk w{kc, vc, table, nkv, kvh, page_shift, (1 << page_shift) - 1, lo, hi};
   bf16x8 qf[GT][KS];
   HeadState<HD> st[GT];
-  const int head0 = kvh * group + hg * GT;
 #pragma unroll
   for (int j = 0; j < GT; ++j)
     load_q<HD>(q + ((size_t)(row0 + (qvalid ? t0 + r : 0)) * nh + head0 + j) * HD, qvalid, g, qf[j]);
 
-  for (int key0 = (lo / 32) * 32; key0 < hi; key0 += 32) {
-    KFrag<HD> kf;
-    load_k<HD>(w, key0, g, r, kf);
-#pragma unroll
-    for (int j = 0; j < GT; ++j)
-      attend32<HD>(w, key0, g, r, kf, qf[j], scale_log2e, st[j],
-                   [&](int key) { return key >= my_lo && key <= my_pos; });
+  int key0 = (lo / 32) * 32;
+  KFrag<HD> kf_next;
+  load_k<HD>(w, key0, g, r, kf_next);
+  for (; key0 < hi; key0 += 32) {
+    const KFrag<HD> kf = kf_next;
+    if (key0 + 32 < hi) load_k<HD>(w, key0 + 32, g, r, kf_next);   // the next step's K rows, a step ahead
+    const bool masked = key0 < all_lo || key0 + 32 > all_hi;
+    attend32<HD, GT>(w, key0, g, r, kf, qf, c, masked, st, [&](int key) { return key >= my_lo && key <= my_pos; });
   }
   if (!qvalid) return;
 #pragma unroll
@@ -380,17 +429,53 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   }
 }
 
+// A workgroup takes the tiles p and (last - p) of its sequence: under the causal mask a late tile sees many
+// keys and an early one few, and a pair always sees about the same number, so workgroups finish together.
+template <int HD, int GT>
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
+    int page_shift, int window, float c, int paired) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int group = nh / nkv;
+  const int hgroups = group / GT;
+  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int seq = seq_ids[blockIdx.z];
+  const int row0 = cu_q[seq];
+  const int q_len = cu_q[seq + 1] - row0;
+  const int ctx = context_lens[seq];
+  const int tiles = (q_len + 63) / 64;
+  // unpaired: one tile per workgroup, late (long) tiles first
+  const int first = paired ? (int)blockIdx.x : tiles - 1 - (int)blockIdx.x;
+  const int second = paired ? tiles - 1 - (int)blockIdx.x : first;
+  if (first > second || first < 0) return;
+  const int* table = block_table + (size_t)seq * table_stride;
+  const int head0 = kvh * group + hg * GT;
+  {
+    const int t0 = second * 64 + wave * 16;   // the long one first
+    if (t0 < q_len)
+      prefill_tile<HD, GT>(q, out, kc, vc, table, row0, q_len, ctx, t0, nh, nkv, kvh, head0, page_shift, window, c, g, r);
+  }
+  if (first != second) {
+    const int t0 = first * 64 + wave * 16;
+    if (t0 < q_len)
+      prefill_tile<HD, GT>(q, out, kc, vc, table, row0, q_len, ctx, t0, nh, nkv, kvh, head0, page_shift, window, c, g, r);
+  }
+}
+
 // ---------------------------------------------------------------------------
 template <int HD>
 int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                  float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_size, int window, float scale,
+                  float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_shift, int window, float scale,
                   int split_keys, int max_splits) {
   const int qtiles = (nh / nkv + 15) / 16;
   dim3 grid(max_splits, nkv * qtiles, nseq);
   hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(kDecodeWaves * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                      (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                     part_ml, nh, nkv, page_size, window, scale * kLog2e, split_keys, max_splits);
+                     part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits);
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
     hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(kWave), 0, st, part_o, part_ml,
@@ -403,23 +488,29 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
 template <int HD, int GT>
 int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                       int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                      int nseq, int max_q_len, int nh, int nkv, int page_size, int window, float scale) {
-  dim3 grid((max_q_len + 63) / 64, nkv * (nh / nkv / GT), nseq);
+                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale) {
+  // pair tiles only when the pairs alone still give every SIMD of the chip several wavefronts
+  const int tiles = (max_q_len + 63) / 64;
+  const long wgs = (long)tiles * nkv * (nh / nkv / GT) * nseq;
+  // (measured: pairing wins even when it leaves wavefront slots empty, so it is on whenever there are two tiles)
+  static const char* env = getenv("PA_PREFILL_PAIRED");
+  const int paired = env ? atoi(env) : (tiles >= 2 && wgs > 0 ? 1 : 0);
+  dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / GT), nseq);
   hipLaunchKernelGGL((attn_prefill_kernel<HD, GT>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kc,
                      (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, nh, nkv,
-                     page_size, window, scale * kLog2e);
+                     page_shift, window, scale * kLog2e, paired);
   return check_launch("attn_prefill");
 }
 
 template <int HD>
 int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
-                   int max_q_len, int nh, int nkv, int page_size, int window, float scale) {
+                   int max_q_len, int nh, int nkv, int page_shift, int window, float scale) {
   const int group = nh / nkv;
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
-                                   max_q_len, nh, nkv, page_size, window, scale)
-  if (group % 4 == 0) PA_GT(4);
+                                   max_q_len, nh, nkv, page_shift, window, scale)
+  if (HD <= 64 && group % 4 == 0) PA_GT(4);  // wider heads would not fit four heads' state in 256 registers
   if (group % 2 == 0) PA_GT(2);
   PA_GT(1);
 #undef PA_GT
@@ -444,7 +535,8 @@ static int check_common(const char* what, int nseq, int nh, int nkv, int page_si
   PA_REQUIRE(nseq > 0 && nh > 0 && nkv > 0 && table_stride > 0, "%s: bad sizes sequences=%d nh=%d nkv=%d table_stride=%d",
              what, nseq, nh, nkv, table_stride);
   PA_REQUIRE(nh % nkv == 0, "%s: %d query heads are not a multiple of %d KV heads", what, nh, nkv);
-  PA_REQUIRE(page_size >= 4 && page_size % 4 == 0, "%s: page size %d is not a multiple of 4", what, page_size);
+  PA_REQUIRE(page_size >= 4 && (page_size & (page_size - 1)) == 0, "%s: page size %d is not a power of two >= 4", what,
+             page_size);
   PA_REQUIRE(window >= 0, "%s: window %d is negative (0 means none)", what, window);
   PA_REQUIRE(nseq <= 65535, "%s: %d sequences exceed the grid", what, nseq);
   return 0;
@@ -453,7 +545,7 @@ static int check_common(const char* what, int nseq, int nh, int nkv, int page_si
 // 1 if the MFMA kernels take this head_dim and page size, else 0 (the caller then uses the generic kernel).
 extern "C" int pa_attn_mfma_supports(int hd, int page_size) {
   const bool hd_ok = hd == 16 || hd == 32 || hd == 48 || hd == 64 || hd == 96 || hd == 128;
-  return hd_ok && page_size >= 4 && page_size % 4 == 0;
+  return hd_ok && page_size >= 4 && (page_size & (page_size - 1)) == 0;
 }
 
 // Workspace the decode kernel needs, in floats, for `nseq` sequences cut into at most `max_splits` splits.
@@ -474,7 +566,8 @@ extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const
   float* part_ml = workspace ? workspace + (size_t)nseq * nh * max_splits * hd : nullptr;
 #define PA_CALL(HD)                                                                                                  \
   return launch_decode<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                           out, part_o, part_ml, nseq, nh, nkv, page_size, window, scale, split_keys, max_splits)
+                           out, part_o, part_ml, nseq, nh, nkv, __builtin_ctz(page_size), window, scale, split_keys,   \
+                           max_splits)
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
@@ -488,7 +581,7 @@ extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, cons
   PA_REQUIRE(max_q_len >= 1, "attn_prefill: longest portion %d", max_q_len);
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, nh, nkv, page_size, window, scale)
+                            out, nseq, max_q_len, nh, nkv, __builtin_ctz(page_size), window, scale)
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
