@@ -153,6 +153,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone and print its record (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus, flush=True)
@@ -167,6 +168,11 @@ def main() -> int:
     el = 2 if args.dtype == "bfloat16" else 4
     short = "bf16" if args.dtype == "bfloat16" else "f32"
 
+    if args.prefill_only:
+        psec = time_prefill(raw, args.dtype, args.prefill_tokens, reps=3)
+        print(json.dumps({"prefill_tokens": args.prefill_tokens, "ms": round(psec * 1e3, 3),
+                          "tok_per_s": round(args.prefill_tokens / psec, 1)}), flush=True)
+        return 0
     sec = decode_point(raw, args.dtype, args.batch, args.context, args.steps, args.warmup, None)
     value = args.batch / sec
     wbytes, matmul_params = weight_bytes(raw, el)
