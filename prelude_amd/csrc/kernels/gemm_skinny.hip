@@ -32,6 +32,7 @@
 namespace pa {
 
 constexpr int kSkinnyMaxM = 64;
+constexpr int kDepth = 2;  // k-steps of loads a wavefront keeps in flight (4 measured slower: the memory system thrashes)
 
 struct Frag {
   bf16x8 lo, hi;
@@ -57,20 +58,27 @@ __device__ __forceinline__ Frag load_frag(const bf16* row, int k0, int k, bool o
 
 enum Epilogue : int { kPlain = 0, kSiluMul = 1 };
 
-template <int MT, int WAVES, typename TC, int EPI>
+// NT tiles of 16 rows of W per workgroup: with two, every X fragment serves two products, which halves the
+// share of the loads that X makes up (X comes from L2, but the loads cost the same as any).
+template <int MT, int NT, int WAVES, typename TC, int EPI>
 __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                    const bf16* __restrict__ w,
                                                                    const float* __restrict__ bias,
                                                                    TC* __restrict__ c, int m, int n, int k, long ldx,
                                                                    long ldc) {
-  __shared__ float red[WAVES][MT][kWave][4];
+  __shared__ float red[WAVES][NT * MT][kWave][4];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int steps = (k + 63) / 64;
 
-  const bool n_ok = n0 + r < n;
-  const bf16* wrow = w + (size_t)(n_ok ? n0 + r : 0) * k + 16 * g;
+  bool n_ok[NT];
+  const bf16* wrow[NT];
+#pragma unroll
+  for (int u = 0; u < NT; ++u) {
+    n_ok[u] = n0 + 16 * u + r < n;
+    wrow[u] = w + (size_t)(n_ok[u] ? n0 + 16 * u + r : 0) * k + 16 * g;
+  }
   const bf16* xrow[MT];
   bool m_ok[MT];
 #pragma unroll
@@ -78,61 +86,79 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
     m_ok[t] = 16 * t + r < m;
     xrow[t] = x + (size_t)(m_ok[t] ? 16 * t + r : 0) * ldx + 16 * g;
   }
-  f32x4 acc[MT];
+  f32x4 acc[NT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < NT; ++u)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // two k-steps in flight per wavefront: the next step's rows of W and X are asked for before this step's are used
+  // kDepth k-steps in flight per wavefront: a ring of fragments, refilled as soon as a slot has been used.
+  // Steps past the end load zeros, so the ring needs no tail handling.
   const int kk = k - 16 * g;
-  int s = wave;
-  Frag wn = load_frag(wrow, s * 64, kk, n_ok && s < steps);
-  Frag xn[MT];
+  Frag wbuf[kDepth][NT], xbuf[kDepth][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xn[t] = load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
-  for (; s < steps; s += WAVES) {
-    const Frag wc = wn;
-    Frag xc[MT];
+  for (int d = 0; d < kDepth; ++d) {
+    const int s = wave + d * WAVES;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) xc[t] = xn[t];
-    const int next = s + WAVES;
-    wn = load_frag(wrow, next * 64, kk, n_ok && next < steps);
+    for (int u = 0; u < NT; ++u) wbuf[d][u] = load_frag(wrow[u], s * 64, kk, n_ok[u] && s < steps);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) xn[t] = load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
+    for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
+  }
+  for (int s0 = wave; s0 < steps; s0 += WAVES * kDepth) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.lo, xc[t].lo, acc[t], 0, 0, 0);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.hi, xc[t].hi, acc[t], 0, 0, 0);
+    for (int d = 0; d < kDepth; ++d) {
+      Frag wc[NT], xc[MT];
+#pragma unroll
+      for (int u = 0; u < NT; ++u) wc[u] = wbuf[d][u];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xc[t] = xbuf[d][t];
+      const int next = s0 + (d + kDepth) * WAVES;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) wbuf[d][u] = load_frag(wrow[u], next * 64, kk, n_ok[u] && next < steps);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u].lo, xc[t].lo, acc[u][t], 0, 0, 0);
+          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u].hi, xc[t].hi, acc[u][t], 0, 0, 0);
+        }
     }
   }
-  // the wavefronts' shares, added in wavefront order by wavefront 0
+  // the wavefronts' shares, added in wavefront order; wavefront u finishes tile u (NT <= WAVES)
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int u = 0; u < NT; ++u)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][t][lane][i] = acc[t][i];
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][u * MT + t][lane][i] = acc[u][t][i];
   __syncthreads();
-  if (wave != 0) return;
+  if (wave >= NT) return;
+  const int u = wave;
+  f32x4 fin[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float v = red[0][t][lane][i];
+      float v = red[0][u * MT + t][lane][i];
 #pragma unroll
-      for (int u = 1; u < WAVES; ++u) v += red[u][t][lane][i];
-      acc[t][i] = v;
+      for (int q = 1; q < WAVES; ++q) v += red[q][u * MT + t][lane][i];
+      fin[t][i] = v;
     }
   // epilogue: lane (g, r) writes four consecutive n of token 16t + r
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int mi = 16 * t + r;
     if (mi >= m) continue;
-    const int nb = n0 + 4 * g;
+    const int nb = n0 + 16 * u + 4 * g;
     if (EPI == kSiluMul) {
       // rows alternate gate_j, up_j: outputs nb/2 and nb/2 + 1
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int nn = nb + 2 * j;
         if (nn + 1 < n) {
-          const float gate = acc[t][2 * j], up = acc[t][2 * j + 1];
+          const float gate = fin[t][2 * j], up = fin[t][2 * j + 1];
           c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate / (1.0f + expf(-gate)) * up);
         }
       }
@@ -140,7 +166,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (nb + i < n) {
-          float v = acc[t][i];
+          float v = fin[t][i];
           if (bias) v += bias[nb + i];
           c[(size_t)mi * ldc + nb + i] = from_f32<TC>(v);
         }
@@ -149,27 +175,41 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
   }
 }
 
-// Wavefronts per workgroup for an [n, k] weight: aim at about 3000 wavefronts on the chip, each with at
-// least two k-steps.  Depends on the weight's shape only, never on the batch.
-static int skinny_waves(int n, int k) {
+// Shape of the launch for an [n, k] weight: tiles of 16 rows per workgroup and wavefronts per workgroup.
+// Wide weights take two tiles; then about 3000 wavefronts on the chip, each with at least two k-steps.
+// Depends on the weight's shape only, never on the batch.
+static void skinny_shape(int n, int k, int mt, int* nt, int* waves) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
+  *nt = mt > 1 ? 1 : (tiles >= 4096 ? 4 : (tiles >= 768 ? 2 : 1));
+  const int wgs = (tiles + *nt - 1) / *nt;
   int w = 4;
-  while (w < 16 && tiles * w < 3000 && steps / (2 * w) >= 2) w *= 2;
-  return w;
+  while (w < 16 && wgs * w < 3000 && steps / (2 * w) >= 2) w *= 2;
+  *waves = w;
 }
 
 template <int MT, typename TC, int EPI>
 int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
                   long ldx, long ldc) {
-  dim3 grid((n + 15) / 16);
-#define PA_W(WV)                                                                                               \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, TC, EPI>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
+  int nt, waves;
+  skinny_shape(n, k, MT, &nt, &waves);
+  dim3 grid(((n + 15) / 16 + nt - 1) / nt);
+#define PA_W(NT, WV)                                                                                            \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
                      (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc)
-  switch (skinny_waves(n, k)) {
-    case 16: PA_W(16); break;
-    case 8: PA_W(8); break;
-    default: PA_W(4); break;
+#define PA_WAVES(NT)            \
+  switch (waves) {              \
+    case 16: PA_W(NT, 16); break; \
+    case 8: PA_W(NT, 8); break;   \
+    default: PA_W(NT, 4); break;  \
   }
+  if (MT == 1 && nt == 4) {
+    PA_WAVES((MT == 1 ? 4 : 1))
+  } else if (MT == 1 && nt == 2) {
+    PA_WAVES((MT == 1 ? 2 : 1))
+  } else {
+    PA_WAVES(1)
+  }
+#undef PA_WAVES
 #undef PA_W
   return check_launch("gemm_skinny");
 }
