@@ -8,7 +8,9 @@ The default run has the layer sizes of the Qwen3-4B shape (36 layers, hidden
 151936, tied head) with random bfloat16 weights, a batch of 8 and a context of
 4,096 tokens: every request is prefilled through the engine's own step
 function, then K decode steps are timed (each step: build the batch, run the
-model from the paged cache, greedy argmax on the device, ids back to the host).
+model from the paged cache, greedy argmax on the device, ids back to the host;
+the host prepares a step while the one before it runs, as the engine's
+generation loop does).
 One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is
 a 2,048-token prompt portion; ``roofline`` prices the decode step against HBM
 bandwidth; ``points`` holds batch 1 and 64.
@@ -87,16 +89,33 @@ def prefill_requests(engine, batch, length, chunk, vocab, seed):
 
 
 def time_decode(engine, batch, steps, warmup, vocab):
-    """Greedy decode steps for `batch` live requests; returns seconds per step."""
+    """Greedy decode steps for `batch` live requests; returns seconds per step.
+
+    As in ``LLM.generate``, a step is launched with the previous step's ids
+    still on the device, and those ids are read on the host while it runs.
+    """
     import torch
     from prelude_amd.engine import StepEntry
     from prelude_amd.ops import kernels as K
-    last = [1] * batch
+    state = {"sampled": None, "pending": None, "ids": [1] * batch}
 
     def one():
-        nonlocal last
-        logits = engine.step([StepEntry(r, [last[r]], [0]) for r in range(batch)])
-        last = K.argmax(logits).tolist()
+        prev = state["sampled"]
+        if prev is None:
+            entries = [StepEntry(r, [state["ids"][r]], [0]) for r in range(batch)]
+        else:
+            entries = [StepEntry(r, [0], [0], carry=r) for r in range(batch)]
+        logits = engine.step(entries, carried=prev)
+        sampled = K.argmax(logits)
+        host = torch.empty(batch, dtype=torch.int32, pin_memory=True)
+        host.copy_(sampled, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        if state["pending"] is not None:
+            pev, phost = state["pending"]
+            pev.synchronize()
+            state["ids"] = phost.tolist()
+        state["sampled"], state["pending"] = sampled, (ev, host)
 
     for _ in range(warmup):
         one()

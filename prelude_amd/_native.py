@@ -38,6 +38,7 @@ _KERNEL_API = {
     "pa_device_arch": (I, [c_char_p, I]),
     "pa_num_compute_units": (I, []),
     "pa_embed_gather": (I, [P, I, P, P, P, I, I, I]),
+    "pa_carry_tokens": (I, [P, P, P, P, P, I, I, I]),
     "pa_rmsnorm": (I, [P, I, P, P, P, P, P, I, I, F]),
     "pa_silu_mul": (I, [P, I, P, P, I, I]),
     "pa_gather_rows": (I, [P, I, P, P, P, I, I]),

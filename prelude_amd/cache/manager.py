@@ -154,7 +154,7 @@ class PageTables:
         G = len(self.groups)
         sizes = [("token_ids", total), ("positions", total), ("seq_of_token", total), ("cu_q", n + 1),
                  ("context_lens", n), ("state_slots", n), ("fresh", n), ("want_rows", wanted),
-                 ("decode_seqs", n), ("prefill_seqs", n),
+                 ("decode_seqs", n), ("prefill_seqs", n), ("carry_src", n), ("carry_dst", n),
                  ("block_tables", G * n * stride), ("slots", G * total)]
         out, off = {}, 0
         for name, sz in sizes:

@@ -14,6 +14,9 @@ int pa_num_compute_units();
 // out[t, :] = table[ids[t], :]
 int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, void* out, int tokens, int hidden,
                     int vocab);
+// ids[dst[i]] = sampled[src[i]] for i < n with src[i] >= 0 (token ids handed from one step to the next on the device).
+int pa_carry_tokens(void* stream, const int* sampled, const int* src, const int* dst, int* ids, int n, int sampled_rows,
+                    int tokens);
 // RMSNorm of x (+ residual, which then receives the sum) with a 32-bit weight;
 // with `rows`, output row r comes from input row rows[r] and the residual is left alone.
 int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out, const int* rows,

@@ -33,6 +33,19 @@ __global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __rest
   }
 }
 
+// ---- token ids that never left the device ------------------------------
+// ids[dst[i]] = sampled[src[i]] for every i with src[i] >= 0: a step that is
+// launched before the host has read the previous step's tokens takes them here.
+__global__ void carry_tokens_kernel(const int* __restrict__ sampled, const int* __restrict__ src,
+                                    const int* __restrict__ dst, int* __restrict__ ids, int n, int sampled_rows,
+                                    int tokens) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int s = src[i], d = dst[i];
+  if (s < 0 || s >= sampled_rows || d < 0 || d >= tokens) return;
+  ids[d] = sampled[s];
+}
+
 // ---- RMSNorm, optionally fused with the residual add --------------------
 //   s = x (+ residual)                         in 32-bit
 //   residual <- round(s)                       (only when `residual` is given and `rows` is not)
@@ -174,6 +187,16 @@ extern "C" int pa_embed_gather(void* stream, int dtype, const int* ids, const vo
   PA_DISPATCH(dtype, hipLaunchKernelGGL(embed_gather_kernel<T>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, ids,
                                         (const T*)table, (T*)out, hidden, vocab));
   return check_launch("embed_gather");
+}
+
+extern "C" int pa_carry_tokens(void* stream, const int* sampled, const int* src, const int* dst, int* ids, int n,
+                               int sampled_rows, int tokens) {
+  if (n == 0) return 0;
+  PA_REQUIRE(n > 0 && sampled_rows > 0 && tokens > 0, "carry_tokens: bad sizes n=%d sampled=%d tokens=%d", n,
+             sampled_rows, tokens);
+  hipLaunchKernelGGL(carry_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, sampled, src, dst,
+                     ids, n, sampled_rows, tokens);
+  return check_launch("carry_tokens");
 }
 
 extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out,

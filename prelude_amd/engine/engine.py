@@ -37,6 +37,7 @@ class StepEntry:
     id: int
     tokens: Sequence[int]
     want: Sequence[int] = ()     # indices into ``tokens`` whose logits are wanted
+    carry: Optional[int] = None  # the last of ``tokens`` is a stand-in: its id is row ``carry`` of the step's ``carried``
 
 
 class _Staging:
@@ -141,14 +142,19 @@ class Engine:
         self._live.pop(rid, None)
 
     # ---- the step -----------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], carried: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Opens unknown requests, takes pages, runs, and records the new lengths.
 
         Returns float32 logits [sum(len(want)), vocab] in the order of the
         entries and of each entry's ``want``.  Raises ``OutOfPages`` (with
         nothing taken and nothing run) if the pools cannot hold the step.
+
+        ``carried`` is an int32 device tensor of token ids the host has not
+        read yet (the previous step's samples): an entry with ``carry`` set
+        takes its last token from there, on the device, so this step can be
+        launched while the previous one still runs.
         """
-        self._validate(entries)
+        self._validate(entries, carried)
         opened, reserved = [], []
         try:
             for e in entries:
@@ -165,7 +171,7 @@ class Engine:
             raise
         starts = [self.tables.length(e.id) for e in entries]
         try:
-            logits = self.run(entries, starts)
+            logits = self.run(entries, starts, carried)
         except Exception:
             for e in entries:
                 self.tables.rollback(e.id)
@@ -178,9 +184,10 @@ class Engine:
             logits = logits.clone()   # the graph's own output tensor is overwritten by the next replay
         return logits
 
-    def _validate(self, entries: Sequence[StepEntry]) -> None:
+    def _validate(self, entries: Sequence[StepEntry], carried: Optional[torch.Tensor] = None) -> None:
         if not entries:
             raise StepError("a step needs at least one entry")
+        self._validate_carried(entries, carried)
         seen = set()
         for e in entries:
             if e.id in seen:
@@ -202,8 +209,21 @@ class Engine:
                 raise StepError(f"request {e.id}: {have} + {n} tokens exceed max_position_embeddings "
                                 f"{self.max_positions}")
 
+    def _validate_carried(self, entries: Sequence[StepEntry], carried: Optional[torch.Tensor]) -> None:
+        rows = [e.carry for e in entries if e.carry is not None]
+        if not rows:
+            return
+        if carried is None:
+            raise StepError("an entry carries a token from the device but the step was given no carried tensor")
+        if carried.dtype != torch.int32 or carried.dim() != 1 or carried.device != self.device:
+            raise StepError(f"carried token ids must be a 1-d int32 tensor on {self.device}")
+        for r in rows:
+            if not 0 <= int(r) < carried.shape[0]:
+                raise StepError(f"carried row {r} is outside the {carried.shape[0]} token ids carried")
+
     def build_batch(self, entries: Sequence[StepEntry], starts: Sequence[int], stride: Optional[int] = None,
-                    device_buffer: Optional[torch.Tensor] = None) -> StepBatch:
+                    device_buffer: Optional[torch.Tensor] = None,
+                    carried: Optional[torch.Tensor] = None) -> StepBatch:
         """Index arrays of the step, built on the host in one pinned buffer and sent in one copy.
 
         ``stride`` widens the block tables beyond what the step needs and
@@ -225,14 +245,24 @@ class Engine:
         host = pinned.numpy()
         off, _ = layout["token_ids"]
         woff, _ = layout["want_rows"]
+        csoff, _ = layout["carry_src"]
+        cdoff, _ = layout["carry_dst"]
         t = 0
         w = 0
-        for e, c in zip(entries, counts):
+        carries = 0
+        for i, (e, c) in enumerate(zip(entries, counts)):
             host[off + t: off + t + c] = e.tokens
             for x in e.want:
                 host[woff + w] = t + int(x)
                 w += 1
             t += c
+            if e.carry is None:
+                host[csoff + i] = -1
+                host[cdoff + i] = -1
+            else:
+                host[csoff + i] = int(e.carry)
+                host[cdoff + i] = t - 1
+                carries += 1
         self.tables.fill_step([e.id for e in entries], starts, counts, stride, host, layout)
         dec = [i for i, c in enumerate(counts) if c == 1]
         pre = [i for i, c in enumerate(counts) if c > 1]
@@ -257,6 +287,10 @@ class Engine:
             o, s = layout[name]
             return dev[o: o + s]
 
+        if carries:
+            from ..ops import kernels as K
+            self._validate_carried(entries, carried)
+            K.carry_tokens(carried, view("carry_src"), view("carry_dst"), view("token_ids"))
         G = len(self.group_specs)
         bt = view("block_tables").view(G, n, stride) if G else None
         sl = view("slots").view(G, total) if G else None
@@ -273,7 +307,8 @@ class Engine:
                          # with fixed buffers the launch shapes must not follow the data: bound by what the tables can hold
                          max_decode_context=(stride * self.page_size if fixed else max([ends[i] for i in dec], default=0)))
 
-    def run(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], starts: Sequence[int],
+            carried: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs a step whose pages are already reserved (the scheduler's path).
 
         A step of single tokens whose logits are all wanted is replayed from a
@@ -281,8 +316,8 @@ class Engine:
         then the graph's own and is overwritten by the next such step.
         """
         if self._graphs is not None and self._graphs.eligible(entries):
-            return self._graphs.run(entries, starts)
-        batch = self.build_batch(entries, starts)
+            return self._graphs.run(entries, starts, carried)
+        batch = self.build_batch(entries, starts, carried=carried)
         if self.model.needs_state:
             fresh = [s for s, f in zip(batch.state_slots_host, batch.fresh_host) if f and s >= 0]
             if fresh:

@@ -13,6 +13,10 @@ with fixed input buffers refreshed before each replay
 block-table width is part of the key (rounded up, so few graphs cover all
 context lengths) and graphs are captured when first needed.
 
+A graph may be launched again while its previous launch still runs (the host
+prepares one step ahead): launches on one stream run in order, and the index
+buffer is refreshed by a copy on that same stream.
+
 Nothing inside a captured step may depend on the step's data through the
 host: launch shapes follow the batch size and the table width only (the
 decode attention kernel is launched for as many splits as the table could
@@ -59,27 +63,27 @@ class DecodeGraphs:
         need = -(-max(ends) // page)
         return -(-need // step) * step
 
-    def run(self, entries: Sequence, starts: Sequence[int]) -> torch.Tensor:
+    def run(self, entries: Sequence, starts: Sequence[int], carried=None) -> torch.Tensor:
         eng = self.engine
         n = len(entries)
         stride = self._stride_for([s + 1 for s in starts])
         key = (n, stride)
         cap = self._graphs.get(key)
         if cap is None:
-            cap = self._capture(entries, starts, stride)
+            cap = self._capture(entries, starts, stride, carried)
             self._graphs[key] = cap
         else:
-            eng.build_batch(entries, starts, stride=stride, device_buffer=cap.buffer)
+            eng.build_batch(entries, starts, stride=stride, device_buffer=cap.buffer, carried=carried)
         cap.graph.replay()
         self.replays += 1
         return cap.logits
 
-    def _capture(self, entries: Sequence, starts: Sequence[int], stride: int) -> _Captured:
+    def _capture(self, entries: Sequence, starts: Sequence[int], stride: int, carried=None) -> _Captured:
         eng = self.engine
         n = len(entries)
         size = eng.tables.step_layout(n, n, stride, n)["_total"][1]
         buffer = torch.empty(size, dtype=torch.int32, device=eng.device)
-        batch = eng.build_batch(entries, starts, stride=stride, device_buffer=buffer)
+        batch = eng.build_batch(entries, starts, stride=stride, device_buffer=buffer, carried=carried)
         # once outside a capture, on a side stream, so that whatever libraries set up lazily exists already;
         # it writes the same keys and values the replay will write
         side = torch.cuda.Stream(device=eng.device)

@@ -6,8 +6,13 @@ types (crates/prelude-core/src/types.rs:388-455): per request a prompt (text
 or token ids), ``max_tokens``, sampling options, stop token ids and a seed;
 per result the generated ids, why it finished (``stop`` | ``length`` | ``eos``),
 token counts and the four timings ``ttft_ms, prefill_ms, decode_ms, total_ms``.
-The loop is the reference's ``ar_loop`` (crates/prelude-core/src/engine/run/ar.rs:180-396)
-made synchronous: schedule, build the step, run it, sample, finish.
+The loop is the reference's ``ar_loop`` (crates/prelude-core/src/engine/run/ar.rs:180-396):
+schedule, build the step, run it, sample, finish.  With ``overlap_steps`` the
+host runs one step ahead of the device: step N+1 is scheduled and launched
+while step N still runs, taking N's sampled ids on the device, and N's ids are
+read only afterwards.  What is computed, and so every token, is the same as
+in the synchronous loop; a request that ends on a token's value (EOS, a stop
+id) has by then been fed one step too many, whose sample is dropped.
 """
 from __future__ import annotations
 
@@ -21,7 +26,7 @@ import torch
 from .config.engine_config import EngineConfig
 from .engine.engine import Engine, StepEntry
 from .engine.scheduler import Scheduler
-from .sampling.sampler import RequestSampler, SamplingParams, sample_rows
+from .sampling.sampler import RequestSampler, SamplingParams, sample_rows_device
 
 DEFAULT_MAX_TOKENS = 4096   # crates/prelude-server/src/routes/generation_common.rs:9
 
@@ -56,6 +61,18 @@ class _Live:
     t_arrive: float
     t_first: Optional[float] = None
     finish_reason: Optional[str] = None
+    pending_row: Optional[int] = None    # the last of ``tokens`` is still on the device: its row among the step's samples
+    done: bool = False
+    preemptions: int = 0
+
+
+@dataclasses.dataclass
+class _InFlight:
+    """A launched step whose sampled ids the host has not read yet."""
+    drawn: List[_Live]
+    sampled: torch.Tensor        # int32 [len(drawn)] on the device
+    host: torch.Tensor           # pinned copy of it, valid once ``ready`` has passed
+    ready: torch.cuda.Event
 
 
 class LLM:
@@ -135,41 +152,90 @@ class LLM:
             self.scheduler.add_request(rid, len(ids), max_new)
             live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop, now)
 
-        while live:
-            portions = self.scheduler.schedule()
-            if not portions:
+        overlap = bool(self.config.overlap_steps)
+        in_flight: Optional[_InFlight] = None
+        while live or in_flight is not None:
+            launched = self._launch(live, in_flight) if live else None
+            if launched is None and in_flight is None:
                 raise RuntimeError("the scheduler has requests but nothing to run")
-            entries = [StepEntry(p.id, live[p.id].tokens[p.start:p.start + p.count], [p.count - 1] if p.samples else [])
-                       for p in portions]
-            try:
-                logits = self.engine.run(entries, [p.start for p in portions])
-            except Exception:
-                self.scheduler.step_cancelled()
-                raise
-            self.scheduler.step_done()
-            self.steps += 1
-            drawn = [live[p.id] for p in portions if p.samples]
-            toks = sample_rows(logits, [r.sampler for r in drawn])   # waits for the device
-            t = time.perf_counter()
-            for r, tok in zip(drawn, toks):
-                self.scheduler.on_token(r.rid)
-                r.tokens.append(int(tok))
-                if r.t_first is None:
-                    r.t_first = t
-                n_out = len(r.tokens) - len(r.prompt)
-                # order of checks: crates/prelude-core/src/engine/run/ar.rs:1525-1578
-                if tok in self.eos_token_ids:
-                    r.finish_reason = "eos"
-                elif tok in r.stop_ids:
-                    r.finish_reason = "stop"
-                elif n_out >= r.max_new:
-                    r.finish_reason = "length"
-                if r.finish_reason:
-                    info = self.scheduler.info(r.rid)
-                    self.scheduler.finish(r.rid)
-                    results[r.index] = self._result(r, t, info.preempt_count)
-                    del live[r.rid]
+            if not overlap and launched is not None:
+                in_flight, launched = launched, None
+            if in_flight is not None:
+                self._resolve(in_flight, live, results)
+            in_flight = launched
         return results  # type: ignore[return-value]
+
+    def _launch(self, live: Dict[int, _Live], previous: Optional[_InFlight]) -> Optional[_InFlight]:
+        """Schedules and launches one step; the scheduler is told at once that its tokens exist."""
+        portions = self.scheduler.schedule()
+        if not portions:
+            return None
+        entries = []
+        for p in portions:
+            r = live[p.id]
+            toks = r.tokens[p.start:p.start + p.count]
+            carry = None
+            if toks[-1] is None:       # sampled by the step before, not read yet
+                toks = toks[:-1] + [0]
+                carry = r.pending_row
+            entries.append(StepEntry(p.id, toks, [p.count - 1] if p.samples else [], carry))
+        try:
+            logits = self.engine.run(entries, [p.start for p in portions],
+                                     previous.sampled if previous is not None else None)
+        except Exception:
+            self.scheduler.step_cancelled()
+            raise
+        self.scheduler.step_done()
+        self.steps += 1
+        drawn = [live[p.id] for p in portions if p.samples]
+        sampled = sample_rows_device(logits, [r.sampler for r in drawn])
+        host = torch.empty(len(drawn), dtype=torch.int32, pin_memory=True)
+        host.copy_(sampled, non_blocking=True)
+        ready = torch.cuda.Event()
+        ready.record()
+        for row, r in enumerate(drawn):
+            self.scheduler.on_token(r.rid)
+            r.tokens.append(None)
+            r.pending_row = row
+            if len(r.tokens) - len(r.prompt) >= r.max_new:
+                # the last token it may have, whatever its value: nothing more is scheduled for it
+                r.preemptions = self.scheduler.info(r.rid).preempt_count
+                self.scheduler.finish(r.rid)
+                r.finish_reason = "length"
+                del live[r.rid]
+        return _InFlight(drawn, sampled, host, ready)
+
+    def _resolve(self, step: _InFlight, live: Dict[int, _Live], results: List[Optional[GenerationResult]]) -> None:
+        """Reads a step's sampled ids and ends the requests they end."""
+        step.ready.synchronize()
+        toks = step.host.tolist()
+        t = time.perf_counter()
+        for r, tok in zip(step.drawn, toks):
+            if r.done:                 # ended by an earlier token while this step was already running
+                continue
+            at = len(r.tokens) - 1
+            if at >= 1 and r.tokens[at - 1] is None:   # the step launched since then has put its own stand-in behind
+                at -= 1
+            r.tokens[at] = int(tok)
+            if r.t_first is None:
+                r.t_first = t
+            # order of checks: crates/prelude-core/src/engine/run/ar.rs:1525-1578
+            if tok in self.eos_token_ids:
+                reason = "eos"
+            elif tok in r.stop_ids:
+                reason = "stop"
+            elif at + 1 - len(r.prompt) >= r.max_new:
+                reason = "length"
+            else:
+                continue
+            del r.tokens[at + 1:]
+            if r.rid in live:          # ended by the token's value: the scheduler still holds it
+                r.preemptions = self.scheduler.info(r.rid).preempt_count
+                self.scheduler.finish(r.rid)
+                del live[r.rid]
+            r.finish_reason = reason
+            r.done = True
+            results[r.index] = self._result(r, t, r.preemptions)
 
     def _result(self, r: _Live, t_end: float, preemptions: int) -> GenerationResult:
         out = r.tokens[len(r.prompt):]

@@ -65,6 +65,17 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def carry_tokens(sampled: torch.Tensor, src: torch.Tensor, dst: torch.Tensor, ids: torch.Tensor) -> None:
+    """ids[dst[i]] = sampled[src[i]] where src[i] >= 0; all int32 on the device."""
+    _dev(sampled, src, dst, ids)
+    for t, name in ((sampled, "sampled"), (src, "src"), (dst, "dst"), (ids, "ids")):
+        _i32(t, name)
+    if src.shape != dst.shape or src.dim() != 1:
+        raise NativeError(f"carry_tokens: src {tuple(src.shape)} / dst {tuple(dst.shape)}")
+    check(kernels().pa_carry_tokens(_stream(), _ptr(sampled), _ptr(src), _ptr(dst), _ptr(ids), src.shape[0],
+                                    sampled.numel(), ids.numel()))
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None,
             rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """RMSNorm over the last axis of x [T, H] with a float32 weight [H].

@@ -56,24 +56,34 @@ class RequestSampler:
         return float(self._rng.random(dtype=np.float32))
 
 
-def sample_rows(logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
-    """One token id per row of float32 logits [R, V]; row i belongs to samplers[i]."""
+def sample_rows_device(logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> torch.Tensor:
+    """One token id per row of float32 logits [R, V], left on the device as int32 [R]; row i belongs to samplers[i].
+
+    Nothing here waits for the device: the ids can feed the next step where
+    they are (``Engine.step(..., carried=ids)``) and be read by the host later.
+    """
     r = logits.shape[0]
     if r != len(samplers):
         raise ValueError(f"{r} logits rows for {len(samplers)} requests")
     if r == 0:
-        return []
+        return torch.empty(0, dtype=torch.int32, device=logits.device)
     if all(s.params.greedy for s in samplers):
-        return K.argmax(logits).tolist()
-    host = np.empty((3, r), dtype=np.float32)
-    topk = np.zeros(r, dtype=np.int32)
+        return K.argmax(logits)
+    host = torch.empty((3, r), dtype=torch.float32, pin_memory=True)
+    topk = torch.zeros(r, dtype=torch.int32, pin_memory=True)
+    hv, kv = host.numpy(), topk.numpy()
     for i, s in enumerate(samplers):
         p = s.params
-        host[0, i] = 0.0 if p.greedy else p.temperature
+        hv[0, i] = 0.0 if p.greedy else p.temperature
         # top_p outside (0, 1) keeps everything (crates/prelude-core/src/engine/sampling/logits_processor.rs:119-125)
-        host[1, i] = p.top_p
-        host[2, i] = 0.0 if p.greedy else s.next_uniform()
-        topk[i] = p.top_k or 0
-    dev = torch.from_numpy(host).to(logits.device)
-    dk = torch.from_numpy(topk).to(logits.device)
-    return K.sample(logits, dev[0], dk, dev[1], dev[2]).tolist()
+        hv[1, i] = p.top_p
+        hv[2, i] = 0.0 if p.greedy else s.next_uniform()
+        kv[i] = p.top_k or 0
+    dev = host.to(logits.device, non_blocking=True)
+    dk = topk.to(logits.device, non_blocking=True)
+    return K.sample(logits, dev[0], dk, dev[1], dev[2])
+
+
+def sample_rows(logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:
+    """As ``sample_rows_device``, read back: waits for the device."""
+    return sample_rows_device(logits, samplers).tolist()

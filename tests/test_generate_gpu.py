@@ -155,3 +155,42 @@ def test_command_line(gpu, tmp_path):
     assert r.returncode == 0, r.stderr[-2000:]
     recs = [json.loads(l) for l in r.stdout.strip().splitlines()]
     assert len(recs) == 2 and all(1 <= len(x["token_ids"]) <= 4 for x in recs)
+
+
+def test_overlapped_steps_change_no_token(gpu, tmp_path):
+    """Steps launched before the previous step's ids reach the host give the tokens, finish reasons and counts of
+    the loop that waits for every step: with requests ending on EOS, on a stop id and on their length at
+    different times, few pages (evictions), and prompts cut into portions.  In float32, where a row's logits
+    are the same bits whatever else is in its step (the two loops put different requests side by side)."""
+    dtype = "float32"
+    from prelude_amd import LLM
+    from prelude_amd.sampling import SamplingParams
+    from prelude_amd.weights import write_safetensors
+    folder, cfg, w = model_folder("c", dtype)
+    prompts = prompts_for(cfg, [40, 70, 25, 90, 55, 33, 8], 11)
+    write_safetensors(str(tmp_path / "model.safetensors"), w)
+    (tmp_path / "config.json").write_text(json.dumps(dict(cfg, eos_token_id=cfg["vocab_size"] - 1)))
+    probe = LLM(str(tmp_path), dtype=dtype, page_size=8, max_cache_tokens=4096, overlap_steps=False)
+    base = probe.generate(prompts, max_tokens=30, temperature=0.0)
+    del probe
+    # an EOS id that request 0 produces midway, a stop id that request 2 produces (both greedy below)
+    eos, stop = base[0].token_ids[9], base[2].token_ids[14]
+    (tmp_path / "config.json").write_text(json.dumps(dict(cfg, eos_token_id=[eos])))
+    params = [SamplingParams(0.0 if i % 2 == 0 else 0.9, 0.95 if i == 5 else 1.0, 20 if i == 3 else None, 100 + i)
+              for i in range(len(prompts))]
+    runs = []
+    for overlap in (False, True):
+        llm = LLM(str(tmp_path), dtype=dtype, page_size=8, max_cache_tokens=200, decode_reservation_cap=1,
+                  max_num_batched_tokens=48, overlap_steps=overlap)
+        outs = llm.generate(prompts, max_tokens=30, sampling_params=params, stop_token_ids=[stop])
+        assert llm.engine.tables.audit() == "" and llm.engine.tables.num_requests() == 0
+        assert llm.scheduler.num_running == 0 and llm.scheduler.num_waiting == 0
+        runs.append((llm, outs))
+    (sync_llm, sync), (over_llm, over) = runs
+    assert [o.token_ids for o in over] == [o.token_ids for o in sync]
+    assert [o.finish_reason for o in over] == [o.finish_reason for o in sync]
+    assert sync[0].finish_reason == "eos" and sync[2].finish_reason in ("stop", "eos")
+    assert "length" in {o.finish_reason for o in sync}
+    assert all(len(o.token_ids) <= 30 and None not in o.token_ids for o in over)
+    assert sync_llm.scheduler.preemptions > 0 and over_llm.scheduler.preemptions > 0
+    assert over_llm.steps <= sync_llm.steps + 3

@@ -254,3 +254,57 @@ def test_graph_replays_equal_eager_steps(gpu):
     assert eager_eng._graphs is None and graph_eng._graphs.captures == 3 and graph_eng._graphs.replays == 19
     for i, (a, b) in enumerate(zip(eager, graphed)):
         assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
+
+
+@pytest.mark.parametrize("dtype,hip_graph", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
+def test_tokens_carried_on_the_device(gpu, dtype, hip_graph):
+    """A step whose last tokens are taken from a device tensor (the previous step's samples, never read by the
+    host) gives the logits of the step fed the same ids from the host, bit for bit: in decode steps, in a
+    mixed step, and at the end of a prompt portion."""
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    from prelude_amd.engine.engine import StepError
+    folder, cfg, _ = model_folder("b", dtype)
+    seqs = [reference_logits("b", 30 + i, n, dtype)[0] for i, n in enumerate([70, 33, 50])]
+    dev = torch.device("cuda:0")
+
+    def play(carry):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype=dtype, page_size=16, max_cache_tokens=1024,
+                                                         hip_graph=hip_graph))
+        outs, at = [], [0, 0, 0]
+
+        def feed(parts):
+            entries, ids = [], []
+            for r, n in parts:
+                toks = list(seqs[r][at[r]:at[r] + n])
+                at[r] += n
+                if carry:
+                    ids.append(toks[-1])
+                    entries.append(StepEntry(r, toks[:-1] + [0], [n - 1], carry=len(ids) - 1))
+                else:
+                    entries.append(StepEntry(r, toks, [n - 1]))
+            # rows in another order than the entries, with a row nobody takes
+            carried = torch.tensor([7] + ids[::-1], dtype=torch.int32, device=dev) if carry else None
+            for e in entries:
+                if carry:
+                    e.carry = len(ids) - e.carry
+            outs.append(eng.step(entries, carried=carried).cpu())
+        feed([(0, 40), (1, 9)])
+        for _ in range(4):
+            feed([(0, 1), (1, 1)])
+        feed([(2, 30), (0, 1)])
+        for _ in range(3):
+            feed([(1, 1), (2, 1), (0, 1)])
+        return eng, outs
+
+    _, plain = play(False)
+    eng, carried = play(True)
+    for i, (a, b) in enumerate(zip(plain, carried)):
+        assert torch.equal(a, b), f"step {i}: carried ids gave other logits"
+    with pytest.raises(StepError, match="carried"):
+        eng.step([StepEntry(0, [0], [0], carry=0)])
+    with pytest.raises(StepError, match="outside"):
+        eng.step([StepEntry(0, [0], [0], carry=3)], carried=torch.zeros(3, dtype=torch.int32, device=dev))
+    with pytest.raises(StepError, match="int32"):
+        eng.step([StepEntry(0, [0], [0], carry=0)], carried=torch.zeros(3, dtype=torch.int64, device=dev))
+    assert eng.tables.audit() == ""
