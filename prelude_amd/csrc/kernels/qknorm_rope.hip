@@ -18,6 +18,7 @@
 namespace pa {
 
 constexpr int kQkWaves = 4;
+constexpr int kQkGroup = 4;   // heads a wavefront of the wide kernel takes
 constexpr int kMaxHeadDim = 256;
 
 // One wavefront per (token, head) over the nh + 2*nkv heads of a token's row.
@@ -119,6 +120,12 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
 // The same for head_dim 64, 128 or 256 rotated over its whole width: a lane owns EPL = head_dim / 64
 // contiguous elements, read and written as one vector; its rotation partner (element + head_dim / 2)
 // sits in lane ^ 32, so nothing goes through LDS.
+//
+// Units (one wavefront each): ceil(tokens / 8) x nkv groups of eight tokens of one value head, then
+// tokens x groups of kQkGroup query and key heads.  In the transposed value page a token's elements lie
+// page_size apart, but eight tokens whose slots are consecutive and start at a multiple of eight (a run: the usual
+// case inside a prompt portion) lie side by side for every element, so a run is written with one vector store
+// per element by the wavefront in whose group the run starts; tokens outside runs are written one by one.
 template <typename T, int EPL>
 __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
@@ -126,56 +133,120 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
     const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int tokens,
     int nh, int nkv, int page_size, float eps) {
   typedef T vec_t __attribute__((ext_vector_type(EPL)));
+  typedef T run_t __attribute__((ext_vector_type(8)));
   constexpr int hd = EPL * kWave;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int heads = nh + 2 * nkv;
-  const long long unit = (long long)blockIdx.x * kQkWaves + wave;
-  if (unit >= (long long)tokens * heads) return;
-  const int t = (int)(unit / heads), h = (int)(unit % heads);
-  const vec_t xv = *reinterpret_cast<const vec_t*>(qkv + ((size_t)t * heads + h) * hd + lane * EPL);
-  if (h >= nh + nkv) {  // V: a copy into the transposed page
-    const long long slot = slots ? (long long)slots[t] : -1;
-    if (slot < 0) return;
-    const long long page = slot / page_size, off = slot % page_size;
-    T* dst = v_cache + ((size_t)page * nkv + (h - nh - nkv)) * hd * page_size + off;
+  const int qk_heads = nh + nkv;
+  const int head_groups = (qk_heads + kQkGroup - 1) / kQkGroup;
+  const long long qk_units = (long long)tokens * head_groups;
+  const long long v_units = (slots && nkv > 0) ? (long long)((tokens + 7) / 8) * nkv : 0;
+  long long unit = (long long)blockIdx.x * kQkWaves + wave;
+  if (unit < v_units) {  // V first (the longer units): copies into the transposed pages
+    const int group = (int)(unit / nkv), kvh = (int)(unit % nkv);
+    const int t0 = group * 8;
+    // slots of the tokens from seven before the group to seven behind it (the same in every lane: scalar loads)
+    int sl[22];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = xv[e];
+    for (int i = 0; i < 22; ++i) {
+      const int x = t0 - 7 + i;
+      sl[i] = (x >= 0 && x < tokens) ? slots[x] : -2;
+    }
+    // bit i: a run starts at token t0 - 7 + i
+    unsigned starts = 0;
+    if (page_size % 8 == 0) {
+#pragma unroll
+      for (int i = 0; i < 15; ++i) {
+        bool ok = sl[i] >= 0 && (sl[i] & 7) == 0;
+#pragma unroll
+        for (int k = 1; k < 8; ++k) ok = ok && sl[i + k] == sl[i] + k;
+        starts |= (ok ? 1u : 0u) << i;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int x = t0 + j;
+      const int slot = sl[7 + j];
+      if (slot < 0) continue;   // not cached, or beyond the batch
+      const int head = 7 + j - (slot & 7);   // where this token's run would start
+      const bool in_run = (starts >> head) & 1u;
+      if (in_run && (slot & 7)) continue;    // written with its run (by this group or the one before)
+      const size_t page = (size_t)(slot / page_size);
+      const int off = slot % page_size;
+      T* dst = v_cache + (page * nkv + kvh) * hd * page_size + off;
+      if (in_run) {
+        vec_t v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          v[i] = *reinterpret_cast<const vec_t*>(qkv + ((size_t)(x + i) * heads + qk_heads + kvh) * hd + lane * EPL);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          run_t r;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) r[i] = v[i][e];
+          *reinterpret_cast<run_t*>(dst + (size_t)(lane * EPL + e) * page_size) = r;
+        }
+      } else {
+        const vec_t xv = *reinterpret_cast<const vec_t*>(qkv + ((size_t)x * heads + qk_heads + kvh) * hd + lane * EPL);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = xv[e];
+      }
+    }
     return;
   }
-  T* dst;
-  const float* weight;
-  if (h < nh) {
-    dst = q_out + ((size_t)t * nh + h) * hd;
-    weight = q_weight;
-  } else {
-    const long long slot = slots ? (long long)slots[t] : -1;
-    if (slot < 0) return;
-    const long long page = slot / page_size, off = slot % page_size;
-    dst = k_cache + (((size_t)page * nkv + (h - nh)) * page_size + off) * hd;
-    weight = k_weight;
-  }
-  float x[EPL];
-  float ss = 0.f;
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    x[e] = to_f32(xv[e]);
-    ss += x[e] * x[e];
-  }
-  ss = wave_sum(ss);
-  const float inv = rsqrtf(ss / (float)hd + eps);
+  unit -= v_units;
+  if (unit >= qk_units) return;
+  // queries and keys: kQkGroup heads of one token, loaded together so one memory round trip serves them all
+  const int t = (int)(unit / head_groups), h0 = (int)(unit % head_groups) * kQkGroup;
+  const long long slot = slots ? (long long)slots[t] : -1;
   const int pos = positions[t];
   const int j0 = (lane % 32) * EPL;  // index into the cos/sin row
-  const float* c = cos_table + (size_t)pos * (hd / 2) + j0;
-  const float* s = sin_table + (size_t)pos * (hd / 2) + j0;
-  vec_t ov;
+  typedef float rot_t __attribute__((ext_vector_type(EPL)));
+  const rot_t c = *reinterpret_cast<const rot_t*>(cos_table + (size_t)pos * (hd / 2) + j0);
+  const rot_t sn = *reinterpret_cast<const rot_t*>(sin_table + (size_t)pos * (hd / 2) + j0);
+  vec_t xv[kQkGroup];
+#pragma unroll
+  for (int i = 0; i < kQkGroup; ++i)
+    if (h0 + i < qk_heads) xv[i] = *reinterpret_cast<const vec_t*>(qkv + ((size_t)t * heads + h0 + i) * hd + lane * EPL);
+  rot_t qw, kw;
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
-    if (weight) x[e] = x[e] * inv * weight[lane * EPL + e];
-    const float partner = __shfl_xor(x[e], 32, kWave);
-    const float r = lane < 32 ? x[e] * c[e] - partner * s[e] : partner * s[e] + x[e] * c[e];
-    ov[e] = from_f32<T>(r);
+    qw[e] = q_weight ? q_weight[lane * EPL + e] : 1.0f;
+    kw[e] = k_weight ? k_weight[lane * EPL + e] : 1.0f;
   }
-  *reinterpret_cast<vec_t*>(dst + lane * EPL) = ov;
+#pragma unroll
+  for (int i = 0; i < kQkGroup; ++i) {
+    const int h = h0 + i;
+    if (h >= qk_heads) break;
+    T* dst;
+    const bool is_q = h < nh;
+    if (is_q) {
+      dst = q_out + ((size_t)t * nh + h) * hd;
+    } else {
+      if (slot < 0) continue;
+      const long long page = slot / page_size, off = slot % page_size;
+      dst = k_cache + (((size_t)page * nkv + (h - nh)) * page_size + off) * hd;
+    }
+    const bool normed = is_q ? q_weight != nullptr : k_weight != nullptr;
+    float x[EPL];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      x[e] = to_f32(xv[i][e]);
+      ss += x[e] * x[e];
+    }
+    ss = wave_sum(ss);
+    const float inv = rsqrtf(ss / (float)hd + eps);
+    vec_t ov;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      if (normed) x[e] = x[e] * inv * (is_q ? qw[e] : kw[e]);
+      const float partner = __shfl_xor(x[e], 32, kWave);
+      const float r = lane < 32 ? x[e] * c[e] - partner * sn[e] : partner * sn[e] + x[e] * c[e];
+      ov[e] = from_f32<T>(r);
+    }
+    *reinterpret_cast<vec_t*>(dst + lane * EPL) = ov;
+  }
 }
 
 }  // namespace pa
@@ -198,8 +269,11 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
   const unsigned blocks = (unsigned)((units + kQkWaves - 1) / kQkWaves);
   hipStream_t st = (hipStream_t)stream;
   if (rot == hd && rot > 0 && (hd == 64 || hd == 128 || hd == 256) && (dtype == kF32 || dtype == kBF16)) {
+    const long long wide_units =
+        (long long)tokens * ((nh + nkv + kQkGroup - 1) / kQkGroup) + (long long)((tokens + 7) / 8) * nkv;
+    const unsigned wide_blocks = (unsigned)((wide_units + kQkWaves - 1) / kQkWaves);
 #define PA_WIDE(T, EPL)                                                                                             \
-  hipLaunchKernelGGL((qknorm_rope_kv_wide_kernel<T, EPL>), dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const T*)qkv, \
+  hipLaunchKernelGGL((qknorm_rope_kv_wide_kernel<T, EPL>), dim3(wide_blocks), dim3(kQkWaves * kWave), 0, st, (const T*)qkv, \
                      q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)q_out, (T*)k_cache, (T*)v_cache, \
                      tokens, nh, nkv, page_size, eps)
     if (dtype == kF32) {

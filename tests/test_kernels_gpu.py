@@ -83,7 +83,7 @@ def test_rmsnorm_reference_vector(gpu):
 
 # ---- SiLU * up ----------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("tokens,inter", [(3, 9728), (5, 160), (2, 7)])
+@pytest.mark.parametrize("tokens,inter", [(3, 9728), (5, 160), (2, 7), (37, 1000), (4, 12)])
 def test_silu_mul(gpu, dtype, tokens, inter):
     gu = rnd(tokens, 2 * inter, dtype=dtype, scale=3.0)
     ref = pm.silu(gu[:, 0::2].double()) * gu[:, 1::2].double()
@@ -204,6 +204,41 @@ def test_qknorm_rope_kv(gpu, dtype, nh, nkv, hd, rot, norm):
     qonly = qkv[:, : nh * hd].contiguous()
     q2 = K().qknorm_rope_kv(dev(qonly), dev(qw), None, dev(cos), dev(sin), dev(pos), None, None, None, nh, 0, hd, rot, eps)
     assert torch.equal(q2, q)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("page,hd", [(16, 128), (8, 64), (32, 256), (12, 128)])
+def test_value_cache_runs(gpu, dtype, page, hd):
+    """Value pages written in runs of eight tokens (aligned, consecutive slots) and one by one around them:
+    a run that starts in the middle of a group of eight tokens, one broken by an uncached token, one cut off
+    by the end of the batch, slots that run backwards, and a page size that allows no runs."""
+    nh, nkv, eps = 2, 3, 1e-6
+    slot_list = (list(range(32, 40))                # a run: tokens 0..7
+                 + list(range(5, 18))               # 5,6,7 alone; 8..15 a run that starts at token 11; 16,17 alone
+                 + [48, 49, 50, -1, 52, 53, 54, 55]  # broken by a token that is not cached
+                 + list(range(71, 63, -1))          # backwards
+                 + list(range(80, 96))              # two runs back to back
+                 + list(range(104, 109)))           # cut off by the end of the batch
+    t = len(slot_list)
+    pages = 112 // page + 1
+    qkv = rnd(t, (nh + 2 * nkv) * hd, dtype=dtype, scale=2.0)
+    pos = torch.arange(t, dtype=torch.int32)
+    cos, sin = pm.rope_tables(hd, 64, 10000.0, torch.float32)
+    w = 1.0 + 0.1 * rnd(hd, seed=3)
+    kcd = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype, device=gpu)
+    vcd = torch.full((pages, nkv, hd, page), 7.0, dtype=dtype, device=gpu)
+    K().qknorm_rope_kv(qkv.to(gpu), w.to(gpu), w.to(gpu), cos.to(gpu), sin.to(gpu), pos.to(gpu),
+                       torch.tensor(slot_list, dtype=torch.int32, device=gpu), kcd, vcd, nh, nkv, hd, hd, eps)
+    want = torch.full((pages, nkv, hd, page), 7.0, dtype=dtype)
+    v = qkv[:, (nh + nkv) * hd:].reshape(t, nkv, hd)
+    for i, sl in enumerate(slot_list):
+        if sl >= 0:
+            want[sl // page, :, :, sl % page] = v[i]
+    assert torch.equal(vcd.cpu(), want)
+    _, rk, _ = qk_reference(qkv, w, w, cos, sin, pos, nh, nkv, hd, hd, eps)
+    for i, sl in enumerate(slot_list):
+        if sl >= 0:
+            close(kcd[sl // page, :, sl % page], rk[i], dtype)
 
 
 def test_qknorm_rope_refuses_bad_sizes(gpu):
