@@ -24,10 +24,11 @@
 // Operand layout of v_mfma_f32_16x16x32_bf16 (lane l, g = l / 16, r = l % 16):
 //   A[16 x 32]: row r,    columns 8g .. 8g+7        B[32 x 16]: column r, rows 8g .. 8g+7
 //   C[16 x 16]: column r, rows 4g .. 4g+3
-// For 32 keys, two score tiles give lane (g, r) the keys {4g..4g+3} and
-// {16+4g..16+4g+3} of query r; packed in that order they are the B operand of
-// O^T = V^T P^T, whose A operand takes the same eight keys of one head_dim row
-// of V^T: two 8-byte loads.
+// A step takes 32 keys as two score tiles.  Which key a tile's row stands for is
+// free, and is chosen so that lane group g ends up with the scores of the eight
+// consecutive keys 8g .. 8g+7: row 4a + i of tile t is key 8a + 4t + i.  Packed
+// in that order they are the B operand of O^T = V^T P^T, whose A operand is then
+// eight consecutive keys of one head_dim row of V^T: one 16-byte load.
 //
 // Reference counterparts: the FA4 / FlashInfer paged kernels the reference
 // calls (crates/prelude-cuda/src/attn/flash_v4.rs:125-277,
@@ -48,13 +49,25 @@ __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+// Reductions over the four lanes r, r + 16, r + 32, r + 48 (one query column), the result in all four.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second,
+// v_permlane32_swap the upper half of the first with the lower half of the second: given the same value
+// twice, the two results hold a lane's own value and its partner's.
 __device__ __forceinline__ float xor_max16_32(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, kWave));
-  return fmaxf(v, __shfl_xor(v, 32, kWave));
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const unsigned w = __float_as_uint(v);
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float xor_sum16_32(float v) {
-  v += __shfl_xor(v, 16, kWave);
-  return v + __shfl_xor(v, 32, kWave);
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const unsigned w = __float_as_uint(v);
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // What a wavefront keeps per head while it walks keys: per lane, query column r.
@@ -92,13 +105,13 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-// K rows of keys key0 .. key0+31 as A operands.  Keys outside [lo, hi) are read
-// from the nearest key inside (their scores are masked by the caller).
+// K rows of keys key0 .. key0+31 as A operands: row r of tile t is key 8 (r / 4) + 4 t + r % 4.  Keys outside
+// [lo, hi) are read from the nearest key inside (their scores are masked by the caller).
 template <int HD>
 __device__ __forceinline__ void load_k(const KeyWalk& w, int key0, int g, int r, KFrag<HD>& f) {
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    int key = key0 + 16 * t + r;
+    int key = key0 + 8 * (r / 4) + 4 * t + (r % 4);
     key = key < w.lo ? w.lo : (key >= w.hi ? w.hi - 1 : key);
     const int page = w.table[key >> w.page_shift];
     const bf16* row =
@@ -114,10 +127,12 @@ __device__ __forceinline__ void load_k(const KeyWalk& w, int key0, int g, int r,
   }
 }
 
-// Where lane group g finds its eight keys of a 32-key step in V^T: two chunks of four keys, each
-// inside one page (pages hold a multiple of four keys).  p[t] points at head_dim row 0; row d is d pages further.
+// Where lane group g finds its eight keys key0 + 8g .. + 7 of a 32-key step in V^T: two chunks of four keys,
+// each inside one page (pages hold a multiple of four keys), side by side when a page holds eight or more.
+// p[t] points at head_dim row 0; row d is d pages further.
 struct VChunks {
   const bf16* p[2];
+  bool joined;  // p[1] == p[0] + 4: one 16-byte load
 };
 
 template <int HD>
@@ -125,17 +140,19 @@ __device__ __forceinline__ VChunks v_chunks(const KeyWalk& w, int key0, int g) {
   VChunks v;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    int c = key0 + 16 * t + 4 * g;  // first key of the chunk
+    int c = key0 + 8 * g + 4 * t;  // first key of the chunk
     // a chunk wholly outside [lo, hi) is read from the chunk that holds the nearest key inside
     if (c + 3 < w.lo) c = w.lo & ~3;
     if (c >= w.hi) c = (w.hi - 1) & ~3;
     const int page = w.table[c >> w.page_shift];
     v.p[t] = w.vc + ((((size_t)page * w.nkv + w.kvh) * HD) << w.page_shift) + (c & w.page_mask);
   }
+  v.joined = w.page_shift >= 3 && __all(v.p[1] == v.p[0] + 4);
   return v;
 }
 
 __device__ __forceinline__ bf16x8 load_v(const VChunks& v, int d, int page_shift) {
+  if (v.joined) return *reinterpret_cast<const bf16x8*>(v.p[0] + ((size_t)d << page_shift));
   union {
     bf16x8 v8;
     short4_t h[2];
@@ -166,7 +183,7 @@ __device__ __forceinline__ bf16x8 scores32(int key0, int g, const KFrag<HD>& kf,
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (!vis(key0 + 16 * t + 4 * g + i)) s[4 * t + i] = -INFINITY;
+        if (!vis(key0 + 8 * g + 4 * t + i)) s[4 * t + i] = -INFINITY;
   }
   float mx = s[0];
 #pragma unroll
@@ -202,18 +219,13 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool valid, int g, bf16
   }
 }
 
-// One step over 32 keys for GT heads that share the keys: the scores and softmax of every head first, then
-// each V^T tile (asked for at the start of the step, so it arrives under the scores) is used by all heads.
-// An output is rescaled only when some maximum moved.  `kf` holds the step's K rows, loaded a step ahead.
+// The arithmetic of one step over 32 keys for GT heads that share the keys: the scores and softmax of every
+// head first, then each V^T tile is used by all heads.  An output is rescaled only when some maximum moved.
 template <int HD, int GT, typename Visible>
-__device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int r, const KFrag<HD>& kf,
-                                         const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked, HeadState<HD>* st,
-                                         Visible vis) {
+__device__ __forceinline__ void attend32_core(int key0, int g, const KFrag<HD>& kf, const bf16x8* va,
+                                              const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked,
+                                              HeadState<HD>* st, Visible vis) {
   constexpr int OT = HeadState<HD>::OT;
-  const VChunks vch = v_chunks<HD>(w, key0, g);
-  bf16x8 va[OT];
-#pragma unroll
-  for (int t = 0; t < OT; ++t) va[t] = load_v(vch, 16 * t + r, w.page_shift);
   bf16x8 pb[GT];
   float alpha[GT];
   bool rescale[GT];
@@ -223,18 +235,33 @@ __device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int 
     rescale[j] = __any(alpha[j] != 1.0f);
   }
 #pragma unroll
-  for (int t = 0; t < OT; ++t) {
+  for (int j = 0; j < GT; ++j) {
+    if (rescale[j]) {
+      asm volatile("" ::: "memory");  // keep this a branch: as selects it would cost a multiply per output every step
 #pragma unroll
-    for (int j = 0; j < GT; ++j) {
-      f32x4 o = st[j].o[t];
-      if (rescale[j]) {
-        asm volatile("" ::: "memory");  // keep this a branch: as selects it would cost a multiply per output every step
+      for (int t = 0; t < OT; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] *= alpha[j];
-      }
-      st[j].o[t] = mfma16(va[t], pb[j], o);
+        for (int i = 0; i < 4; ++i) st[j].o[t][i] *= alpha[j];
     }
   }
+#pragma unroll
+  for (int t = 0; t < OT; ++t)
+#pragma unroll
+    for (int j = 0; j < GT; ++j) st[j].o[t] = mfma16(va[t], pb[j], st[j].o[t]);
+}
+
+// One step over 32 keys read from the cache: the V^T tiles are asked for at the start of the step, so they
+// arrive under the scores.  `kf` holds the step's K rows, loaded a step ahead.
+template <int HD, int GT, typename Visible>
+__device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int r, const KFrag<HD>& kf,
+                                         const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked, HeadState<HD>* st,
+                                         Visible vis) {
+  constexpr int OT = HeadState<HD>::OT;
+  const VChunks vch = v_chunks<HD>(w, key0, g);
+  bf16x8 va[OT];
+#pragma unroll
+  for (int t = 0; t < OT; ++t) va[t] = load_v(vch, 16 * t + r, w.page_shift);
+  attend32_core<HD, GT>(key0, g, kf, va, qf, c, masked, st, vis);
 }
 
 // ---------------------------------------------------------------------------
@@ -466,6 +493,213 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// prefill with the keys staged in LDS: grid as above; the four wavefronts of a workgroup own 16 tokens each
+// of one 64-token tile and see almost the same keys, so the workgroup reads every block of 64 keys from the
+// cache once (each thread a few 16-byte pieces, a block ahead, into registers), puts it into one of two LDS
+// buffers, and all four take their MFMA operands from there.  One barrier a block.
+//
+// LDS layout: K rows [key][head_dim], the keys of each 32 in the order the score tiles want them (key
+// 8a + 4t + i in row 16t + 4a + i); V^T rows [head_dim][64 keys], keys in their own order.  Rows are padded
+// to 32 bytes past a multiple of 64: measured on gfx950, 16-byte reads of sixteen rows at such a stride run
+// at the full 256 bytes a cycle, and at half that with 16 bytes of padding.
+// ---------------------------------------------------------------------------
+constexpr int kStageKeys = 64;
+
+template <int HD>
+struct StageLds {
+  static constexpr int KROW = (2 * HD + 63) / 64 * 32 + 16;   // elements
+  static constexpr int VROW = kStageKeys + 16;
+  bf16 k[2][kStageKeys][KROW];
+  bf16 v[2][HD][VROW];
+};
+
+// A thread's share of the staging.  Wavefront w takes the 16 keys 16w .. 16w+15 of a block of 64: of K, lane
+// (r = lane % 16, q = lane / 16) takes the 16-byte pieces 4j + q of key 16w + r; of V^T, lane (d = lane / 2,
+// h = lane % 2) takes the eight keys 16w + 8h .. + 7 of the rows d + 32j.  Pages hold 8 to 64 keys here, so a
+// block starts at a page's first key, and a thread reads one page of each cache per block, at places inside
+// the page that never change.  A page outside the pages [lo_page, hi_page] that hold the tile's keys is
+// replaced by the nearest of those; the scores of its keys are masked.
+template <int HD>
+struct Stage {
+  static constexpr int CPK = HD / 8;          // 16-byte pieces per K row
+  static constexpr int NK = (CPK + 3) / 4;
+  static constexpr int NV = (HD + 31) / 32;
+  bf16x8 k[NK];
+  bf16x8 v[NV];
+  int kpage, vpage;
+
+  __device__ __forceinline__ void load_pages(const KeyWalk& w, int key0, int wave, int lane, int lo_page, int hi_page) {
+    int kp = (key0 + 16 * wave + lane % 16) >> w.page_shift;
+    int vp = (key0 + 16 * wave + 8 * (lane % 2)) >> w.page_shift;
+    kp = kp < lo_page ? lo_page : (kp > hi_page ? hi_page : kp);
+    vp = vp < lo_page ? lo_page : (vp > hi_page ? hi_page : vp);
+    kpage = w.table[kp];
+    vpage = w.table[vp];
+  }
+
+  __device__ __forceinline__ void load(const KeyWalk& w, int wave, int lane) {
+    const unsigned page_elems = ((unsigned)w.nkv * HD) << w.page_shift;   // elements per page, all KV heads
+    const unsigned head_off = ((unsigned)w.kvh * HD) << w.page_shift;
+    const int r = lane % 16, q = lane / 16;
+    const bf16* kp = w.kc + ((unsigned long long)(unsigned)kpage * page_elems + head_off +
+                             (unsigned)((16 * wave + r) & w.page_mask) * HD + 8 * q);
+#pragma unroll
+    for (int j = 0; j < NK; ++j)
+      if (CPK % 4 == 0 || 4 * j + q < CPK) k[j] = *reinterpret_cast<const bf16x8*>(kp + 32 * j);
+    const int d = lane / 2, h = lane % 2;
+    const bf16* vp = w.vc + ((unsigned long long)(unsigned)vpage * page_elems + head_off + ((unsigned)d << w.page_shift) +
+                             (unsigned)((16 * wave + 8 * h) & w.page_mask));
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (HD % 32 == 0 || d + 32 * j < HD) v[j] = *reinterpret_cast<const bf16x8*>(vp + ((size_t)(32 * j) << w.page_shift));
+  }
+
+  __device__ __forceinline__ void store(StageLds<HD>& lds, int buf, int wave, int lane) const {
+    const int r = lane % 16, q = lane / 16;
+    const int key = 16 * wave + r;   // 32 s + 8 a + 4 t + i  ->  row 32 s + 16 t + 4 a + i
+    const int row = (key & 32) | ((key & 4) << 2) | ((key & 24) >> 1) | (key & 3);
+#pragma unroll
+    for (int j = 0; j < NK; ++j)
+      if (CPK % 4 == 0 || 4 * j + q < CPK) *reinterpret_cast<bf16x8*>(&lds.k[buf][row][8 * (4 * j + q)]) = k[j];
+    const int d = lane / 2, h = lane % 2;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if (HD % 32 == 0 || d + 32 * j < HD) *reinterpret_cast<bf16x8*>(&lds.v[buf][d + 32 * j][16 * wave + 8 * h]) = v[j];
+  }
+};
+
+// One step over the 32 keys `sub` of the staged block.
+template <int HD, int GT, typename Visible>
+__device__ __forceinline__ void attend32_lds(const StageLds<HD>& lds, int buf, int sub, int key0, int g, int r,
+                                             const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked,
+                                             HeadState<HD>* st, Visible vis) {
+  constexpr int OT = HeadState<HD>::OT;
+  KFrag<HD> kf;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KFrag<HD>::KS; ++ks) {
+      if (HD % 32 == 0 || 32 * ks + 8 * g < HD) {
+        kf.k[t][ks] = *reinterpret_cast<const bf16x8*>(&lds.k[buf][32 * sub + 16 * t + r][32 * ks + 8 * g]);
+      } else {
+        kf.k[t][ks] = zero8();
+      }
+    }
+  bf16x8 va[OT];
+#pragma unroll
+  for (int t = 0; t < OT; ++t) va[t] = *reinterpret_cast<const bf16x8*>(&lds.v[buf][16 * t + r][32 * sub + 8 * g]);
+  attend32_core<HD, GT>(key0, g, kf, va, qf, c, masked, st, vis);
+}
+
+// A 64-token tile from tile0: wavefront `wave` owns its tokens 16 wave .. 16 wave + 15.  Every wavefront takes
+// part in the staging and the barriers, also one whose tokens lie beyond the portion's end.
+template <int HD, int GT>
+__device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* __restrict__ q, bf16* __restrict__ out,
+                                                 const bf16* kc, const bf16* vc, const int* table, int row0, int q_len,
+                                                 int ctx, int tile0, int nh, int nkv, int kvh, int head0, int page_shift,
+                                                 int window, float c, int wave, int g, int r) {
+  constexpr int OT = HD / 16;
+  constexpr int KS = (HD + 31) / 32;
+  const int lane = 16 * g + r;
+  const int start = ctx - q_len;                // position of the portion's first token
+  const int t0 = tile0 + 16 * wave;
+  const bool wave_on = t0 < q_len;
+  const bool qvalid = t0 + r < q_len;
+  const int my_pos = start + t0 + r;            // this lane's query position
+  const int last_valid = t0 + 15 < q_len ? t0 + 15 : q_len - 1;
+  const int last_pos = start + last_valid;
+  const int first_pos = start + t0;
+  const int lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+  const int hi = last_pos + 1;
+  const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+  const int all_lo = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
+  const int all_hi = first_pos + 1;
+  // what the workgroup stages: from the first token's window start to the last valid token of the tile
+  const int wg_first = start + tile0;
+  const int wg_last = start + (tile0 + 63 < q_len ? tile0 + 63 : q_len - 1);
+  const int wg_lo = (window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0;
+  const int wg_hi = wg_last + 1;
+
+  KeyWalk w{kc, vc, table, nkv, kvh, page_shift, (1 << page_shift) - 1, wg_lo, wg_hi};
+  bf16x8 qf[GT][KS];
+  HeadState<HD> st[GT];
+#pragma unroll
+  for (int j = 0; j < GT; ++j)
+    load_q<HD>(q + ((size_t)(row0 + (qvalid ? t0 + r : 0)) * nh + head0 + j) * HD, qvalid, g, qf[j]);
+
+  Stage<HD> stage;
+  const int lo_page = wg_lo >> page_shift, hi_page = (wg_hi - 1) >> page_shift;
+  int key0 = (wg_lo / kStageKeys) * kStageKeys;
+  stage.load_pages(w, key0, wave, lane, lo_page, hi_page);
+  stage.load(w, wave, lane);
+  if (key0 + kStageKeys < wg_hi) stage.load_pages(w, key0 + kStageKeys, wave, lane, lo_page, hi_page);
+  int buf = 0;
+  for (; key0 < wg_hi; key0 += kStageKeys, buf ^= 1) {
+    stage.store(lds, buf, wave, lane);
+    __syncthreads();
+    if (key0 + kStageKeys < wg_hi) {
+      stage.load(w, wave, lane);   // the next block, from the pages looked up a block ago
+      if (key0 + 2 * kStageKeys < wg_hi)
+        stage.load_pages(w, key0 + 2 * kStageKeys, wave, lane, lo_page, hi_page);  // and the pages of the one after
+    }
+    if (wave_on) {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const int k32 = key0 + 32 * sub;
+        if (k32 + 32 <= lo || k32 >= hi) continue;
+        const bool masked = k32 < all_lo || k32 + 32 > all_hi;
+        attend32_lds<HD, GT>(lds, buf, sub, k32, g, r, qf, c, masked, st,
+                             [&](int key) { return key >= my_lo && key <= my_pos; });
+      }
+    }
+  }
+  __syncthreads();  // the buffers are free for the next tile
+  if (!qvalid) return;
+#pragma unroll
+  for (int j = 0; j < GT; ++j) {
+    const float inv = 1.0f / xor_sum16_32(st[j].l);
+    bf16* orow = out + ((size_t)(row0 + t0 + r) * nh + head0 + j) * HD;
+#pragma unroll
+    for (int t = 0; t < OT; ++t) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(st[j].o[t][i] * inv);
+      *reinterpret_cast<bf16x4*>(orow + 16 * t + 4 * g) = v;
+    }
+  }
+}
+
+template <int HD, int GT>
+__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
+    int page_shift, int window, float c, int paired) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  StageLds<HD>& lds = *reinterpret_cast<StageLds<HD>*>(lds_raw);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int group = nh / nkv;
+  const int hgroups = group / GT;
+  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int seq = seq_ids[blockIdx.z];
+  const int row0 = cu_q[seq];
+  const int q_len = cu_q[seq + 1] - row0;
+  const int ctx = context_lens[seq];
+  const int tiles = (q_len + 63) / 64;
+  const int first = paired ? (int)blockIdx.x : tiles - 1 - (int)blockIdx.x;
+  const int second = paired ? tiles - 1 - (int)blockIdx.x : first;
+  if (first > second || first < 0) return;   // the same for the whole workgroup
+  const int* table = block_table + (size_t)seq * table_stride;
+  const int head0 = kvh * group + hg * GT;
+  prefill_tile_lds<HD, GT>(lds, q, out, kc, vc, table, row0, q_len, ctx, second * 64, nh, nkv, kvh, head0, page_shift,
+                           window, c, wave, g, r);   // the long one first
+  if (first != second)
+    prefill_tile_lds<HD, GT>(lds, q, out, kc, vc, table, row0, q_len, ctx, first * 64, nh, nkv, kvh, head0, page_shift,
+                             window, c, wave, g, r);
+}
+
+// ---------------------------------------------------------------------------
 template <int HD>
 int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
@@ -496,6 +730,20 @@ int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void*
   static const char* env = getenv("PA_PREFILL_PAIRED");
   const int paired = env ? atoi(env) : (tiles >= 2 && wgs > 0 ? 1 : 0);
   dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / GT), nseq);
+  static const char* lds_env = getenv("PA_PREFILL_LDS");
+  const bool staged = page_shift >= 3 && page_shift <= 6 && (lds_env ? atoi(lds_env) != 0 : true);
+  if (staged) {
+    // the two buffers are more than the 64 KB a kernel may declare: asked for at launch, allowed once per kernel
+    static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_lds_kernel<HD, GT>),
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                          (int)sizeof(StageLds<HD>));
+    if (allowed != hipSuccess)
+      return pa::fail("attn_prefill: %zu bytes of LDS refused: %s", sizeof(StageLds<HD>), hipGetErrorString(allowed));
+    hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, GT>), grid, dim3(256), sizeof(StageLds<HD>), st, (const bf16*)q,
+                       (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens,
+                       (bf16*)out, nh, nkv, page_shift, window, scale * kLog2e, paired);
+    return check_launch("attn_prefill");
+  }
   hipLaunchKernelGGL((attn_prefill_kernel<HD, GT>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kc,
                      (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, nh, nkv,
                      page_shift, window, scale * kLog2e, paired);
@@ -510,8 +758,10 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
                                    max_q_len, nh, nkv, page_shift, window, scale)
-  if (HD <= 64 && group % 4 == 0) PA_GT(4);  // wider heads would not fit four heads' state in 256 registers
-  if (group % 2 == 0) PA_GT(2);
+  static const char* gt_env = getenv("PA_PREFILL_GT");
+  const int gt_max = gt_env ? atoi(gt_env) : 4;
+  if (HD <= 64 && group % 4 == 0 && gt_max >= 4) PA_GT(4);  // wider heads would not fit four heads' state in 256 registers
+  if (group % 2 == 0 && gt_max >= 2) PA_GT(2);
   PA_GT(1);
 #undef PA_GT
 }
