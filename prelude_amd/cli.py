@@ -40,6 +40,8 @@ def build_parser() -> argparse.ArgumentParser:
     g = ap.add_mutually_exclusive_group()
     g.add_argument("--cuda-graph", "--hip-graph", dest="hip_graph", action="store_true", default=True)
     g.add_argument("--no-cuda-graph", "--no-hip-graph", dest="hip_graph", action="store_false")
+    g.add_argument("--no-weight-tiles", dest="weight_tiles", action="store_false", default=True,
+                   help="keep no second, tiled copy of the weights for decode steps (saves their memory)")
     g.add_argument("--no-overlap-steps", dest="overlap_steps", action="store_false", default=True,
                    help="wait for every step's token ids before scheduling the next step")
     # the request
@@ -89,7 +91,7 @@ def main(argv=None) -> int:
                        max_running_requests=args.max_running_requests, max_total_tokens=args.max_total_tokens,
                        decode_reservation_cap=args.decode_reservation_cap,
                        decode_priority_max_remaining_tokens=args.decode_priority_max_remaining_tokens,
-                       hip_graph=args.hip_graph, overlap_steps=args.overlap_steps)
+                       hip_graph=args.hip_graph, overlap_steps=args.overlap_steps, weight_tiles=args.weight_tiles)
     llm = LLM(model, config=cfg)
     prompts = list(args.prompt)
     prompts += [[int(x) for x in s.split(",") if x.strip()] for s in args.prompt_ids]

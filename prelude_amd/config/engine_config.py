@@ -29,6 +29,9 @@ class EngineConfig:
     # decode steps replayed from HIP graphs
     hip_graph: bool = True
     hip_graph_max_bs: int = 64
+    # a second copy of every bfloat16 weight matrix, in the tiles the few-row product streams fastest
+    # (decode steps run about a tenth faster for twice the weight memory)
+    weight_tiles: bool = True
     # launch a step before the previous step's token ids have reached the host (they are handed on
     # on the device); a request that ends on a token value then runs one step too many, which is dropped
     overlap_steps: bool = True

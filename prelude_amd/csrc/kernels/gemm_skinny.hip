@@ -60,7 +60,21 @@ enum Epilogue : int { kPlain = 0, kSiluMul = 1 };
 
 // NT tiles of 16 rows of W per workgroup: with two, every X fragment serves two products, which halves the
 // share of the loads that X makes up (X comes from L2, but the loads cost the same as any).
-template <int MT, int NT, int WAVES, typename TC, int EPI>
+// A fragment of a weight stored in tiles (see pa_pack_tiles): the wavefront's 64 lanes read 1 KB side by side.
+__device__ __forceinline__ Frag load_tiled(const bf16* tile, int step, int lane, bool ok) {
+  Frag f;
+  if (ok) {
+    const bf16* p = tile + (size_t)step * 1024 + lane * 8;
+    f.lo = *reinterpret_cast<const bf16x8*>(p);
+    f.hi = *reinterpret_cast<const bf16x8*>(p + 512);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f.lo[i] = f.hi[i] = (bf16)0.f;
+  }
+  return f;
+}
+
+template <int MT, int NT, int WAVES, typename TC, int EPI, bool TILED>
 __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                    const bf16* __restrict__ w,
                                                                    const float* __restrict__ bias,
@@ -76,8 +90,9 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
   const bf16* wrow[NT];
 #pragma unroll
   for (int u = 0; u < NT; ++u) {
-    n_ok[u] = n0 + 16 * u + r < n;
-    wrow[u] = w + (size_t)(n_ok[u] ? n0 + 16 * u + r : 0) * k + 16 * g;
+    n_ok[u] = TILED ? n0 + 16 * u < n : n0 + 16 * u + r < n;
+    wrow[u] = TILED ? w + (size_t)(n_ok[u] ? n0 / 16 + u : 0) * steps * 1024
+                    : w + (size_t)(n_ok[u] ? n0 + 16 * u + r : 0) * k + 16 * g;
   }
   const bf16* xrow[MT];
   bool m_ok[MT];
@@ -100,7 +115,9 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
   for (int d = 0; d < kDepth; ++d) {
     const int s = wave + d * WAVES;
 #pragma unroll
-    for (int u = 0; u < NT; ++u) wbuf[d][u] = load_frag(wrow[u], s * 64, kk, n_ok[u] && s < steps);
+    for (int u = 0; u < NT; ++u)
+      wbuf[d][u] = TILED ? load_tiled(wrow[u], s, lane, n_ok[u] && s < steps)
+                         : load_frag(wrow[u], s * 64, kk, n_ok[u] && s < steps);
 #pragma unroll
     for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
   }
@@ -114,7 +131,9 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
       for (int t = 0; t < MT; ++t) xc[t] = xbuf[d][t];
       const int next = s0 + (d + kDepth) * WAVES;
 #pragma unroll
-      for (int u = 0; u < NT; ++u) wbuf[d][u] = load_frag(wrow[u], next * 64, kk, n_ok[u] && next < steps);
+      for (int u = 0; u < NT; ++u)
+        wbuf[d][u] = TILED ? load_tiled(wrow[u], next, lane, n_ok[u] && next < steps)
+                           : load_frag(wrow[u], next * 64, kk, n_ok[u] && next < steps);
 #pragma unroll
       for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
 #pragma unroll
@@ -187,14 +206,14 @@ static void skinny_shape(int n, int k, int mt, int* nt, int* waves) {
   *waves = w;
 }
 
-template <int MT, typename TC, int EPI>
+template <int MT, typename TC, int EPI, bool TILED>
 int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
                   long ldx, long ldc) {
   int nt, waves;
   skinny_shape(n, k, MT, &nt, &waves);
   dim3 grid(((n + 15) / 16 + nt - 1) / nt);
 #define PA_W(NT, WV)                                                                                            \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
                      (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc)
 #define PA_WAVES(NT)            \
   switch (waves) {              \
@@ -216,13 +235,30 @@ int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bia
 
 template <typename TC, int EPI>
 int launch_skinny_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                     long ldx, long ldc) {
+                     long ldx, long ldc, int tiled) {
+  if (tiled) return launch_skinny<1, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
   switch ((m + 15) / 16) {
-    case 1: return launch_skinny<1, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
-    case 2: return launch_skinny<2, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
-    case 3: return launch_skinny<3, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
-    default: return launch_skinny<4, TC, EPI>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    case 1: return launch_skinny<1, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    case 2: return launch_skinny<2, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    case 3: return launch_skinny<3, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    default: return launch_skinny<4, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
   }
+}
+
+__global__ void pack_tiles_kernel(const bf16* __restrict__ w, bf16* __restrict__ out, int n, int k, int steps,
+                                  long total) {
+  const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;   // piece [tile][step][half][g][r]
+  if (p >= total) return;
+  const int r = p % 16, g = (p / 16) % 4, half = (p / 64) % 2;
+  const long ts = p / 128;
+  const int step = ts % steps;
+  const long tile = ts / steps;
+  const long row = 16 * tile + r;
+  const int col = 64 * step + 16 * g + 8 * half;
+  bf16x8 v;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (row < n && col + j < k) ? w[row * k + col + j] : (bf16)0.f;
+  *reinterpret_cast<bf16x8*>(out + p * 8) = v;
 }
 
 }  // namespace pa
@@ -230,8 +266,21 @@ int launch_skinny_mt(hipStream_t st, const void* x, const void* w, const float* 
 using namespace pa;
 
 // epilogue 0: C[m, n] (+ bias); 1: C[m, n/2] = silu(gate) * up over a weight whose rows alternate gate_j, up_j.
+// out[tile][step][half][g][r][j] = w[16 tile + r][64 step + 16 g + 8 half + j], zero beyond n and k: every
+// fragment a wavefront of the product kernel loads is then 1 KB of consecutive memory, and a workgroup's tile
+// one run of ceil(k / 64) * 2 KB.  `out` holds ceil(n / 16) * ceil(k / 64) * 1024 elements.
+extern "C" int pa_pack_tiles(void* stream, const void* w, void* out, int n, int k) {
+  PA_REQUIRE(n > 0 && k > 0, "pack_tiles: bad sizes n=%d k=%d", n, k);
+  const long tiles = (n + 15) / 16, steps = (k + 63) / 64;
+  const long total = tiles * steps * 128;   // 16-byte pieces
+  hipLaunchKernelGGL(pack_tiles_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16*)w, (bf16*)out, n, k, (int)steps, total);
+  return check_launch("pack_tiles");
+}
+
+// tiled 1: w is the weight in tiles (pa_pack_tiles), and m <= 16.
 extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w,
-                              const float* bias, void* c, int m, int n, int k, long ldx, long ldc) {
+                              const float* bias, void* c, int m, int n, int k, long ldx, long ldc, int tiled) {
   if (m == 0 || n == 0) return 0;
   PA_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_skinny: bad sizes m=%d n=%d k=%d", m, n, k);
   PA_REQUIRE(m <= kSkinnyMaxM, "gemm_skinny: %d rows exceed %d", m, kSkinnyMaxM);
@@ -239,10 +288,13 @@ extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const v
   PA_REQUIRE(ldx >= k, "gemm_skinny: row stride %ld is smaller than k=%d", ldx, k);
   PA_REQUIRE(epilogue == kPlain || (n % 2 == 0 && !bias), "gemm_skinny: the SiLU*up epilogue needs an even n and no bias");
   PA_REQUIRE(ldc >= (epilogue == kSiluMul ? n / 2 : n), "gemm_skinny: output row stride %ld is too small", ldc);
+  PA_REQUIRE(!tiled || m <= 16, "gemm_skinny: a tiled weight takes at most 16 rows, not %d", m);
   hipStream_t st = (hipStream_t)stream;
-  if (epilogue == kPlain && out_dtype == kBF16) return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc);
-  if (epilogue == kPlain && out_dtype == kF32) return launch_skinny_mt<float, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  if (epilogue == kPlain && out_dtype == kBF16)
+    return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);
+  if (epilogue == kPlain && out_dtype == kF32)
+    return launch_skinny_mt<float, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);
   if (epilogue == kSiluMul && out_dtype == kBF16)
-    return launch_skinny_mt<bf16, kSiluMul>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    return launch_skinny_mt<bf16, kSiluMul>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);
   return pa::fail("gemm_skinny: unsupported output type %d with epilogue %d", out_dtype, epilogue);
 }

@@ -110,6 +110,8 @@ class Engine:
         model = CausalLM(arch.build_spec(arch.parse_config(raw)))
         device = torch.device(config.device)
         torch.cuda.set_device(device)
+        from ..ops import kernels as K
+        K.set_weight_tiles(config.weight_tiles)
         load_into(model, model_dir, config.torch_dtype(), device)
         return cls(model, config, raw)
 

@@ -214,15 +214,68 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
 SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel itself takes up to 64)
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+class TiledWeight:
+    """A bfloat16 weight [n, k] laid out in the tiles the weight-streaming kernel reads (``pack_tiles``)."""
+
+    def __init__(self, data: torch.Tensor, n: int, k: int):
+        self.data, self.n, self.k = data, n, k
+        self.shape = (n, k)
+        self.dtype, self.device = data.dtype, data.device
+
+
+def pack_tiles(w: torch.Tensor) -> TiledWeight:
+    """The weight in tiles of 16 rows x 64 columns, each stored in the order a wavefront's lanes load it."""
+    _dev(w)
+    if w.dim() != 2 or w.dtype != torch.bfloat16:
+        raise NativeError(f"pack_tiles: w {tuple(w.shape)} {w.dtype}")
+    n, k = w.shape
+    out = torch.empty(((n + 15) // 16) * ((k + 63) // 64) * 1024, dtype=torch.bfloat16, device=w.device)
+    check(kernels().pa_pack_tiles(_stream(), _ptr(w), _ptr(out), n, k))
+    return TiledWeight(out, n, k)
+
+
+WEIGHT_TILES = True   # keep a tiled copy of bfloat16 weights for products of few rows (``set_weight_tiles``)
+
+
+def set_weight_tiles(on: bool) -> None:
+    """Whether ``prepare_weight`` adds the tiled copy (a second copy of the weight in device memory)."""
+    global WEIGHT_TILES
+    WEIGHT_TILES = bool(on)
+
+
+class LinearWeight:
+    """A matrix [out, in] as the products read it: by rows for many-row products (the library's) and the
+    32-bit path, and, for bfloat16, in tiles for the weight-streaming product of few rows."""
+
+    def __init__(self, rows: torch.Tensor, tiles: Optional[TiledWeight] = None):
+        self.rows, self.tiles = rows, tiles
+        self.shape, self.dtype, self.device = tuple(rows.shape), rows.dtype, rows.device
+
+    def first_rows(self, n: int) -> torch.Tensor:
+        """The first n outputs as a plain matrix (a view)."""
+        return self.rows[:n]
+
+
+def prepare_weight(w: torch.Tensor) -> LinearWeight:
+    """What a part keeps of a weight it multiplies by: called once when weights are loaded."""
+    tiles = None
+    if WEIGHT_TILES and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2:
+        tiles = pack_tiles(w.contiguous())
+    return LinearWeight(w, tiles)
+
+
+def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False) -> torch.Tensor:
     """x [M <= 64, K] @ w[N, K]^T in bfloat16 on the matrix cores, streaming w once.
 
-    With ``silu_mul_epilogue`` the rows of w alternate gate_j, up_j and the
+    ``w`` is a tensor [N, K] or a ``TiledWeight`` (then M <= 16).  With
+    ``silu_mul_epilogue`` the rows of w alternate gate_j, up_j and the
     result is silu(gate) * up, [M, N/2]."""
-    _dev(x, w, bias)
+    tiled = isinstance(w, TiledWeight)
+    wt = w.data if tiled else w
+    _dev(x, wt, bias)
     _f32(bias, "bias")
-    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+    if x.dim() != 2 or len(w.shape) != 2 or x.shape[1] != w.shape[1] or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise NativeError(f"gemm_skinny: x {tuple(x.shape)} {x.dtype} / w {tuple(w.shape)} {w.dtype}")
     m, k = x.shape
     n = w.shape[0]
@@ -231,23 +284,26 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
         raise NativeError(f"gemm_skinny: bias {tuple(bias.shape)} is not [{n}]")
     cols = n // 2 if silu_mul_epilogue else n
     out = torch.empty((m, cols), dtype=out_dtype, device=x.device)
-    check(kernels().pa_gemm_skinny(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w),
-                                   _ptr(bias), _ptr(out), m, n, k, k, cols))
+    check(kernels().pa_gemm_skinny(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(wt),
+                                   _ptr(bias), _ptr(out), m, n, k, k, cols, 1 if tiled else 0))
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """y = x W^T (+ b), W [out, in].  float32: our own true 32-bit product.
-    bfloat16: up to 64 rows our weight-streaming kernel, above that the library
-    product; 32-bit accumulation in both."""
+    """y = x W^T (+ b), W [out, in] as a tensor or a ``LinearWeight``.  float32: our own true 32-bit product.
+    bfloat16: few rows our weight-streaming kernel (from the tiled copy if the weight has one), above that the
+    library product; 32-bit accumulation in both."""
+    tiles = None
+    if isinstance(w, LinearWeight):
+        w, tiles = w.rows, w.tiles
     if x.dtype == torch.float32:
         return gemm_plain(x, w, bias, out_dtype)
     _dev(x, w, bias)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise NativeError(f"linear: x {x.dtype} / w {w.dtype}")
     if x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0:
-        return gemm_skinny(x, w, bias, out_dtype)
+        return gemm_skinny(x, tiles if tiles is not None and x.shape[0] <= 16 else w, bias, out_dtype)
     y = torch.matmul(x, w.t())
     if bias is not None:
         add_bias_(y, bias)
@@ -262,9 +318,11 @@ def set_skinny_max_rows(n: int) -> None:
     SKINNY_MAX_ROWS = max(0, min(int(n), 64))
 
 
-def linear_silu_mul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) for a weight [2I, K] whose rows alternate gate_j, up_j."""
     if x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0:
+        if isinstance(w, LinearWeight):
+            w = w.tiles if w.tiles is not None and x.shape[0] <= 16 else w.rows
         return gemm_skinny(x, w, silu_mul_epilogue=True)
     return silu_mul(linear(x, w))
 

@@ -61,9 +61,9 @@ class GQAAttention(Mixer):
         return t
 
     def load(self, tensors, dtype, device):
-        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]],
-                               dim=0).contiguous()
-        self.w_o = tensors["o_proj.weight"]
+        self.w_qkv = K.prepare_weight(torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
+                                                 tensors["v_proj.weight"]], dim=0).contiguous())
+        self.w_o = K.prepare_weight(tensors["o_proj.weight"])
         if self.bias:
             self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
             self.b_o = tensors["o_proj.bias"]
@@ -81,7 +81,7 @@ class GQAAttention(Mixer):
                                  nh, nkv, hd, self.rotary_dim, self.norm_eps)
         else:  # reads keys and values another layer wrote: only the queries are projected
             bq = self.b_qkv[: nh * hd] if self.b_qkv is not None else None
-            qx = K.linear(x, self.w_qkv[: nh * hd], bq)
+            qx = K.linear(x, self.w_qkv.first_rows(nh * hd), bq)
             q = K.qknorm_rope_kv(qx, self.q_norm, None, cos, sin, step.positions, None, None, None, nh, 0, hd,
                                  self.rotary_dim, self.norm_eps)
         o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale)

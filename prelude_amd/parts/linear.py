@@ -38,7 +38,7 @@ class LinearHead(Part):
         return {"weight": TensorReq((self.vocab_size, self.hidden_size), MATRIX)}
 
     def load(self, tensors, dtype, device):
-        self.weight = tensors["weight"]
+        self.weight = K.prepare_weight(tensors["weight"])
 
     def forward(self, hidden_rows: torch.Tensor) -> torch.Tensor:
         return K.linear(hidden_rows, self.weight, out_dtype=torch.float32)

@@ -30,8 +30,9 @@ class GatedMLP(FeedForward):
 
     def load(self, tensors, dtype, device):
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
-        self.gate_up = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
-        self.down = tensors["down_proj.weight"]
+        self.gate_up = K.prepare_weight(
+            torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous())
+        self.down = K.prepare_weight(tensors["down_proj.weight"])
 
     def forward(self, x):
         return K.linear(K.linear_silu_mul(x, self.gate_up), self.down)

@@ -139,6 +139,34 @@ def test_gemm_skinny(gpu, m, n, k):
         act = K().gemm_skinny(xd, wd, silu_mul_epilogue=True)
         close(act, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
         close(K().linear_silu_mul(xd, wd), pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
+    # the weight in tiles: the same sums in the same order, so the same bits (few rows only)
+    tiles = K().pack_tiles(wd)
+    if m <= 16:
+        assert torch.equal(K().gemm_skinny(xd, tiles, out_dtype=torch.float32), full)
+        assert torch.equal(K().gemm_skinny(xd, tiles, b.to(gpu)), K().gemm_skinny(xd, wd, b.to(gpu)))
+        lw = K().LinearWeight(wd, tiles)
+        assert torch.equal(K().linear(xd, lw, out_dtype=torch.float32), full)
+        if n % 2 == 0:
+            assert torch.equal(K().gemm_skinny(xd, tiles, silu_mul_epilogue=True), act)
+            assert torch.equal(K().linear_silu_mul(xd, lw), act)
+    else:
+        from prelude_amd._native import NativeError
+        with pytest.raises(NativeError, match="at most 16 rows"):
+            K().gemm_skinny(xd, tiles)
+        close(K().linear(xd, K().LinearWeight(wd, tiles)), ref, torch.bfloat16)   # more rows: from the row-major copy
+
+
+def test_pack_tiles_layout(gpu):
+    """out[tile][step][half][g][r][j] = w[16 tile + r][64 step + 16 g + 8 half + j], zeros beyond the matrix."""
+    n, k = 40, 200
+    w = torch.arange(n * k, dtype=torch.float32).reshape(n, k).remainder(251.0).to(torch.bfloat16)
+    t = K().pack_tiles(w.to(gpu))
+    assert (t.n, t.k) == (n, k) and t.data.numel() == 3 * 4 * 1024
+    got = t.data.cpu().reshape(3, 4, 2, 4, 16, 8)
+    pad = torch.zeros(48, 256, dtype=torch.bfloat16)
+    pad[:n, :k] = w
+    want = pad.reshape(3, 16, 4, 4, 2, 8).permute(0, 2, 4, 3, 1, 5)   # [tile, r, step, g, half, j] -> [tile, step, half, g, r, j]
+    assert torch.equal(got, want)
 
 
 def test_gemm_skinny_refuses(gpu):
