@@ -29,10 +29,13 @@
 #include "common.h"
 #include "api.h"
 
+#include <stdio.h>
+#include <stdlib.h>
+
 namespace pa {
 
 constexpr int kSkinnyMaxM = 64;
-constexpr int kDepth = 2;  // k-steps of loads a wavefront keeps in flight (4 measured slower: the memory system thrashes)
+constexpr int kDepth = 2;  // k-steps of loads a wavefront keeps in flight from a row-major weight
 
 struct Frag {
   bf16x8 lo, hi;
@@ -74,7 +77,7 @@ __device__ __forceinline__ Frag load_tiled(const bf16* tile, int step, int lane,
   return f;
 }
 
-template <int MT, int NT, int WAVES, typename TC, int EPI, bool TILED>
+template <int MT, int NT, int WAVES, typename TC, int EPI, bool TILED, int DEPTH>
 __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                    const bf16* __restrict__ w,
                                                                    const float* __restrict__ bias,
@@ -107,12 +110,12 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // kDepth k-steps in flight per wavefront: a ring of fragments, refilled as soon as a slot has been used.
+  // DEPTH k-steps in flight per wavefront: a ring of fragments, refilled as soon as a slot has been used.
   // Steps past the end load zeros, so the ring needs no tail handling.
   const int kk = k - 16 * g;
-  Frag wbuf[kDepth][NT], xbuf[kDepth][MT];
+  Frag wbuf[DEPTH][NT], xbuf[DEPTH][MT];
 #pragma unroll
-  for (int d = 0; d < kDepth; ++d) {
+  for (int d = 0; d < DEPTH; ++d) {
     const int s = wave + d * WAVES;
 #pragma unroll
     for (int u = 0; u < NT; ++u)
@@ -121,15 +124,15 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
     for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
   }
-  for (int s0 = wave; s0 < steps; s0 += WAVES * kDepth) {
+  for (int s0 = wave; s0 < steps; s0 += WAVES * DEPTH) {
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
+    for (int d = 0; d < DEPTH; ++d) {
       Frag wc[NT], xc[MT];
 #pragma unroll
       for (int u = 0; u < NT; ++u) wc[u] = wbuf[d][u];
 #pragma unroll
       for (int t = 0; t < MT; ++t) xc[t] = xbuf[d][t];
-      const int next = s0 + (d + kDepth) * WAVES;
+      const int next = s0 + (d + DEPTH) * WAVES;
 #pragma unroll
       for (int u = 0; u < NT; ++u)
         wbuf[d][u] = TILED ? load_tiled(wrow[u], next, lane, n_ok[u] && next < steps)
@@ -194,26 +197,37 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
   }
 }
 
-// Shape of the launch for an [n, k] weight: tiles of 16 rows per workgroup and wavefronts per workgroup.
-// Wide weights take two tiles; then about 3000 wavefronts on the chip, each with at least two k-steps.
-// Depends on the weight's shape only, never on the batch.
-static void skinny_shape(int n, int k, int mt, int* nt, int* waves) {
+// Shape of the launch for an [n, k] weight: tiles of 16 rows per workgroup, wavefronts per workgroup, k-steps
+// of loads a wavefront keeps in flight.  Row-major: wide weights take two tiles; then about 3000 wavefronts on
+// the chip, each with at least two k-steps.  Depends on the weight's shape and layout only, never on the batch.
+static void skinny_shape(int n, int k, int mt, bool tiled, int* nt, int* waves, int* depth) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
+  if (tiled) {
+    // measured over (tiles per workgroup, wavefronts, depth) at the shapes of a 4B model: one step in flight per
+    // wavefront streams a tiled weight best; long rows want 16 wavefronts, the widest weights two tiles
+    *nt = tiles >= 4096 ? 2 : 1;
+    *waves = steps >= 128 ? 16 : 8;
+    *depth = 1;
+    static const char* env = getenv("PA_SKINNY_SHAPE");   // "nt,waves,depth": for measurements
+    if (env) sscanf(env, "%d,%d,%d", nt, waves, depth);
+    return;
+  }
   *nt = mt > 1 ? 1 : (tiles >= 4096 ? 4 : (tiles >= 768 ? 2 : 1));
   const int wgs = (tiles + *nt - 1) / *nt;
   int w = 4;
   while (w < 16 && wgs * w < 3000 && steps / (2 * w) >= 2) w *= 2;
   *waves = w;
+  *depth = kDepth;
 }
 
-template <int MT, typename TC, int EPI, bool TILED>
-int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
+template <int MT, typename TC, int EPI, bool TILED, int DEPTH>
+int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
                   long ldx, long ldc) {
-  int nt, waves;
-  skinny_shape(n, k, MT, &nt, &waves);
+  int nt, waves, depth;
+  skinny_shape(n, k, MT, TILED, &nt, &waves, &depth);
   dim3 grid(((n + 15) / 16 + nt - 1) / nt);
 #define PA_W(NT, WV)                                                                                            \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED, DEPTH>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
                      (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc)
 #define PA_WAVES(NT)            \
   switch (waves) {              \
@@ -231,6 +245,17 @@ int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bia
 #undef PA_WAVES
 #undef PA_W
   return check_launch("gemm_skinny");
+}
+
+template <int MT, typename TC, int EPI, bool TILED>
+int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
+                  long ldx, long ldc) {
+  if (TILED) {
+    int nt, waves, depth;
+    skinny_shape(n, k, MT, TILED, &nt, &waves, &depth);
+    if (depth == 1) return launch_skinny_depth<MT, TC, EPI, TILED, 1>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  }
+  return launch_skinny_depth<MT, TC, EPI, TILED, kDepth>(st, x, w, bias, c, m, n, k, ldx, ldc);
 }
 
 template <typename TC, int EPI>
