@@ -121,7 +121,7 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
 // contiguous elements, read and written as one vector; its rotation partner (element + head_dim / 2)
 // sits in lane ^ 32, so nothing goes through LDS.
 //
-// Units (one wavefront each): ceil(tokens / 8) x nkv groups of eight tokens of one value head, then
+// Units (one wavefront each): ceil(tokens / vgroup) x nkv groups of vgroup (1 or 8) tokens of one value head, then
 // tokens x groups of kQkGroup query and key heads.  In the transposed value page a token's elements lie
 // page_size apart, but eight tokens whose slots are consecutive and start at a multiple of eight (a run: the usual
 // case inside a prompt portion) lie side by side for every element, so a run is written with one vector store
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, const int* __restrict__ positions,
     const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int tokens,
-    int nh, int nkv, int page_size, float eps) {
+    int nh, int nkv, int page_size, float eps, int vgroup) {
   typedef T vec_t __attribute__((ext_vector_type(EPL)));
   typedef T run_t __attribute__((ext_vector_type(8)));
   constexpr int hd = EPL * kWave;
@@ -140,8 +140,18 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
   const int qk_heads = nh + nkv;
   const int head_groups = (qk_heads + kQkGroup - 1) / kQkGroup;
   const long long qk_units = (long long)tokens * head_groups;
-  const long long v_units = (slots && nkv > 0) ? (long long)((tokens + 7) / 8) * nkv : 0;
+  const long long v_units = (slots && nkv > 0) ? (long long)((tokens + vgroup - 1) / vgroup) * nkv : 0;
   long long unit = (long long)blockIdx.x * kQkWaves + wave;
+  if (unit < v_units && vgroup == 1) {  // few tokens (decode steps): a wavefront per token and value head
+    const int x = (int)(unit / nkv), kvh = (int)(unit % nkv);
+    const int slot = slots[x];
+    if (slot < 0) return;
+    const vec_t xv = *reinterpret_cast<const vec_t*>(qkv + ((size_t)x * heads + qk_heads + kvh) * hd + lane * EPL);
+    T* dst = v_cache + ((size_t)(slot / page_size) * nkv + kvh) * hd * page_size + slot % page_size;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = xv[e];
+    return;
+  }
   if (unit < v_units) {  // V first (the longer units): copies into the transposed pages
     const int group = (int)(unit / nkv), kvh = (int)(unit % nkv);
     const int t0 = group * 8;
@@ -269,13 +279,14 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
   const unsigned blocks = (unsigned)((units + kQkWaves - 1) / kQkWaves);
   hipStream_t st = (hipStream_t)stream;
   if (rot == hd && rot > 0 && (hd == 64 || hd == 128 || hd == 256) && (dtype == kF32 || dtype == kBF16)) {
+    const int vgroup = tokens >= 64 ? 8 : 1;   // runs of eight tokens pay only in prompt portions
     const long long wide_units =
-        (long long)tokens * ((nh + nkv + kQkGroup - 1) / kQkGroup) + (long long)((tokens + 7) / 8) * nkv;
+        (long long)tokens * ((nh + nkv + kQkGroup - 1) / kQkGroup) + (long long)((tokens + vgroup - 1) / vgroup) * nkv;
     const unsigned wide_blocks = (unsigned)((wide_units + kQkWaves - 1) / kQkWaves);
 #define PA_WIDE(T, EPL)                                                                                             \
   hipLaunchKernelGGL((qknorm_rope_kv_wide_kernel<T, EPL>), dim3(wide_blocks), dim3(kQkWaves * kWave), 0, st, (const T*)qkv, \
                      q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)q_out, (T*)k_cache, (T*)v_cache, \
-                     tokens, nh, nkv, page_size, eps)
+                     tokens, nh, nkv, page_size, eps, vgroup)
     if (dtype == kF32) {
       if (hd == 64) PA_WIDE(float, 1);
       else if (hd == 128) PA_WIDE(float, 2);

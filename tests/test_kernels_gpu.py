@@ -249,12 +249,14 @@ def test_value_cache_runs(gpu, dtype, page, hd):
                  + [48, 49, 50, -1, 52, 53, 54, 55]  # broken by a token that is not cached
                  + list(range(71, 63, -1))          # backwards
                  + list(range(80, 96))              # two runs back to back
+                 + [110, 96, 97, 98, 99, 111, 109, 100]   # scattered (and enough tokens for the kernel to look for runs)
                  + list(range(104, 109)))           # cut off by the end of the batch
     t = len(slot_list)
+    assert t >= 64
     pages = 112 // page + 1
     qkv = rnd(t, (nh + 2 * nkv) * hd, dtype=dtype, scale=2.0)
     pos = torch.arange(t, dtype=torch.int32)
-    cos, sin = pm.rope_tables(hd, 64, 10000.0, torch.float32)
+    cos, sin = pm.rope_tables(hd, 128, 10000.0, torch.float32)
     w = 1.0 + 0.1 * rnd(hd, seed=3)
     kcd = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype, device=gpu)
     vcd = torch.full((pages, nkv, hd, page), 7.0, dtype=dtype, device=gpu)
