@@ -353,52 +353,58 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   }
 }
 
-// Merges the splits of one (sequence, head): grid (nh, sequences), one wavefront.  Lanes first take a split
-// each (maximum and weights), then a head_dim column each; the sums run over the splits in order.
+// Merges the splits of one (sequence, head): grid (nh, sequences), a thread per head_dim column.  Every
+// wavefront keeps a split per lane (maximum, weight), sixteen splits' outputs are asked for before the weights
+// are known, and the sums run over the splits in order.
 template <int HD>
-__global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* __restrict__ part_o,
-                                                                  const float* __restrict__ part_ml,
-                                                                  const int* __restrict__ seq_ids,
-                                                                  const int* __restrict__ cu_q,
-                                                                  const int* __restrict__ context_lens,
-                                                                  bf16* __restrict__ out, int nh, int window,
-                                                                  int split_keys, int max_splits) {
-  __shared__ float weight[1024];
+__global__ __launch_bounds__((HD + kWave - 1) / kWave* kWave) void attn_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int window,
+    int split_keys, int max_splits) {
+  constexpr int kBatch = 16;
   const int h = blockIdx.x;
   const int seq = seq_ids[blockIdx.y];
   const int ctx = context_lens[seq];
+  const size_t token = cu_q[seq];
   const int pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int nsplit = (ctx + split_keys - 1) / split_keys - lo / split_keys;
   if (nsplit == 1) return;  // written by the first kernel
-  const int lane = threadIdx.x;
+  const int d = threadIdx.x, lane = threadIdx.x % kWave;
+  const bool col = d < HD;
   const size_t base = ((size_t)blockIdx.y * nh + h) * max_splits;
+  const float* po = part_o + base * HD + (col ? d : 0);
+  // the first batch of outputs, on its way while the weights are worked out
+  float o[kBatch];
+#pragma unroll
+  for (int i = 0; i < kBatch; ++i) o[i] = (col && i < nsplit) ? po[(size_t)i * HD] : 0.f;
   float mm = -INFINITY;
   for (int s = lane; s < nsplit; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
   mm = wave_max(mm);
-  float l = 0.f;
-  for (int s0 = 0; s0 < nsplit; s0 += kWave) {   // in order of the splits
+  float acc = 0.f, l = 0.f;
+  for (int s0 = 0; s0 < nsplit; s0 += kWave) {   // a split per lane; in order of the splits
     const int s = s0 + lane;
     float f = 0.f, ls = 0.f;
     if (s < nsplit) {
       f = exp2f(part_ml[(base + s) * 2] - mm);
       ls = part_ml[(base + s) * 2 + 1] * f;
-      if (s < 1024) weight[s] = f;
     }
     l += wave_sum(ls);
-  }
-  __syncthreads();
-  const size_t token = cu_q[seq];
-  const float inv = 1.0f / l;
-  for (int d = lane; d < HD; d += kWave) {
-    float o = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < nsplit; ++s) {
-      const float f = s < 1024 ? weight[s] : exp2f(part_ml[(base + s) * 2] - mm);
-      o += part_o[(base + s) * HD + d] * f;
+    const int count = nsplit - s0 < kWave ? nsplit - s0 : kWave;
+    for (int b0 = 0; b0 < count; b0 += kBatch) {
+      if (s0 + b0 > 0) {
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) o[i] = (col && b0 + i < count) ? po[(size_t)(s0 + b0 + i) * HD] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        // the index is the same in every lane: a read of one lane's register, no exchange
+        const float fi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), b0 + i < kWave ? b0 + i : 0));
+        if (b0 + i < count) acc += o[i] * fi;
+      }
     }
-    out[(token * nh + h) * HD + d] = (bf16)(o * inv);
   }
+  if (col) out[(token * nh + h) * HD + d] = (bf16)(acc / l);
 }
 
 // ---------------------------------------------------------------------------
@@ -712,8 +718,8 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
                      part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits);
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
-    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(kWave), 0, st, part_o, part_ml,
-                       seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys, max_splits);
+    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3((HD + kWave - 1) / kWave * kWave), 0, st,
+                       part_o, part_ml, seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys, max_splits);
     return check_launch("attn_decode_merge");
   }
   return 0;
