@@ -269,13 +269,106 @@ __device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int 
 // ---------------------------------------------------------------------------
 constexpr int kDecodeWaves = 4;
 
+// What the decode kernel needs to take the merged QKV projection as it leaves the product instead of queries
+// that have been through the QK-norm + RoPE kernel: it norms and rotates its own queries, and the workgroup
+// whose split holds the token's own position first norms, rotates and writes the token's key and copies its
+// value into the cache (the kernel of qknorm_rope.hip, for one token and KV head).
+struct FusedQkv {
+  const bf16* qkv;          // [tokens, (nh + 2 nkv) * head_dim]
+  const float* q_weight;    // may be null: no norm
+  const float* k_weight;
+  const float* cos_table;   // [positions, head_dim / 2]
+  const float* sin_table;
+  const int* positions;
+  const int* slots;
+  float eps;
+};
+
 template <int HD>
+__device__ __forceinline__ void fused_write_kv(const FusedQkv& f, bf16* kc, bf16* vc, size_t token, int heads, int nh,
+                                               int nkv, int kvh, int page_shift, int lane) {
+  constexpr int EPL = HD / kWave;   // 64 -> 1, 128 -> 2: a lane's elements; its rotation partner is lane ^ 32
+  typedef bf16 vec_t __attribute__((ext_vector_type(EPL)));
+  const int slot = f.slots[token];
+  if (slot < 0) return;
+  const int page = slot >> page_shift, off = slot & ((1 << page_shift) - 1);
+  const bf16* krow = f.qkv + (token * heads + nh + kvh) * HD;
+  const bf16* vrow = f.qkv + (token * heads + nh + nkv + kvh) * HD;
+  const vec_t kv = *reinterpret_cast<const vec_t*>(krow + lane * EPL);
+  const vec_t vv = *reinterpret_cast<const vec_t*>(vrow + lane * EPL);
+  bf16* vdst = vc + ((((size_t)page * nkv + kvh) * HD) << page_shift) + off;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) vdst[(size_t)(lane * EPL + e) << page_shift] = vv[e];
+  float x[EPL], ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    x[e] = (float)kv[e];
+    ss += x[e] * x[e];
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / (float)HD + f.eps);
+  const int pos = f.positions[token];
+  const int j0 = (lane % 32) * EPL;
+  vec_t ov;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    if (f.k_weight) x[e] = x[e] * inv * f.k_weight[lane * EPL + e];
+    const float partner = __shfl_xor(x[e], 32, kWave);
+    const float cs = f.cos_table[(size_t)pos * (HD / 2) + j0 + e], sn = f.sin_table[(size_t)pos * (HD / 2) + j0 + e];
+    ov[e] = (bf16)(lane < 32 ? x[e] * cs - partner * sn : partner * sn + x[e] * cs);
+  }
+  bf16* kdst = kc + ((((size_t)page * nkv + kvh) << page_shift) + off) * HD;
+  *reinterpret_cast<vec_t*>(kdst + lane * EPL) = ov;
+}
+
+// Q^T of one head as B operands from the raw projection: normed and rotated in the lane.  Lane (g, r) holds
+// head_dim 32 ks + 8g .. + 7 of its head; the element head_dim / 2 further on, its rotation partner, is in
+// the same lane (ks + KS / 2), and the sum of squares runs over the lane's elements and the four lane groups.
+template <int HD>
+__device__ __forceinline__ void fused_load_q(const FusedQkv& f, const bf16* qrow, bool valid, int pos, int g, bf16x8* qf) {
+  constexpr int KS = HD / 32;
+  static_assert(HD == 64 || HD == 128, "the rotation partner must sit in the same lane");
+  float x[KS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    bf16x8 raw = zero8();
+    if (valid) raw = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      x[ks][j] = (float)raw[j];
+      ss += x[ks][j] * x[ks][j];
+    }
+  }
+  ss = xor_sum16_32(ss);
+  const float inv = rsqrtf(ss / (float)HD + f.eps);
+#pragma unroll
+  for (int ks = 0; ks < KS / 2; ++ks) {
+    const int d = 32 * ks + 8 * g;   // the first-half element; its partner is d + HD / 2
+    bf16x8 lo, hi;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float a = x[ks][j], b = x[ks + KS / 2][j];
+      if (f.q_weight) {
+        a = a * inv * f.q_weight[d + j];
+        b = b * inv * f.q_weight[d + HD / 2 + j];
+      }
+      const float cs = f.cos_table[(size_t)pos * (HD / 2) + d + j], sn = f.sin_table[(size_t)pos * (HD / 2) + d + j];
+      lo[j] = (bf16)(a * cs - b * sn);
+      hi[j] = (bf16)(a * sn + b * cs);
+    }
+    qf[ks] = lo;
+    qf[ks + KS / 2] = hi;
+  }
+}
+
+template <int HD, bool FUSED>
 __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const bf16* __restrict__ q, const bf16* kc, const bf16* vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
     float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_shift, int window, float c,
-    int split_keys, int max_splits) {
+    int split_keys, int max_splits, FusedQkv fq) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
   __shared__ float lds_o[kDecodeWaves][16][HD + 1];
@@ -301,7 +394,17 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   const bool qvalid = qt * 16 + r < group;
   const size_t token = cu_q[seq];
   bf16x8 qf[1][KS];
-  load_q<HD>(q + (token * nh + (qvalid ? head : 0)) * HD, qvalid, g, qf[0]);
+  if constexpr (FUSED) {
+    const int heads = nh + 2 * nkv;
+    fused_load_q<HD>(fq, fq.qkv + (token * heads + (qvalid ? head : 0)) * HD, qvalid, fq.positions[token], g, qf[0]);
+    if ((int)blockIdx.x == nsplit - 1) {   // the split that holds the token's own position: its key and value first
+      if (wave == 0)
+        fused_write_kv<HD>(fq, const_cast<bf16*>(kc), const_cast<bf16*>(vc), token, heads, nh, nkv, kvh, page_shift, lane);
+      __syncthreads();   // the other wavefronts read them from the cache below
+    }
+  } else {
+    load_q<HD>(q + (token * nh + (qvalid ? head : 0)) * HD, qvalid, g, qf[0]);
+  }
 
   HeadState<HD> st[1];
   const int step0 = (sp * split_keys) / 32;  // splits start at multiples of 32 keys
@@ -706,16 +809,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(
 }
 
 // ---------------------------------------------------------------------------
-template <int HD>
+template <int HD, bool FUSED>
 int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                   float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_shift, int window, float scale,
-                  int split_keys, int max_splits) {
+                  int split_keys, int max_splits, const FusedQkv& fq) {
   const int qtiles = (nh / nkv + 15) / 16;
   dim3 grid(max_splits, nkv * qtiles, nseq);
-  hipLaunchKernelGGL(attn_decode_kernel<HD>, grid, dim3(kDecodeWaves * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
-                     (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                     part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits);
+  hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED>), grid, dim3(kDecodeWaves * kWave), 0, st, (const bf16*)q,
+                     (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens,
+                     (bf16*)out, part_o, part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits,
+                     fq);
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
     hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3((HD + kWave - 1) / kWave * kWave), 0, st,
@@ -821,11 +925,48 @@ extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const
   float* part_o = workspace;
   float* part_ml = workspace ? workspace + (size_t)nseq * nh * max_splits * hd : nullptr;
 #define PA_CALL(HD)                                                                                                  \
-  return launch_decode<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                           out, part_o, part_ml, nseq, nh, nkv, __builtin_ctz(page_size), window, scale, split_keys,   \
-                           max_splits)
+  return launch_decode<HD, false>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q,         \
+                                  context_lens, out, part_o, part_ml, nseq, nh, nkv, __builtin_ctz(page_size), window, \
+                                  scale, split_keys, max_splits, FusedQkv{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
+}
+
+// 1 if pa_attn_decode_fused takes these sizes: whole-width rotation of a head_dim whose half is a multiple of
+// 32, and all query heads of a KV head in one tile (two workgroups must not wait for one another's key).
+extern "C" int pa_attn_decode_fused_supports(int nh, int nkv, int hd, int rot, int page_size) {
+  return (hd == 64 || hd == 128) && rot == hd && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16 &&
+         pa_attn_mfma_supports(hd, page_size);
+}
+
+// pa_qknorm_rope_kv and pa_attn_decode in one: `qkv` is the merged projection [tokens, (nh + 2 nkv) * hd] of a
+// step in which the sequences `seq_ids` feed one token each; their keys and values are written to the caches
+// at `slots` and their outputs to `out`.  Tokens of other sequences are not touched.
+extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* q_weight, const float* k_weight,
+                                    const float* cos_table, const float* sin_table, const int* positions,
+                                    const int* slots, float eps, void* kc, void* vc, const int* block_table,
+                                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                                    void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
+                                    int window, float scale, int split_keys, int max_splits) {
+  if (nseq == 0) return 0;
+  if (int rc = check_common("attn_decode_fused", nseq, nh, nkv, page_size, table_stride, window)) return rc;
+  PA_REQUIRE(pa_attn_decode_fused_supports(nh, nkv, hd, hd, page_size), "attn_decode_fused: nh=%d nkv=%d head_dim=%d page=%d are not taken",
+             nh, nkv, hd, page_size);
+  PA_REQUIRE(qkv && cos_table && sin_table && positions && slots && kc && vc, "attn_decode_fused: a null operand");
+  PA_REQUIRE(split_keys >= 32 && split_keys % 32 == 0, "attn_decode_fused: split of %d keys is not a multiple of 32", split_keys);
+  PA_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attn_decode_fused: %d splits", max_splits);
+  PA_REQUIRE(max_splits == 1 || workspace, "attn_decode_fused: no workspace for %d splits", max_splits);
+  float* part_o = workspace;
+  float* part_ml = workspace ? workspace + (size_t)nseq * nh * max_splits * hd : nullptr;
+  const FusedQkv fq{(const bf16*)qkv, q_weight, k_weight, cos_table, sin_table, positions, slots, eps};
+  const int shift = __builtin_ctz(page_size);
+  if (hd == 64)
+    return launch_decode<64, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,
+                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, split_keys,
+                                   max_splits, fq);
+  return launch_decode<128, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,
+                                  context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, split_keys,
+                                  max_splits, fq);
 }
 
 extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,

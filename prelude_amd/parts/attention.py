@@ -70,11 +70,28 @@ class GQAAttention(Mixer):
         if self.qk_norm:
             self.q_norm, self.k_norm = tensors["q_norm.weight"], tensors["k_norm.weight"]
 
+    FUSED_DECODE_MAX_SEQS = 8   # measured: +3 % tokens a second at batch 1, +1 % at 8, -5 % at 64
+
+    def _fused_decode(self, x, step, cache) -> bool:
+        """Few sequences, each feeding one token: a kernel less per layer counts for more than the norm and the
+        rotation that every workgroup of the attention kernel then does for itself."""
+        return (x.dtype == torch.bfloat16 and self.rope is not None and step.decode_seqs is not None
+                and step.n_prefill == 0 and step.n_decode == step.num_seqs <= self.FUSED_DECODE_MAX_SEQS
+                and K.attention_decode_fused_supported(self.num_heads, self.num_kv_heads, self.head_dim,
+                                                       self.rotary_dim, cache.k.shape[2]))
+
     def forward(self, x, step, cache, write_cache=True):
         nh, nkv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         g = step.kv[cache.group]
         cos = self.rope.cos if self.rope is not None else None
         sin = self.rope.sin if self.rope is not None else None
+        if write_cache and self._fused_decode(x, step, cache):
+            # a step of single tokens: the norm, the rotation and the cache write happen inside the attention kernel
+            qkv = K.linear(x, self.w_qkv, self.b_qkv)
+            o = K.attention_decode_fused(qkv, self.q_norm, self.k_norm, cos, sin, step.positions, g.slots, self.norm_eps,
+                                         cache.k, cache.v, g.block_table, step.decode_seqs, step.cu_q, step.context_lens,
+                                         nh, step.max_decode_context, self.window, self.scale)
+            return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o)
         if write_cache:
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
             q = K.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, cos, sin, step.positions, g.slots, cache.k, cache.v,

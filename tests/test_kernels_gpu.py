@@ -435,6 +435,71 @@ def test_mfma_attention_batch_and_page_independence(gpu):
     assert torch.equal(one, other)                               # other page size, other pages
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window,norm", [(32, 8, 128, 16, 0, True), (8, 8, 64, 8, 0, True), (16, 1, 128, 64, 40, True),
+                                                        (4, 2, 64, 16, 0, False)])
+def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, window, norm):
+    """QK-norm, rotation, cache write and split attention in one kernel against the two kernels one after the
+    other: the same outputs and the same keys and values in the cache, for contexts that end at a page's first
+    and last place and at a split's edge; sequences outside the list are left alone."""
+    eps = 1e-6
+    ctxs = [1, 17, 256, 257, 700, 33, 512]             # 33: a sequence that is not in the list
+    listed = [0, 1, 2, 3, 4, 6]
+    t = len(ctxs)
+    g = torch.Generator().manual_seed(3)
+    total_pages = sum(-(-c // page) for c in ctxs) + 2
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    stride = max(-(-c // page) for c in ctxs)
+    table = torch.full((t, stride), -1, dtype=torch.int32)
+    kc = torch.zeros(total_pages, nkv, page, hd, dtype=torch.bfloat16)
+    vc = torch.zeros(total_pages, nkv, hd, page, dtype=torch.bfloat16)
+    slots = []
+    for i, c in enumerate(ctxs):
+        for p in range(-(-c // page)):
+            table[i, p] = perm.pop()
+        hist = c - 1                                   # keys before the token's own
+        for pos in range(hist):
+            ph = int(table[i, pos // page])
+            kc[ph, :, pos % page] = torch.randn(nkv, hd, generator=g).to(torch.bfloat16)
+            vc[ph, :, :, pos % page] = torch.randn(nkv, hd, generator=g).to(torch.bfloat16)
+        slots.append(int(table[i, (c - 1) // page]) * page + (c - 1) % page)
+    qkv = (2.0 * torch.randn(t, (nh + 2 * nkv) * hd, generator=g)).to(torch.bfloat16)
+    qw = (1.0 + 0.2 * rnd(hd, seed=1)) if norm else None
+    kw = (1.0 + 0.2 * rnd(hd, seed=2)) if norm else None
+    cos, sin = pm.rope_tables(hd, 1024, 10000.0, torch.float32)
+    dev = lambda x: None if x is None else x.to(gpu)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    pos, sl, seqs, cu, cl = i32([c - 1 for c in ctxs]), i32(slots), i32(listed), i32(list(range(t + 1))), i32(ctxs)
+    scale = 1.0 / math.sqrt(hd)
+    assert K().attention_decode_fused_supported(nh, nkv, hd, hd, page)
+    # the two kernels
+    k1, v1 = kc.to(gpu), vc.to(gpu)
+    q = K().qknorm_rope_kv(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), pos, sl, k1, v1, nh, nkv, hd, hd, eps)
+    out1 = torch.zeros(t, nh, hd, dtype=torch.bfloat16, device=gpu)
+    K().attention_decode(q, k1, v1, dev(table), seqs, cu, cl, out1, max(ctxs), window, scale)
+    # the one kernel
+    k2, v2 = kc.to(gpu), vc.to(gpu)
+    out2 = K().attention_decode_fused(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), pos, sl, eps, k2, v2, dev(table),
+                                      seqs, cu, cl, nh, max(ctxs), window, scale)
+    for i in listed:
+        close(out2[i], out1[i].double().cpu(), torch.bfloat16)
+        ph, off = slots[i] // page, slots[i] % page
+        assert torch.equal(v2[ph, :, :, off], v1[ph, :, :, off])
+        close(k2[ph, :, off], k1[ph, :, off].double().cpu(), torch.bfloat16)
+    # the sequence that was not listed: its key and value were not written
+    ph, off = slots[5] // page, slots[5] % page
+    assert float(k2[ph, :, off].abs().max()) == 0.0 and float(v2[ph, :, :, off].abs().max()) == 0.0
+    # nothing else in the caches changed
+    mask = torch.ones(total_pages, page, dtype=torch.bool)
+    for i in listed:
+        mask[slots[i] // page, slots[i] % page] = False
+    assert torch.equal(k2.cpu()[mask[:, None, :].expand(total_pages, nkv, page)], kc[mask[:, None, :].expand(total_pages, nkv, page)])
+    assert torch.equal(v2.cpu().transpose(2, 3)[mask[:, None, :].expand(total_pages, nkv, page)],
+                       vc.transpose(2, 3)[mask[:, None, :].expand(total_pages, nkv, page)])
+    assert not K().attention_decode_fused_supported(nh, nkv, hd, hd // 2, page)      # partial rotation
+    assert not K().attention_decode_fused_supported(34, 2, 128, 128, 16)             # more than 16 heads per KV head
+    assert not K().attention_decode_fused_supported(4, 2, 96, 96, 16)
+
+
 def test_mfma_attention_refuses_what_it_does_not_take(gpu):
     from prelude_amd._native import NativeError
     assert K().mfma_attention_supported(128, 16) and K().mfma_attention_supported(48, 8)
