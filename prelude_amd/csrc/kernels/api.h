@@ -65,7 +65,7 @@ int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, 
 // pa_qknorm_rope_kv + pa_attn_decode in one kernel for steps of single tokens: takes the merged projection,
 // norms and rotates the queries in place of loading them, and writes each token's key and value first.
 int pa_attn_decode_fused(void* stream, const void* qkv, const float* q_weight, const float* k_weight,
-                         const float* cos_table, const float* sin_table, const int* positions, const int* slots, float eps,
+                         const float* cos_table, const float* sin_table, const int* slots, float eps,
                          void* kc, void* vc, const int* block_table, int table_stride, const int* seq_ids, const int* cu_q,
                          const int* context_lens, void* out, float* workspace, int nseq, int nh, int nkv, int hd,
                          int page_size, int window, float scale, int split_keys, int max_splits);

@@ -279,14 +279,13 @@ struct FusedQkv {
   const float* k_weight;
   const float* cos_table;   // [positions, head_dim / 2]
   const float* sin_table;
-  const int* positions;
   const int* slots;
   float eps;
 };
 
 template <int HD>
-__device__ __forceinline__ void fused_write_kv(const FusedQkv& f, bf16* kc, bf16* vc, size_t token, int heads, int nh,
-                                               int nkv, int kvh, int page_shift, int lane) {
+__device__ __forceinline__ void fused_write_kv(const FusedQkv& f, bf16* kc, bf16* vc, size_t token, int pos, int heads,
+                                               int nh, int nkv, int kvh, int page_shift, int lane) {
   constexpr int EPL = HD / kWave;   // 64 -> 1, 128 -> 2: a lane's elements; its rotation partner is lane ^ 32
   typedef bf16 vec_t __attribute__((ext_vector_type(EPL)));
   const int slot = f.slots[token];
@@ -307,7 +306,6 @@ __device__ __forceinline__ void fused_write_kv(const FusedQkv& f, bf16* kc, bf16
   }
   ss = wave_sum(ss);
   const float inv = rsqrtf(ss / (float)HD + f.eps);
-  const int pos = f.positions[token];
   const int j0 = (lane % 32) * EPL;
   vec_t ov;
 #pragma unroll
@@ -396,10 +394,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   bf16x8 qf[1][KS];
   if constexpr (FUSED) {
     const int heads = nh + 2 * nkv;
-    fused_load_q<HD>(fq, fq.qkv + (token * heads + (qvalid ? head : 0)) * HD, qvalid, fq.positions[token], g, qf[0]);
+    // a sequence that feeds one token feeds the one at its last position: no need to wait for positions[token]
+    fused_load_q<HD>(fq, fq.qkv + (token * heads + (qvalid ? head : 0)) * HD, qvalid, pos, g, qf[0]);
     if ((int)blockIdx.x == nsplit - 1) {   // the split that holds the token's own position: its key and value first
       if (wave == 0)
-        fused_write_kv<HD>(fq, const_cast<bf16*>(kc), const_cast<bf16*>(vc), token, heads, nh, nkv, kvh, page_shift, lane);
+        fused_write_kv<HD>(fq, const_cast<bf16*>(kc), const_cast<bf16*>(vc), token, pos, heads, nh, nkv, kvh, page_shift,
+                           lane);
       __syncthreads();   // the other wavefronts read them from the cache below
     }
   } else {
@@ -941,10 +941,10 @@ extern "C" int pa_attn_decode_fused_supports(int nh, int nkv, int hd, int rot, i
 
 // pa_qknorm_rope_kv and pa_attn_decode in one: `qkv` is the merged projection [tokens, (nh + 2 nkv) * hd] of a
 // step in which the sequences `seq_ids` feed one token each; their keys and values are written to the caches
-// at `slots` and their outputs to `out`.  Tokens of other sequences are not touched.
+// at `slots` and their outputs to `out`; a token's position is its sequence's context length less one.  Tokens
+// of other sequences are not touched.
 extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* q_weight, const float* k_weight,
-                                    const float* cos_table, const float* sin_table, const int* positions,
-                                    const int* slots, float eps, void* kc, void* vc, const int* block_table,
+                                    const float* cos_table, const float* sin_table, const int* slots, float eps, void* kc, void* vc, const int* block_table,
                                     int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                                     void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
                                     int window, float scale, int split_keys, int max_splits) {
@@ -952,13 +952,13 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
   if (int rc = check_common("attn_decode_fused", nseq, nh, nkv, page_size, table_stride, window)) return rc;
   PA_REQUIRE(pa_attn_decode_fused_supports(nh, nkv, hd, hd, page_size), "attn_decode_fused: nh=%d nkv=%d head_dim=%d page=%d are not taken",
              nh, nkv, hd, page_size);
-  PA_REQUIRE(qkv && cos_table && sin_table && positions && slots && kc && vc, "attn_decode_fused: a null operand");
+  PA_REQUIRE(qkv && cos_table && sin_table && slots && kc && vc, "attn_decode_fused: a null operand");
   PA_REQUIRE(split_keys >= 32 && split_keys % 32 == 0, "attn_decode_fused: split of %d keys is not a multiple of 32", split_keys);
   PA_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attn_decode_fused: %d splits", max_splits);
   PA_REQUIRE(max_splits == 1 || workspace, "attn_decode_fused: no workspace for %d splits", max_splits);
   float* part_o = workspace;
   float* part_ml = workspace ? workspace + (size_t)nseq * nh * max_splits * hd : nullptr;
-  const FusedQkv fq{(const bf16*)qkv, q_weight, k_weight, cos_table, sin_table, positions, slots, eps};
+  const FusedQkv fq{(const bf16*)qkv, q_weight, k_weight, cos_table, sin_table, slots, eps};
   const int shift = __builtin_ctz(page_size);
   if (hd == 64)
     return launch_decode<64, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,

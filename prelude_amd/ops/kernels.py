@@ -395,13 +395,13 @@ def attention_decode_fused_supported(nh: int, nkv: int, hd: int, rot: int, page_
     return bool(kernels().pa_attn_decode_fused_supports(int(nh), int(nkv), int(hd), int(rot), int(page_size)))
 
 
-def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, positions, slots, eps: float, k_cache, v_cache,
+def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float, k_cache, v_cache,
                            block_table, seq_ids, cu_q, context_lens, nh: int, max_context: int, window: int,
                            scale: float) -> torch.Tensor:
     """``qknorm_rope_kv`` and ``attention_decode`` in one kernel, for a step in which every sequence feeds one
     token: takes the merged projection [T, (nh + 2 nkv) * hd], writes the tokens' keys and values into the caches
-    and returns the attention output [T, nh, hd]."""
-    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens)
+    and returns the attention output [T, nh, hd].  A token's position is its sequence's context length less one."""
+    _dev(qkv, q_weight, k_weight, cos, sin, slots, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens)
     nkv, page, hd = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     _check_caches(k_cache, v_cache, nkv, hd, torch.bfloat16, "attention_decode_fused")
     t = qkv.shape[0]
@@ -411,10 +411,9 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, positions, slots, 
     _f32(k_weight, "k_weight")
     _f32(cos, "cos")
     _f32(sin, "sin")
-    _i32(positions, "positions")
     _i32(slots, "slots")
-    if cos.shape[1] != hd // 2 or sin.shape != cos.shape or positions.shape[0] != t or slots.shape[0] != t:
-        raise NativeError("attention_decode_fused: rotary tables, positions or slots do not match the tokens")
+    if cos.shape[1] != hd // 2 or sin.shape != cos.shape or slots.shape[0] != t:
+        raise NativeError("attention_decode_fused: rotary tables or slots do not match the tokens")
     out = torch.empty((t, nh, hd), dtype=torch.bfloat16, device=qkv.device)
     n = seq_ids.shape[0]
     if n == 0:
@@ -424,7 +423,7 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, positions, slots, 
     words = kernels().pa_attn_decode_workspace(n, nh, hd, max_splits)
     ws = torch.empty((max(words, 1),), dtype=torch.float32, device=qkv.device)
     check(kernels().pa_attn_decode_fused(_stream(), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin),
-                                         _ptr(positions), _ptr(slots), float(eps), _ptr(k_cache), _ptr(v_cache),
+                                         _ptr(slots), float(eps), _ptr(k_cache), _ptr(v_cache),
                                          _ptr(block_table), block_table.shape[1], _ptr(seq_ids), _ptr(cu_q),
                                          _ptr(context_lens), _ptr(out), _ptr(ws), n, nh, nkv, hd, page, int(window),
                                          float(scale), DECODE_SPLIT_KEYS, max_splits))

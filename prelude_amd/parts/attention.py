@@ -88,7 +88,7 @@ class GQAAttention(Mixer):
         if write_cache and self._fused_decode(x, step, cache):
             # a step of single tokens: the norm, the rotation and the cache write happen inside the attention kernel
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
-            o = K.attention_decode_fused(qkv, self.q_norm, self.k_norm, cos, sin, step.positions, g.slots, self.norm_eps,
+            o = K.attention_decode_fused(qkv, self.q_norm, self.k_norm, cos, sin, g.slots, self.norm_eps,
                                          cache.k, cache.v, g.block_table, step.decode_seqs, step.cu_q, step.context_lens,
                                          nh, step.max_decode_context, self.window, self.scale)
             return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o)

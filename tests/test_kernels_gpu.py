@@ -478,7 +478,7 @@ def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, windo
     K().attention_decode(q, k1, v1, dev(table), seqs, cu, cl, out1, max(ctxs), window, scale)
     # the one kernel
     k2, v2 = kc.to(gpu), vc.to(gpu)
-    out2 = K().attention_decode_fused(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), pos, sl, eps, k2, v2, dev(table),
+    out2 = K().attention_decode_fused(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), sl, eps, k2, v2, dev(table),
                                       seqs, cu, cl, nh, max(ctxs), window, scale)
     for i in listed:
         close(out2[i], out1[i].double().cpu(), torch.bfloat16)
