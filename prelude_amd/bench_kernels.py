@@ -1,0 +1,152 @@
+"""Times single kernels against their rooflines on one MI355X.
+
+    python -m prelude_amd.bench_kernels [gemm] [decode] [prefill] [elementwise] [--shape 4b|8b|32b]
+
+Each line gives the kernel's time (device events around repeated launches,
+operands rotated over copies larger than the caches where the kernel streams
+memory), the rate it reached and that rate as a fraction of the published peak
+(HBM 8 TB/s, dense bfloat16 MFMA 2.5 PFLOP/s).  The shapes are those of the
+Qwen3 sizes the benchmark configurations name.
+"""
+from __future__ import annotations
+
+import argparse
+import math
+
+import torch
+
+from .ops import kernels as K
+
+HBM_PEAK = 8.0e12
+MFMA_PEAK = 2.5e15
+SHAPES = {   # hidden, intermediate, heads, kv heads, head_dim, vocabulary
+    "4b": (2560, 9728, 32, 8, 128, 151936),
+    "8b": (4096, 12288, 32, 8, 128, 151936),
+    "32b": (5120, 25600, 64, 8, 128, 151936),
+}
+
+
+def timeit(fn, variants: int, iters: int = 50) -> float:
+    """Microseconds per call of fn(i), i cycling over the operand copies."""
+    for i in range(5):
+        fn(i % variants)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(iters):
+        fn(i % variants)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters * 1e3
+
+
+def line(name: str, us: float, nbytes: float = 0.0, flops: float = 0.0) -> None:
+    parts = [f"{name:46s} {us:9.1f} us"]
+    if nbytes:
+        rate = nbytes / us * 1e6
+        parts.append(f"{rate / 1e9:8.0f} GB/s  {rate / HBM_PEAK:5.2f} of HBM peak")
+    if flops:
+        rate = flops / us * 1e6
+        parts.append(f"{rate / 1e12:8.1f} TFLOP/s  {rate / MFMA_PEAK:5.2f} of MFMA peak")
+    print("  ".join(parts), flush=True)
+
+
+def bench_gemm(dev, shape) -> None:
+    h, inter, nh, nkv, hd, vocab = shape
+    weights = {"qkv": ((nh + 2 * nkv) * hd, h), "o": (h, nh * hd), "gate_up (SiLU*up)": (2 * inter, h),
+               "down": (h, inter), "head (f32 out)": (vocab, h)}
+    for name, (n, k) in weights.items():
+        copies = max(2, int(600e6 // (n * k * 2)))
+        rows = [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        tiles = [K.pack_tiles(w) for w in rows]
+        silu = name.startswith("gate_up")
+        f32 = torch.float32 if name.startswith("head") else None
+        for m in (1, 8, 16):
+            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            us = timeit(lambda i: K.gemm_skinny(x, tiles[i], out_dtype=f32, silu_mul_epilogue=silu), copies)
+            line(f"gemm {name} [{n}x{k}] M={m} tiled", us, nbytes=n * k * 2)
+        for m in (64, 2048):
+            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            us = timeit(lambda i: torch.matmul(x, rows[i].t()), copies, iters=20)
+            line(f"gemm {name} [{n}x{k}] M={m} library", us, nbytes=n * k * 2 if m == 64 else 0.0,
+                 flops=2.0 * m * n * k if m > 64 else 0.0)
+        del rows, tiles
+
+
+def bench_decode(dev, shape, page: int = 16) -> None:
+    _, _, nh, nkv, hd, _ = shape
+    for batch, ctx in ((1, 4096), (8, 512), (8, 4096), (8, 32768), (64, 4096)):
+        pages = batch * ctx // page
+        per_copy = pages * nkv * page * hd * 2 * 2
+        copies = max(2, min(8, int(1.2e9 // per_copy)))
+        kcs = [torch.randn(pages, nkv, page, hd, device=dev, dtype=torch.bfloat16) for _ in range(copies)]
+        vcs = [torch.randn(pages, nkv, hd, page, device=dev, dtype=torch.bfloat16) for _ in range(copies)]
+        table = torch.randperm(pages, device=dev).to(torch.int32).view(batch, ctx // page)
+        q = torch.randn(batch, nh, hd, device=dev, dtype=torch.bfloat16)
+        seqs = torch.arange(batch, device=dev, dtype=torch.int32)
+        cu = torch.arange(batch + 1, device=dev, dtype=torch.int32)
+        lens = torch.full((batch,), ctx, device=dev, dtype=torch.int32)
+        out = torch.empty_like(q)
+        scale = 1 / math.sqrt(hd)
+        us = timeit(lambda i: K.attention_decode(q, kcs[i], vcs[i], table, seqs, cu, lens, out, ctx, 0, scale), copies)
+        line(f"decode attention + merge, batch {batch}, context {ctx}", us, nbytes=per_copy)
+        del kcs, vcs
+
+
+def bench_prefill(dev, shape, page: int = 16) -> None:
+    _, _, nh, nkv, hd, _ = shape
+    for nseq, t, ctx in ((1, 512, 512), (4, 512, 512), (1, 2048, 2048), (1, 2048, 4096), (1, 8192, 8192)):
+        pages = nseq * ctx // page
+        kc = torch.randn(pages, nkv, page, hd, device=dev, dtype=torch.bfloat16)
+        vc = torch.randn(pages, nkv, hd, page, device=dev, dtype=torch.bfloat16)
+        table = torch.randperm(pages, device=dev).to(torch.int32).view(nseq, ctx // page)
+        q = torch.randn(nseq * t, nh, hd, device=dev, dtype=torch.bfloat16)
+        seqs = torch.arange(nseq, device=dev, dtype=torch.int32)
+        cu = torch.arange(0, (nseq + 1) * t, t, device=dev, dtype=torch.int32)
+        lens = torch.full((nseq,), ctx, device=dev, dtype=torch.int32)
+        out = torch.empty_like(q)
+        scale = 1 / math.sqrt(hd)
+        us = timeit(lambda i: K.attention_prefill(q, kc, vc, table, seqs, cu, lens, out, t, 0, scale), 1, iters=20)
+        line(f"prefill attention, {nseq} x {t} tokens, context {ctx}", us, flops=2.0 * nseq * nh * hd * t * (2 * ctx - t))
+
+
+def bench_elementwise(dev, shape, page: int = 16) -> None:
+    h, inter, nh, nkv, hd, _ = shape
+    for t in (8, 2048):
+        x = torch.randn(t, h, device=dev, dtype=torch.bfloat16)
+        r = torch.randn(t, h, device=dev, dtype=torch.bfloat16)
+        w = torch.ones(h, device=dev)
+        line(f"residual add + RMSNorm, {t} tokens", timeit(lambda i: K.rmsnorm(x, w, 1e-6, residual=r), 1), nbytes=t * h * 2 * 4)
+        gu = torch.randn(t, 2 * inter, device=dev, dtype=torch.bfloat16)
+        line(f"SiLU*up, {t} tokens", timeit(lambda i: K.silu_mul(gu), 1), nbytes=t * inter * 2 * 3)
+        qkv = torch.randn(t, (nh + 2 * nkv) * hd, device=dev, dtype=torch.bfloat16)
+        nw = torch.ones(hd, device=dev)
+        cos = torch.randn(4096, hd // 2, device=dev)
+        pos = torch.arange(t, device=dev, dtype=torch.int32)
+        kc = torch.zeros(max(t // page, 1), nkv, page, hd, device=dev, dtype=torch.bfloat16)
+        vc = torch.zeros(max(t // page, 1), nkv, hd, page, device=dev, dtype=torch.bfloat16)
+        line(f"QK-norm + RoPE + cache write, {t} tokens",
+             timeit(lambda i: K.qknorm_rope_kv(qkv, nw, nw, cos, cos, pos, pos, kc, vc, nh, nkv, hd, hd, 1e-6), 1),
+             nbytes=t * (nh * 2 + nkv * 4) * hd * 2)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
+    ap.add_argument("what", nargs="*", help="gemm, decode, prefill, elementwise (default: all)")
+    ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        print("bench_kernels needs a GPU")
+        return 1
+    dev = torch.device("cuda:0")
+    shape = SHAPES[args.shape]
+    todo = args.what or ["gemm", "decode", "prefill", "elementwise"]
+    print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
+          f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
+    for name in todo:
+        {"gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise}[name](dev, shape)
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

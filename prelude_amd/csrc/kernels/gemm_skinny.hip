@@ -200,12 +200,15 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
 // Shape of the launch for an [n, k] weight: tiles of 16 rows per workgroup, wavefronts per workgroup, k-steps
 // of loads a wavefront keeps in flight.  Row-major: wide weights take two tiles; then about 3000 wavefronts on
 // the chip, each with at least two k-steps.  Depends on the weight's shape and layout only, never on the batch.
-static void skinny_shape(int n, int k, int mt, bool tiled, int* nt, int* waves, int* depth) {
+static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* waves, int* depth) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
   if (tiled) {
     // measured over (tiles per workgroup, wavefronts, depth) at the shapes of a 4B model: one step in flight per
     // wavefront streams a tiled weight best; long rows want 16 wavefronts, the widest weights two tiles
+    // (how K is split over wavefronts fixes the order of the sums and follows the weight alone; the tiles per
+    // workgroup do not touch it, and more than 8 rows read X often enough that sharing it over two tiles pays)
     *nt = tiles >= 4096 ? 2 : 1;
+    if (m > 8 && tiles >= 384) *nt *= 2;
     *waves = steps >= 128 ? 16 : 8;
     *depth = 1;
     static const char* env = getenv("PA_SKINNY_SHAPE");   // "nt,waves,depth": for measurements
@@ -224,7 +227,7 @@ template <int MT, typename TC, int EPI, bool TILED, int DEPTH>
 int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
                   long ldx, long ldc) {
   int nt, waves, depth;
-  skinny_shape(n, k, MT, TILED, &nt, &waves, &depth);
+  skinny_shape(m, n, k, MT, TILED, &nt, &waves, &depth);
   dim3 grid(((n + 15) / 16 + nt - 1) / nt);
 #define PA_W(NT, WV)                                                                                            \
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED, DEPTH>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
@@ -252,7 +255,7 @@ int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bia
                   long ldx, long ldc) {
   if (TILED) {
     int nt, waves, depth;
-    skinny_shape(n, k, MT, TILED, &nt, &waves, &depth);
+    skinny_shape(m, n, k, MT, TILED, &nt, &waves, &depth);
     if (depth == 1) return launch_skinny_depth<MT, TC, EPI, TILED, 1>(st, x, w, bias, c, m, n, k, ldx, ldc);
   }
   return launch_skinny_depth<MT, TC, EPI, TILED, kDepth>(st, x, w, bias, c, m, n, k, ldx, ldc);
