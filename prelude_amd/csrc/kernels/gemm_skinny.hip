@@ -29,8 +29,6 @@
 #include "common.h"
 #include "api.h"
 
-#include <stdio.h>
-#include <stdlib.h>
 
 namespace pa {
 
@@ -209,10 +207,9 @@ static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* 
     // workgroup do not touch it, and more than 8 rows read X often enough that sharing it over two tiles pays)
     *nt = tiles >= 4096 ? 2 : 1;
     if (m > 8 && tiles >= 384) *nt *= 2;
+    if (mt > 1 && *nt > 2) *nt = 2;
     *waves = steps >= 128 ? 16 : 8;
     *depth = 1;
-    static const char* env = getenv("PA_SKINNY_SHAPE");   // "nt,waves,depth": for measurements
-    if (env) sscanf(env, "%d,%d,%d", nt, waves, depth);
     return;
   }
   *nt = mt > 1 ? 1 : (tiles >= 4096 ? 4 : (tiles >= 768 ? 2 : 1));
@@ -240,8 +237,8 @@ int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const floa
   }
   if (MT == 1 && nt == 4) {
     PA_WAVES((MT == 1 ? 4 : 1))
-  } else if (MT == 1 && nt == 2) {
-    PA_WAVES((MT == 1 ? 2 : 1))
+  } else if ((MT == 1 || (TILED && waves <= 8)) && nt == 2) {
+    PA_WAVES(((MT == 1 || TILED) ? 2 : 1))
   } else {
     PA_WAVES(1)
   }
@@ -253,18 +250,21 @@ int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const floa
 template <int MT, typename TC, int EPI, bool TILED>
 int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
                   long ldx, long ldc) {
-  if (TILED) {
-    int nt, waves, depth;
-    skinny_shape(m, n, k, MT, TILED, &nt, &waves, &depth);
-    if (depth == 1) return launch_skinny_depth<MT, TC, EPI, TILED, 1>(st, x, w, bias, c, m, n, k, ldx, ldc);
-  }
-  return launch_skinny_depth<MT, TC, EPI, TILED, kDepth>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  // the depth is part of the kernel's type: one step in flight for tiles, kDepth for rows (see skinny_shape)
+  return launch_skinny_depth<MT, TC, EPI, TILED, TILED ? 1 : kDepth>(st, x, w, bias, c, m, n, k, ldx, ldc);
 }
 
 template <typename TC, int EPI>
 int launch_skinny_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
                      long ldx, long ldc, int tiled) {
-  if (tiled) return launch_skinny<1, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  if (tiled) {
+    switch ((m + 15) / 16) {
+      case 1: return launch_skinny<1, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
+      case 2: return launch_skinny<2, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
+      case 3: return launch_skinny<3, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
+      default: return launch_skinny<4, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    }
+  }
   switch ((m + 15) / 16) {
     case 1: return launch_skinny<1, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
     case 2: return launch_skinny<2, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
@@ -306,7 +306,7 @@ extern "C" int pa_pack_tiles(void* stream, const void* w, void* out, int n, int 
   return check_launch("pack_tiles");
 }
 
-// tiled 1: w is the weight in tiles (pa_pack_tiles), and m <= 16.
+// tiled 1: w is the weight in tiles (pa_pack_tiles); more than 16 rows then only for k < 8192.
 extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w,
                               const float* bias, void* c, int m, int n, int k, long ldx, long ldc, int tiled) {
   if (m == 0 || n == 0) return 0;
@@ -316,7 +316,9 @@ extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const v
   PA_REQUIRE(ldx >= k, "gemm_skinny: row stride %ld is smaller than k=%d", ldx, k);
   PA_REQUIRE(epilogue == kPlain || (n % 2 == 0 && !bias), "gemm_skinny: the SiLU*up epilogue needs an even n and no bias");
   PA_REQUIRE(ldc >= (epilogue == kSiluMul ? n / 2 : n), "gemm_skinny: output row stride %ld is too small", ldc);
-  PA_REQUIRE(!tiled || m <= 16, "gemm_skinny: a tiled weight takes at most 16 rows, not %d", m);
+
+  PA_REQUIRE(!tiled || m <= 16 || k < 128 * 64,
+             "gemm_skinny: a tiled weight with %d columns takes at most 16 rows, not %d", k, m);
   hipStream_t st = (hipStream_t)stream;
   if (epilogue == kPlain && out_dtype == kBF16)
     return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);

@@ -211,7 +211,9 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
     return out
 
 
-SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel itself takes up to 64)
+SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel itself takes up to 64) ...
+TILED_MAX_ROWS = 48    # ... except for small weights in tiles: measured at [6144, 2560] and [2560, 4096], the
+TILED_SMALL_WEIGHT = 1 << 24   # streaming kernel wins up to 48 rows (11 against 19 us at 32), loses for larger weights
 
 
 class TiledWeight:
@@ -268,7 +270,7 @@ def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False) -> torch.Tensor:
     """x [M <= 64, K] @ w[N, K]^T in bfloat16 on the matrix cores, streaming w once.
 
-    ``w`` is a tensor [N, K] or a ``TiledWeight`` (then M <= 16).  With
+    ``w`` is a tensor [N, K] or a ``TiledWeight`` (then more than 16 rows only for K < 8192).  With
     ``silu_mul_epilogue`` the rows of w alternate gate_j, up_j and the
     result is silu(gate) * up, [M, N/2]."""
     tiled = isinstance(w, TiledWeight)
@@ -302,8 +304,11 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     _dev(x, w, bias)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise NativeError(f"linear: x {x.dtype} / w {w.dtype}")
-    if x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0:
-        return gemm_skinny(x, tiles if tiles is not None and x.shape[0] <= 16 else w, bias, out_dtype)
+    m, k = x.shape
+    if m <= SKINNY_MAX_ROWS and k % 8 == 0:
+        return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
+    if tiles is not None and m <= TILED_MAX_ROWS and w.shape[0] * k <= TILED_SMALL_WEIGHT and k < 8192 and k % 8 == 0:
+        return gemm_skinny(x, tiles, bias, out_dtype)
     y = torch.matmul(x, w.t())
     if bias is not None:
         add_bias_(y, bias)

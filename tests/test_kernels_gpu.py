@@ -152,11 +152,20 @@ def test_gemm_skinny(gpu, m, n, k):
             tact = K().gemm_skinny(xd, tiles, silu_mul_epilogue=True)
             close(tact, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
             assert torch.equal(K().linear_silu_mul(xd, lw), tact)
-    else:
-        from prelude_amd._native import NativeError
-        with pytest.raises(NativeError, match="at most 16 rows"):
-            K().gemm_skinny(xd, tiles)
-        close(K().linear(xd, K().LinearWeight(wd, tiles)), ref, torch.bfloat16)   # more rows: from the row-major copy
+    else:                                # more rows from tiles: the same sums per row as with few rows
+        many = K().gemm_skinny(xd, tiles, out_dtype=torch.float32)
+        close(many, ref, torch.float32, f32=2e-5)
+        assert torch.equal(K().gemm_skinny(xd[m - 1:].contiguous(), tiles, out_dtype=torch.float32)[0], many[m - 1])
+        close(K().linear(xd, K().LinearWeight(wd, tiles)), ref, torch.bfloat16)
+
+
+def test_tiled_weight_refuses_many_rows_of_long_weights(gpu):
+    from prelude_amd._native import NativeError
+    w = K().pack_tiles(torch.zeros(32, 8192, dtype=torch.bfloat16, device=gpu))
+    x = torch.zeros(17, 8192, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(NativeError, match="at most 16 rows"):
+        K().gemm_skinny(x, w)
+    assert float(K().linear(x, K().LinearWeight(torch.zeros(32, 8192, dtype=torch.bfloat16, device=gpu), w)).abs().max()) == 0.0
 
 
 def test_pack_tiles_layout(gpu):
