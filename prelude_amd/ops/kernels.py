@@ -24,7 +24,14 @@ def _code(t: torch.Tensor) -> int:
         raise NativeError(f"element type {t.dtype} is not supported (float32 or bfloat16)") from None
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current stream's handle.  Asked for before every launch (a graph capture switches streams), so
+    through torch's raw accessor where it has one: the Stream object costs several microseconds to build."""
+    if _RAW_STREAM is not None:
+        return _RAW_STREAM(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
