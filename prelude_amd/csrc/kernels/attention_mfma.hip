@@ -832,13 +832,8 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
 template <int HD, int GT>
 int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                       int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale) {
-  // pair tiles only when the pairs alone still give every SIMD of the chip several wavefronts
+                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, int paired) {
   const int tiles = (max_q_len + 63) / 64;
-  const long wgs = (long)tiles * nkv * (nh / nkv / GT) * nseq;
-  // (measured: pairing wins even when it leaves wavefront slots empty, so it is on whenever there are two tiles)
-  static const char* env = getenv("PA_PREFILL_PAIRED");
-  const int paired = env ? atoi(env) : (tiles >= 2 && wgs > 0 ? 1 : 0);
   dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / GT), nseq);
   static const char* lds_env = getenv("PA_PREFILL_LDS");
   const bool staged = page_shift >= 3 && page_shift <= 6 && (lds_env ? atoi(lds_env) != 0 : true);
@@ -865,13 +860,35 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
                    int max_q_len, int nh, int nkv, int page_shift, int window, float scale) {
   const int group = nh / nkv;
+  // How the work is cut: tiles in pairs (an early and a late tile of the causal triangle, so workgroups finish
+  // together) and as many heads per wavefront as share the keys and fit the registers (wider heads would not fit
+  // four heads' state in 256) -- unless that leaves compute units without a workgroup: a short prompt is better
+  // off unpaired and with a head per wavefront.  Measured at head_dim 128: one prompt of 512 tokens takes 16 us
+  // as 256 workgroups and 26 us as 64.
+  const int gt_best = (HD <= 64 && group % 4 == 0) ? 4 : (group % 2 == 0 ? 2 : 1);
+  const long tiles = (max_q_len + 63) / 64;
+  int paired = tiles >= 2, gt = gt_best;
+  auto workgroups = [&](int p, int g_) { return (p ? (tiles + 1) / 2 : tiles) * nkv * (group / g_) * nseq; };
+  const long enough = 256;
+  if (workgroups(paired, gt) < enough) {
+    if (gt > 1 && workgroups(paired, 1) >= enough) {
+      gt = 1;
+    } else if (workgroups(0, gt) >= enough) {
+      paired = 0;
+    } else {
+      paired = 0;
+      gt = 1;
+    }
+  }
+  static const char* paired_env = getenv("PA_PREFILL_PAIRED");   // for measurements
+  static const char* gt_env = getenv("PA_PREFILL_GT");
+  if (paired_env) paired = atoi(paired_env) != 0 && tiles >= 2;
+  if (gt_env && atoi(gt_env) >= 1 && atoi(gt_env) <= gt_best) gt = atoi(gt_env) == 3 ? 2 : atoi(gt_env);
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
-                                   max_q_len, nh, nkv, page_shift, window, scale)
-  static const char* gt_env = getenv("PA_PREFILL_GT");
-  const int gt_max = gt_env ? atoi(gt_env) : 4;
-  if (HD <= 64 && group % 4 == 0 && gt_max >= 4) PA_GT(4);  // wider heads would not fit four heads' state in 256 registers
-  if (group % 2 == 0 && gt_max >= 2) PA_GT(2);
+                                   max_q_len, nh, nkv, page_shift, window, scale, paired)
+  if (gt == 4) PA_GT(4);
+  if (gt == 2) PA_GT(2);
   PA_GT(1);
 #undef PA_GT
 }
