@@ -622,24 +622,31 @@ struct StageLds {
   bf16 v[2][HD][VROW];
 };
 
-// A thread's share of the staging.  Wavefront w takes the 16 keys 16w .. 16w+15 of a block of 64: of K, lane
-// (r = lane % 16, q = lane / 16) takes the 16-byte pieces 4j + q of key 16w + r; of V^T, lane (d = lane / 2,
-// h = lane % 2) takes the eight keys 16w + 8h .. + 7 of the rows d + 32j.  Pages hold 8 to 64 keys here, so a
-// block starts at a page's first key, and a thread reads one page of each cache per block, at places inside
-// the page that never change.  A page outside the pages [lo_page, hi_page] that hold the tile's keys is
-// replaced by the nearest of those; the scores of its keys are masked.
-template <int HD>
+// A thread's share of the staging, for workgroups of WAVES = 4 or 8 wavefronts.  Wavefront w takes the
+// KW = 64 / WAVES keys KW w .. of a block of 64: of K, lane (r = lane / QL, q = lane % QL; QL = 64 / KW) takes the
+// 16-byte pieces q, q + QL, .. of key KW w + r, so that the lanes of a load cover whole 64-byte stretches of a row
+// (a lane per row would ask the memory pipeline for four times as many of them); of V^T, lane (d = lane / HL, h = lane % HL; HL = KW / 8 halves)
+// takes the eight keys KW w + 8h .. + 7 of the rows d, d + 64 / HL, ...  Pages hold 8 to 64 keys here, so a block
+// starts at a page's first key, and a thread reads one page of each cache per block, at places inside the page
+// that never change.  A page outside the pages [lo_page, hi_page] that hold the tile's keys is replaced by the
+// nearest of those; the scores of its keys are masked.
+template <int HD, int WAVES>
 struct Stage {
-  static constexpr int CPK = HD / 8;          // 16-byte pieces per K row
-  static constexpr int NK = (CPK + 3) / 4;
-  static constexpr int NV = (HD + 31) / 32;
+  static_assert(WAVES == 4 || WAVES == 8, "four or eight wavefronts stage a block");
+  static constexpr int KW = kStageKeys / WAVES;   // keys a wavefront stages
+  static constexpr int QL = kWave / KW;           // lane groups along a K row
+  static constexpr int HL = KW / 8;               // 8-key halves of a wavefront's keys
+  static constexpr int DL = kWave / HL;           // V^T rows a wavefront covers at once
+  static constexpr int CPK = HD / 8;              // 16-byte pieces per K row
+  static constexpr int NK = (CPK + QL - 1) / QL;
+  static constexpr int NV = (HD + DL - 1) / DL;
   bf16x8 k[NK];
   bf16x8 v[NV];
   int kpage, vpage;
 
   __device__ __forceinline__ void load_pages(const KeyWalk& w, int key0, int wave, int lane, int lo_page, int hi_page) {
-    int kp = (key0 + 16 * wave + lane % 16) >> w.page_shift;
-    int vp = (key0 + 16 * wave + 8 * (lane % 2)) >> w.page_shift;
+    int kp = (key0 + KW * wave + lane / QL) >> w.page_shift;
+    int vp = (key0 + KW * wave + 8 * (lane % HL)) >> w.page_shift;
     kp = kp < lo_page ? lo_page : (kp > hi_page ? hi_page : kp);
     vp = vp < lo_page ? lo_page : (vp > hi_page ? hi_page : vp);
     kpage = w.table[kp];
@@ -649,31 +656,31 @@ struct Stage {
   __device__ __forceinline__ void load(const KeyWalk& w, int wave, int lane) {
     const unsigned page_elems = ((unsigned)w.nkv * HD) << w.page_shift;   // elements per page, all KV heads
     const unsigned head_off = ((unsigned)w.kvh * HD) << w.page_shift;
-    const int r = lane % 16, q = lane / 16;
+    const int r = lane / QL, q = lane % QL;
     const bf16* kp = w.kc + ((unsigned long long)(unsigned)kpage * page_elems + head_off +
-                             (unsigned)((16 * wave + r) & w.page_mask) * HD + 8 * q);
+                             (unsigned)((KW * wave + r) & w.page_mask) * HD + 8 * q);
 #pragma unroll
     for (int j = 0; j < NK; ++j)
-      if (CPK % 4 == 0 || 4 * j + q < CPK) k[j] = *reinterpret_cast<const bf16x8*>(kp + 32 * j);
-    const int d = lane / 2, h = lane % 2;
+      if (CPK % QL == 0 || QL * j + q < CPK) k[j] = *reinterpret_cast<const bf16x8*>(kp + 8 * QL * j);
+    const int d = lane / HL, h = lane % HL;
     const bf16* vp = w.vc + ((unsigned long long)(unsigned)vpage * page_elems + head_off + ((unsigned)d << w.page_shift) +
-                             (unsigned)((16 * wave + 8 * h) & w.page_mask));
+                             (unsigned)((KW * wave + 8 * h) & w.page_mask));
 #pragma unroll
     for (int j = 0; j < NV; ++j)
-      if (HD % 32 == 0 || d + 32 * j < HD) v[j] = *reinterpret_cast<const bf16x8*>(vp + ((size_t)(32 * j) << w.page_shift));
+      if (HD % DL == 0 || d + DL * j < HD) v[j] = *reinterpret_cast<const bf16x8*>(vp + ((size_t)(DL * j) << w.page_shift));
   }
 
   __device__ __forceinline__ void store(StageLds<HD>& lds, int buf, int wave, int lane) const {
-    const int r = lane % 16, q = lane / 16;
-    const int key = 16 * wave + r;   // 32 s + 8 a + 4 t + i  ->  row 32 s + 16 t + 4 a + i
+    const int r = lane / QL, q = lane % QL;
+    const int key = KW * wave + r;   // 32 s + 8 a + 4 t + i  ->  row 32 s + 16 t + 4 a + i
     const int row = (key & 32) | ((key & 4) << 2) | ((key & 24) >> 1) | (key & 3);
 #pragma unroll
     for (int j = 0; j < NK; ++j)
-      if (CPK % 4 == 0 || 4 * j + q < CPK) *reinterpret_cast<bf16x8*>(&lds.k[buf][row][8 * (4 * j + q)]) = k[j];
-    const int d = lane / 2, h = lane % 2;
+      if (CPK % QL == 0 || QL * j + q < CPK) *reinterpret_cast<bf16x8*>(&lds.k[buf][row][8 * (QL * j + q)]) = k[j];
+    const int d = lane / HL, h = lane % HL;
 #pragma unroll
     for (int j = 0; j < NV; ++j)
-      if (HD % 32 == 0 || d + 32 * j < HD) *reinterpret_cast<bf16x8*>(&lds.v[buf][d + 32 * j][16 * wave + 8 * h]) = v[j];
+      if (HD % DL == 0 || d + DL * j < HD) *reinterpret_cast<bf16x8*>(&lds.v[buf][d + DL * j][KW * wave + 8 * h]) = v[j];
   }
 };
 
@@ -700,9 +707,10 @@ __device__ __forceinline__ void attend32_lds(const StageLds<HD>& lds, int buf, i
   attend32_core<HD, GT>(key0, g, kf, va, qf, c, masked, st, vis);
 }
 
-// A 64-token tile from tile0: wavefront `wave` owns its tokens 16 wave .. 16 wave + 15.  Every wavefront takes
-// part in the staging and the barriers, also one whose tokens lie beyond the portion's end.
-template <int HD, int GT>
+// A 64-token tile from tile0 for GT * HW heads from head0: wavefront `wave` owns the tokens 16 (wave % 4) .. + 15 of
+// the GT heads from head0 + GT (wave / 4).  Every wavefront takes part in the staging and the barriers, also one
+// whose tokens lie beyond the portion's end.
+template <int HD, int GT, int HW>
 __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* __restrict__ q, bf16* __restrict__ out,
                                                  const bf16* kc, const bf16* vc, const int* table, int row0, int q_len,
                                                  int ctx, int tile0, int nh, int nkv, int kvh, int head0, int page_shift,
@@ -711,7 +719,8 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
   constexpr int KS = (HD + 31) / 32;
   const int lane = 16 * g + r;
   const int start = ctx - q_len;                // position of the portion's first token
-  const int t0 = tile0 + 16 * wave;
+  const int t0 = tile0 + 16 * (wave % 4);
+  head0 += GT * (wave / 4);
   const bool wave_on = t0 < q_len;
   const bool qvalid = t0 + r < q_len;
   const int my_pos = start + t0 + r;            // this lane's query position
@@ -736,7 +745,7 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
   for (int j = 0; j < GT; ++j)
     load_q<HD>(q + ((size_t)(row0 + (qvalid ? t0 + r : 0)) * nh + head0 + j) * HD, qvalid, g, qf[j]);
 
-  Stage<HD> stage;
+  Stage<HD, 4 * HW> stage;
   const int lo_page = wg_lo >> page_shift, hi_page = (wg_hi - 1) >> page_shift;
   int key0 = (wg_lo / kStageKeys) * kStageKeys;
   stage.load_pages(w, key0, wave, lane, lo_page, hi_page);
@@ -778,8 +787,8 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
   }
 }
 
-template <int HD, int GT>
-__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(
+template <int HD, int GT, int HW>
+__global__ __launch_bounds__(256 * HW, 2) void attn_prefill_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
@@ -789,7 +798,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int group = nh / nkv;
-  const int hgroups = group / GT;
+  const int hgroups = group / (GT * HW);
   const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
   const int seq = seq_ids[blockIdx.z];
   const int row0 = cu_q[seq];
@@ -800,12 +809,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(
   const int second = paired ? tiles - 1 - (int)blockIdx.x : first;
   if (first > second || first < 0) return;   // the same for the whole workgroup
   const int* table = block_table + (size_t)seq * table_stride;
-  const int head0 = kvh * group + hg * GT;
-  prefill_tile_lds<HD, GT>(lds, q, out, kc, vc, table, row0, q_len, ctx, second * 64, nh, nkv, kvh, head0, page_shift,
-                           window, c, wave, g, r);   // the long one first
+  const int head0 = kvh * group + hg * GT * HW;
+  prefill_tile_lds<HD, GT, HW>(lds, q, out, kc, vc, table, row0, q_len, ctx, second * 64, nh, nkv, kvh, head0,
+                               page_shift, window, c, wave, g, r);   // the long one first
   if (first != second)
-    prefill_tile_lds<HD, GT>(lds, q, out, kc, vc, table, row0, q_len, ctx, first * 64, nh, nkv, kvh, head0, page_shift,
-                             window, c, wave, g, r);
+    prefill_tile_lds<HD, GT, HW>(lds, q, out, kc, vc, table, row0, q_len, ctx, first * 64, nh, nkv, kvh, head0,
+                                 page_shift, window, c, wave, g, r);
 }
 
 // ---------------------------------------------------------------------------
@@ -829,25 +838,40 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   return 0;
 }
 
+template <int HD, int GT, int HW>
+int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
+                          int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                          int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale,
+                          int paired) {
+  const int tiles = (max_q_len + 63) / 64;
+  dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / (GT * HW)), nseq);
+  // the two buffers are more than the 64 KB a kernel may declare: asked for at launch, allowed once per kernel
+  static const hipError_t allowed =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_lds_kernel<HD, GT, HW>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(StageLds<HD>));
+  if (allowed != hipSuccess)
+    return pa::fail("attn_prefill: %zu bytes of LDS refused: %s", sizeof(StageLds<HD>), hipGetErrorString(allowed));
+  hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, GT, HW>), grid, dim3(256 * HW), sizeof(StageLds<HD>), st,
+                     (const bf16*)q, (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q,
+                     context_lens, (bf16*)out, nh, nkv, page_shift, window, scale * kLog2e, paired);
+  return check_launch("attn_prefill");
+}
+
 template <int HD, int GT>
 int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                       int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, int paired) {
+                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, int paired,
+                      int hw) {
   const int tiles = (max_q_len + 63) / 64;
   dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / GT), nseq);
   static const char* lds_env = getenv("PA_PREFILL_LDS");
   const bool staged = page_shift >= 3 && page_shift <= 6 && (lds_env ? atoi(lds_env) != 0 : true);
   if (staged) {
-    // the two buffers are more than the 64 KB a kernel may declare: asked for at launch, allowed once per kernel
-    static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_lds_kernel<HD, GT>),
-                                                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                          (int)sizeof(StageLds<HD>));
-    if (allowed != hipSuccess)
-      return pa::fail("attn_prefill: %zu bytes of LDS refused: %s", sizeof(StageLds<HD>), hipGetErrorString(allowed));
-    hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, GT>), grid, dim3(256), sizeof(StageLds<HD>), st, (const bf16*)q,
-                       (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens,
-                       (bf16*)out, nh, nkv, page_shift, window, scale * kLog2e, paired);
-    return check_launch("attn_prefill");
+    if (hw == 2)
+      return launch_prefill_staged<HD, GT, 2>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
+                                              nseq, max_q_len, nh, nkv, page_shift, window, scale, paired);
+    return launch_prefill_staged<HD, GT, 1>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
+                                            nseq, max_q_len, nh, nkv, page_shift, window, scale, paired);
   }
   hipLaunchKernelGGL((attn_prefill_kernel<HD, GT>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kc,
                      (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, nh, nkv,
@@ -880,13 +904,22 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
       gt = 1;
     }
   }
+  // one workgroup per compute unit is one wavefront per SIMD, which waits for every one of its own steps: then
+  // rather eight wavefronts a workgroup, half of them on the other heads (measured at 2,048 tokens: 69 against 77 us)
+  int hw = 1;
+  if (workgroups(paired, gt) >= enough && workgroups(paired, gt) < 2 * enough && gt >= 2 && gt == gt_best) {
+    gt /= 2;
+    hw = 2;
+  }
   static const char* paired_env = getenv("PA_PREFILL_PAIRED");   // for measurements
   static const char* gt_env = getenv("PA_PREFILL_GT");
+  static const char* hw_env = getenv("PA_PREFILL_HW");
   if (paired_env) paired = atoi(paired_env) != 0 && tiles >= 2;
   if (gt_env && atoi(gt_env) >= 1 && atoi(gt_env) <= gt_best) gt = atoi(gt_env) == 3 ? 2 : atoi(gt_env);
+  if (hw_env) hw = (atoi(hw_env) == 2 && group % (gt * 2) == 0) ? 2 : 1;
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
-                                   max_q_len, nh, nkv, page_shift, window, scale, paired)
+                                   max_q_len, nh, nkv, page_shift, window, scale, paired, hw)
   if (gt == 4) PA_GT(4);
   if (gt == 2) PA_GT(2);
   PA_GT(1);
