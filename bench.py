@@ -36,6 +36,13 @@ QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_si
                 use_sliding_window=False, hidden_act="silu", eos_token_id=151645)
 
 
+# the other shapes the benchmark configurations name (not the default run): --shape 8b | 32b
+QWEN3_8B = dict(QWEN3_4B, hidden_size=4096, intermediate_size=12288, tie_word_embeddings=False)
+QWEN3_32B = dict(QWEN3_4B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
+                 max_window_layers=64, tie_word_embeddings=False)
+SHAPES = {"4b": QWEN3_4B, "8b": QWEN3_8B, "32b": QWEN3_32B}
+
+
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
     """The engine's own model with weights drawn on the device (no 8 GB file is written)."""
     import torch
@@ -69,7 +76,7 @@ def weight_bytes(raw, el):
     h, i, v = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
     nh, nkv, hd, L = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"], raw["num_hidden_layers"]
     per_layer = ((nh + 2 * nkv) * hd * h + nh * hd * h + 3 * i * h) * el + (2 * h + 2 * hd) * 4
-    head = v * h * el           # the head matrix is read whole; the embedding only gathers rows
+    head = v * h * el           # the head matrix is read whole; the embedding (the same matrix when tied) only gathers rows
     return L * per_layer + head + h * 4, L * ((nh + 2 * nkv) * hd * h + nh * hd * h + 3 * i * h)
 
 
@@ -169,6 +176,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 8B or 32B")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
@@ -179,7 +187,8 @@ def main() -> int:
         return 2
 
     import torch
-    raw = dict(QWEN3_4B)
+    raw = dict(SHAPES[args.shape])
+    name = f"Qwen3-{args.shape.upper()} shape"
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -199,15 +208,14 @@ def main() -> int:
     achieved = step_bytes / sec / 1e9
 
     out = {
-        "metric": "decode tok/s @ batch 8, context 4096 (Qwen3-4B shape, bf16)" if args.batch == 8 else
-                  f"decode tok/s @ batch {args.batch}, context {args.context} (Qwen3-4B shape)",
+        "metric": f"decode tok/s @ batch {args.batch}, context {args.context} ({name}, {short})",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic (random tokens, random-init weights)",
-        "config": {"model": "Qwen3-4B shape", "layers": raw["num_hidden_layers"], "layers_full": full_layers,
+        "config": {"model": name, "layers": raw["num_hidden_layers"], "layers_full": full_layers,
                    "hidden": raw["hidden_size"], "heads": raw["num_attention_heads"],
                    "kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
-                   "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"], "tied": True,
+                   "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"], "tied": bool(raw["tie_word_embeddings"]),
                    "global_batch": args.batch, "seq_len": args.context, "page_size": 16, "parallelism": "none"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
