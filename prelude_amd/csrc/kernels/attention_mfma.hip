@@ -861,11 +861,9 @@ template <int HD, int GT>
 int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                       int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                       int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, int paired,
-                      int hw) {
+                      int hw, bool staged) {
   const int tiles = (max_q_len + 63) / 64;
   dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / GT), nseq);
-  static const char* lds_env = getenv("PA_PREFILL_LDS");
-  const bool staged = page_shift >= 3 && page_shift <= 6 && (lds_env ? atoi(lds_env) != 0 : true);
   if (staged) {
     if (hw == 2)
       return launch_prefill_staged<HD, GT, 2>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
@@ -879,10 +877,16 @@ int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void*
   return check_launch("attn_prefill");
 }
 
+// How a prefill launch is cut, -1 where the launcher chooses: tiles in pairs, heads a wavefront (1, 2, 4), head
+// groups a workgroup (1, 2), keys staged in LDS.
+struct PrefillCut {
+  int paired = -1, heads = -1, groups = -1, staged = -1;
+};
+
 template <int HD>
 int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
-                   int max_q_len, int nh, int nkv, int page_shift, int window, float scale) {
+                   int max_q_len, int nh, int nkv, int page_shift, int window, float scale, const PrefillCut& want) {
   const int group = nh / nkv;
   // How the work is cut: tiles in pairs (an early and a late tile of the causal triangle, so workgroups finish
   // together) and as many heads per wavefront as share the keys and fit the registers (wider heads would not fit
@@ -911,15 +915,30 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
     gt /= 2;
     hw = 2;
   }
-  static const char* paired_env = getenv("PA_PREFILL_PAIRED");   // for measurements
-  static const char* gt_env = getenv("PA_PREFILL_GT");
-  static const char* hw_env = getenv("PA_PREFILL_HW");
-  if (paired_env) paired = atoi(paired_env) != 0 && tiles >= 2;
-  if (gt_env && atoi(gt_env) >= 1 && atoi(gt_env) <= gt_best) gt = atoi(gt_env) == 3 ? 2 : atoi(gt_env);
-  if (hw_env) hw = (atoi(hw_env) == 2 && group % (gt * 2) == 0) ? 2 : 1;
+  // keys staged in LDS for pages of 8 to 64 keys; smaller and larger pages go to the kernel that reads them itself
+  bool staged = page_shift >= 3 && page_shift <= 6;
+  // a caller's own cut (tests and measurements), where it is one the kernels have
+  if (want.paired >= 0) paired = want.paired != 0 && tiles >= 2;
+  if (want.heads >= 0) {
+    PA_REQUIRE((want.heads == 1 || want.heads == 2 || want.heads == 4) && want.heads <= gt_best,
+               "attn_prefill: %d heads a wavefront, this shape takes up to %d (1, 2 or 4)", want.heads, gt_best);
+    gt = want.heads;
+    if (want.groups < 0) hw = 1;
+  }
+  if (want.groups >= 0) {
+    PA_REQUIRE(want.groups == 1 || (want.groups == 2 && group % (gt * 2) == 0),
+               "attn_prefill: %d head groups a workgroup with %d heads a wavefront and %d heads a KV head", want.groups,
+               gt, group);
+    hw = want.groups;
+  }
+  if (want.staged >= 0) {
+    PA_REQUIRE(want.staged == 0 || staged, "attn_prefill: pages of %d keys are not staged", 1 << page_shift);
+    staged = want.staged != 0;
+  }
+  PA_REQUIRE(staged || hw == 1, "attn_prefill: two head groups a workgroup only with staged keys");
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
-                                   max_q_len, nh, nkv, page_shift, window, scale, paired, hw)
+                                   max_q_len, nh, nkv, page_shift, window, scale, paired, hw, staged)
   if (gt == 4) PA_GT(4);
   if (gt == 2) PA_GT(2);
   PA_GT(1);
@@ -1019,6 +1038,25 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
                                   max_splits, fq);
 }
 
+// pa_attn_prefill with the cut given: paired (tiles in pairs), heads a wavefront (1, 2, 4), head groups a
+// workgroup (1, 2), staged (keys through LDS); -1 leaves one to the launcher.  A cut the shape does not take is
+// refused.  Every cut gives the same result up to rounding.
+extern "C" int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                                   void* out, int nseq, int max_q_len, int nh, int nkv, int hd, int page_size,
+                                   int window, float scale, int paired, int heads, int groups, int staged) {
+  if (nseq == 0) return 0;
+  if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
+  PA_REQUIRE(max_q_len >= 1, "attn_prefill: longest portion %d", max_q_len);
+  PrefillCut cut;
+  cut.paired = paired, cut.heads = heads, cut.groups = groups, cut.staged = staged;
+#define PA_CALL(HD)                                                                                                   \
+  return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
+                            out, nseq, max_q_len, nh, nkv, __builtin_ctz(page_size), window, scale, cut)
+  PA_HD_SWITCH(hd, PA_CALL)
+#undef PA_CALL
+}
+
 extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                                int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                                void* out, int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window,
@@ -1028,7 +1066,7 @@ extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, cons
   PA_REQUIRE(max_q_len >= 1, "attn_prefill: longest portion %d", max_q_len);
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, nh, nkv, __builtin_ctz(page_size), window, scale)
+                            out, nseq, max_q_len, nh, nkv, __builtin_ctz(page_size), window, scale, PrefillCut{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }

@@ -443,18 +443,24 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
 
 
 def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_q_len: int,
-                      window: int, scale: float) -> None:
-    """Matrix-core attention for the sequences ``seq_ids`` (portions of several tokens); writes their rows of ``out``."""
+                      window: int, scale: float, cut=None) -> None:
+    """Matrix-core attention for the sequences ``seq_ids`` (portions of several tokens); writes their rows of ``out``.
+
+    ``cut`` (tests and measurements) fixes how the launch is cut instead of leaving it to the launcher:
+    ``(paired, heads a wavefront, head groups a workgroup, staged)``, -1 for the launcher's choice."""
     _dev(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out)
     t, nh, hd = q.shape
     _check_caches(k_cache, v_cache, k_cache.shape[1], hd, torch.bfloat16, "attention_prefill")
     n = seq_ids.shape[0]
     if n == 0:
         return
-    check(kernels().pa_attn_prefill(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
-                                    block_table.shape[1], _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out), n,
-                                    int(max_q_len), nh, k_cache.shape[1], hd, k_cache.shape[2], int(window),
-                                    float(scale)))
+    args = (_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_ids),
+            _ptr(cu_q), _ptr(context_lens), _ptr(out), n, int(max_q_len), nh, k_cache.shape[1], hd, k_cache.shape[2],
+            int(window), float(scale))
+    if cut is None:
+        check(kernels().pa_attn_prefill(*args))
+    else:
+        check(kernels().pa_attn_prefill_cut(*args, *(int(c) for c in cut)))
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int,

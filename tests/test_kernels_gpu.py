@@ -292,7 +292,7 @@ def test_qknorm_rope_refuses_bad_sizes(gpu):
 
 
 # ---- attention over the paged cache --------------------------------------------------------------
-def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None, kernel="generic"):
+def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None, kernel="generic", cut=None):
     """seqs: list of (context_len, q_len): the last q_len tokens of each context are this step's queries.
     Pages are handed out in a scrambled order.  Returns (engine output, plain output)."""
     g = torch.Generator().manual_seed(seed)
@@ -341,7 +341,7 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
         K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, out, max([seqs[i][0] for i in dec], default=0),
                              window, 1.0 / math.sqrt(hd))
         K().attention_prefill(qd, kd, vd, td, i32(pre), i32(cu), ctxs, out, max([seqs[i][1] for i in pre], default=0),
-                              window, 1.0 / math.sqrt(hd))
+                              window, 1.0 / math.sqrt(hd), cut=cut)
         return out, torch.cat(refs)
     out = K().attention_generic(q.to(gpu), kc.to(dtype).to(gpu), vc.to(dtype).to(gpu), table.to(gpu),
                                 torch.tensor(seq_of, dtype=torch.int32, device=gpu),
@@ -434,6 +434,40 @@ def test_mfma_attention_far_key_and_edges(gpu):
             out, ref = paged_case(gpu, torch.bfloat16, 2, 1, hd, 16, seqs, 20, scale_trick=trick2, kernel="mfma")
             close(out, ref, torch.bfloat16)
             assert (float(out[-1].float().abs().max()) > 50.0) == seen
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0)])
+def test_prefill_attention_every_cut(gpu, nh, nkv, hd, page, window):
+    """The launcher cuts a prefill by the size of the step (tiles in pairs, 1, 2 or 4 heads a wavefront, one or two
+    head groups a workgroup, keys staged in LDS or not); small cases would only ever see one cut, so each is
+    asked for here, on portions that start inside a context, end inside a tile and share a step."""
+    seqs = [(333, 333), (500, 70), (1, 1), (129, 128), (64, 64), (700, 450)]
+    group = nh // nkv
+    most = 4 if hd <= 64 and group % 4 == 0 else 2
+    base = None
+    for staged in (1, 0):
+        for paired in (1, 0):
+            for heads in (1, 2, 4):
+                for groups in (1, 2):
+                    if heads > most or (groups == 2 and (not staged or group % (2 * heads))):
+                        continue
+                    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=3, kernel="mfma",
+                                          cut=(paired, heads, groups, staged))
+                    assert not bool(torch.isnan(out).any()), (staged, paired, heads, groups)
+                    close(out, ref, torch.bfloat16)
+                    if base is None:
+                        base = out
+                    # the cut moves no key to another block of 32: the same sums in the same order
+                    assert torch.equal(out, base), (staged, paired, heads, groups)
+
+
+def test_prefill_attention_refuses_a_cut_the_shape_does_not_take(gpu):
+    with pytest.raises(NativeError, match="heads a wavefront"):
+        paged_case(gpu, torch.bfloat16, 8, 2, 128, 16, [(70, 70)], 0, kernel="mfma", cut=(-1, 4, -1, -1))
+    with pytest.raises(NativeError, match="head groups"):
+        paged_case(gpu, torch.bfloat16, 3, 3, 64, 16, [(70, 70)], 0, kernel="mfma", cut=(-1, 1, 2, -1))
+    with pytest.raises(NativeError, match="not staged"):
+        paged_case(gpu, torch.bfloat16, 4, 2, 64, 4, [(70, 70)], 0, kernel="mfma", cut=(-1, -1, -1, 1))
 
 
 def test_mfma_attention_batch_and_page_independence(gpu):
