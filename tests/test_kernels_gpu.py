@@ -462,6 +462,7 @@ def test_prefill_attention_every_cut(gpu, nh, nkv, hd, page, window):
 
 
 def test_prefill_attention_refuses_a_cut_the_shape_does_not_take(gpu):
+    from prelude_amd._native import NativeError
     with pytest.raises(NativeError, match="heads a wavefront"):
         paged_case(gpu, torch.bfloat16, 8, 2, 128, 16, [(70, 70)], 0, kernel="mfma", cut=(-1, 4, -1, -1))
     with pytest.raises(NativeError, match="head groups"):
