@@ -167,6 +167,62 @@ def time_prefill(raw, dtype, tokens, reps):
     return best
 
 
+def time_mixed(raw, dtype, chunk, decoding, context, steps, warmup):
+    """A step with one prompt portion of `chunk` tokens beside `decoding` requests that feed one token each, at
+    contexts spread up to `context`; the portion continues a prompt that is already `context - chunk` long.
+    Returns seconds per step."""
+    import numpy as np
+    import torch
+    from prelude_amd.engine import StepEntry
+    total = steps + warmup
+    rng = np.random.default_rng(11)
+    vocab = raw["vocab_size"]
+    lens = [int(x) for x in np.linspace(256, context - total - 1, decoding)]
+    need = sum(-(-(n + total + 1) // 64) * 64 for n in lens) + total * (context + 64)
+    eng = build_engine(raw, dtype, cache_tokens=need + 4096)
+    for rid, n in enumerate(lens):
+        p = rng.integers(0, vocab, size=n).tolist()
+        for s0 in range(0, n, 2048):
+            eng.step([StepEntry(rid, p[s0:s0 + 2048], [])])
+    times = []
+    for it in range(total):
+        big = 1000 + it
+        head = rng.integers(0, vocab, size=context - chunk).tolist()
+        for s0 in range(0, len(head), 2048):
+            eng.step([StepEntry(big, head[s0:s0 + 2048], [])])
+        entries = [StepEntry(big, rng.integers(0, vocab, size=chunk).tolist(), [chunk - 1])]
+        entries += [StepEntry(rid, [int(rng.integers(0, vocab))], [0]) for rid in range(decoding)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.step(entries)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        eng.release(big)
+    del eng
+    torch.cuda.empty_cache()
+    return sum(times[warmup:]) / steps
+
+
+def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency):
+    """`requests` prompts of `prompt_len` random tokens, `max_tokens` new tokens each, through LLM.generate with
+    at most `concurrency` of them handed over at a time (the reference's published workload is this with one
+    new token, over HTTP).  Returns (seconds in all, list of seconds per call)."""
+    import numpy as np
+    from prelude_amd import LLM
+    eng = build_engine(raw, dtype, cache_tokens=min(requests, max(concurrency, 16)) * (prompt_len + max_tokens + 64))
+    llm = LLM.from_engine(eng)
+    rng = np.random.default_rng(5)
+    prompts = [rng.integers(0, raw["vocab_size"] - 1000, size=prompt_len).tolist() for _ in range(requests)]
+    llm.generate(prompts[:min(concurrency, 8)], max_tokens=max_tokens, temperature=0.0)   # warm-up
+    calls = []
+    t0 = time.perf_counter()
+    for s0 in range(0, requests, concurrency):
+        t1 = time.perf_counter()
+        llm.generate(prompts[s0:s0 + concurrency], max_tokens=max_tokens, temperature=0.0)
+        calls.append(time.perf_counter() - t1)
+    return time.perf_counter() - t0, calls
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -181,6 +237,13 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone and print its record (for profiles)")
+    ap.add_argument("--mixed", action="store_true",
+                    help="time a step of one --prefill-tokens portion beside 63 decoding requests at contexts up to "
+                         "--context, and print its record")
+    ap.add_argument("--requests", type=int, default=0,
+                    help="time this many 512-token prompts with one new token each through LLM.generate, "
+                         "--concurrency at a time, and print the record")
+    ap.add_argument("--concurrency", type=int, default=96)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus, flush=True)
@@ -196,6 +259,21 @@ def main() -> int:
     el = 2 if args.dtype == "bfloat16" else 4
     short = "bf16" if args.dtype == "bfloat16" else "f32"
 
+    if args.mixed:
+        sec = time_mixed(raw, args.dtype, args.prefill_tokens, 63, args.context, max(4, args.steps // 8), 2)
+        toks = args.prefill_tokens + 63
+        print(json.dumps({"model": name, "mixed_step": f"{args.prefill_tokens} prompt tokens + 63 decoding requests",
+                          "context": args.context, "ms": round(sec * 1e3, 3), "tok_per_s": round(toks / sec, 1)}),
+              flush=True)
+        return 0
+    if args.requests:
+        total, calls = time_requests(raw, args.dtype, args.requests, 512, 1, args.concurrency)
+        calls.sort()
+        print(json.dumps({"model": name, "workload": f"{args.requests} prompts of 512 tokens, 1 new token, "
+                          f"{args.concurrency} at a time (LLM.generate, no HTTP)",
+                          "req_per_s": round(args.requests / total, 1), "tok_per_s": round(args.requests * 512 / total, 1),
+                          "call_ms_p50": round(calls[len(calls) // 2] * 1e3, 2)}), flush=True)
+        return 0
     if args.prefill_only:
         psec = time_prefill(raw, args.dtype, args.prefill_tokens, reps=3)
         print(json.dumps({"prefill_tokens": args.prefill_tokens, "ms": round(psec * 1e3, 3),

@@ -85,9 +85,22 @@ class LLM:
             if not hasattr(cfg, k):
                 raise TypeError(f"unknown engine option {k!r}")
             setattr(cfg, k, v)
-        self.config = cfg
         self.model_dir = model
-        self.engine = Engine.from_model_dir(model, cfg)
+        self._attach(Engine.from_model_dir(model, cfg))
+
+    @classmethod
+    def from_engine(cls, engine: Engine, model_dir: Optional[str] = None) -> "LLM":
+        """An LLM around an engine that is already built (its ``config`` gives the scheduler's limits);
+        ``model_dir`` is only needed for text prompts (its tokenizer.json)."""
+        self = cls.__new__(cls)
+        self.model_dir = model_dir
+        self._attach(engine)
+        return self
+
+    def _attach(self, engine: Engine) -> None:
+        cfg = engine.config
+        self.config = cfg
+        self.engine = engine
         spec = self.engine.model.spec
         self.eos_token_ids = frozenset(spec.eos_token_ids)
         self.max_positions = spec.max_positions
@@ -102,7 +115,7 @@ class LLM:
     # ---- tokenizer (only when prompts are text) --------------------------------
     def tokenizer(self):
         if self._tokenizer is None:
-            path = os.path.join(self.model_dir, "tokenizer.json")
+            path = os.path.join(self.model_dir or "", "tokenizer.json")
             if not os.path.isfile(path):
                 raise ValueError(f"text prompts need {path}; pass token ids instead")
             from tokenizers import Tokenizer
