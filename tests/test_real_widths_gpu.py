@@ -1,0 +1,88 @@
+"""The engine at the layer widths of a real model (Qwen3-4B: hidden 2560, 32 heads over 8 KV heads of 128,
+intermediate 9728) against the plain implementation.  Two layers and a vocabulary of 70,001 keep it small; the
+tiny configurations never reach the kernels' wide variants (products over hundreds of tiles, the head over
+thousands, vector norms, the decode attention that takes the raw projection), this does."""
+import functools
+import json
+import os
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+from helpers import check
+
+pytestmark = pytest.mark.gpu
+_keep = []
+
+
+def wide_config() -> dict:
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=70001, hidden_size=2560,
+                intermediate_size=9728, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8,
+                head_dim=128, attention_bias=False, max_position_embeddings=1024, sliding_window=None,
+                max_window_layers=2, tie_word_embeddings=True, rope_theta=1000000.0, rms_norm_eps=1e-6,
+                use_sliding_window=False, hidden_act="silu", eos_token_id=70000)
+
+
+@functools.lru_cache(maxsize=None)
+def wide_model():
+    """(folder, tokens, float64 logits of the plain implementation, its weights); weights stored in bfloat16 so that both
+    paths of the engine and the plain implementation start from the same numbers."""
+    from prelude_amd.weights import write_safetensors
+    cfg = wide_config()
+    w = pm.random_weights(cfg, seed=4, std=0.02, norm_std=0.02)
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    tmp = tempfile.TemporaryDirectory(prefix="prelude_amd_test_wide_")
+    _keep.append(tmp)
+    with open(os.path.join(tmp.name, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(tmp.name, "model.safetensors"), w)
+    toks = torch.randint(0, cfg["vocab_size"], (96,), generator=torch.Generator().manual_seed(21)).tolist()
+    w64 = {k: v.double() for k, v in w.items()}
+    return tmp.name, toks, pm.forward(cfg, w64, toks), w64
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_then_decoded_then_mixed(gpu, dtype):
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref, _ = wide_model()
+    r = TraceRunner(folder, dtype, 512, page_size=16)
+    n = len(toks)
+    got = r.step([{"id": "whole", "tokens": toks, "want": list(range(n))}], ["whole"])
+    check(got, ref, dtype, "whole")
+    # most of it in one step, the last 32 one by one
+    outs = [r.step([{"id": "d", "tokens": toks[:n - 32], "want": list(range(n - 32))}])]
+    for i in range(n - 32, n):
+        outs.append(r.step([{"id": "d", "tokens": [toks[i]], "want": [0]}]))
+    r.step([], ["d"])
+    check(np.concatenate(outs), ref, dtype, "decoded")
+    # three requests a step: two decode (at different places) beside portions of a third
+    for rid, upto in (("x", 40), ("y", 70)):
+        r.step([{"id": rid, "tokens": toks[:upto], "want": []}])
+    at = {"x": 40, "y": 70, "z": 0}
+    rows = {k: [] for k in at}
+    for size in (17, 2, 23, 5, 1, 9):
+        entries = []
+        for rid in ("x", "y"):
+            entries.append({"id": rid, "tokens": [toks[at[rid]]], "want": [0]})
+        entries.append({"id": "z", "tokens": toks[at["z"]:at["z"] + size], "want": list(range(size))})
+        out = r.step(entries)
+        rows["x"].append(out[0:1]), rows["y"].append(out[1:2]), rows["z"].append(out[2:])
+        at["x"] += 1
+        at["y"] += 1
+        at["z"] += size
+    check(np.concatenate(rows["x"]), ref[40:46], dtype, "mixed, first decoding request")
+    check(np.concatenate(rows["y"]), ref[70:76], dtype, "mixed, second decoding request")
+    check(np.concatenate(rows["z"]), ref[:57], dtype, "mixed, portions")
+    r.step([], ["x", "y", "z"])
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
+def test_greedy_generation_at_real_widths(gpu):
+    from prelude_amd import LLM
+    folder, toks, _, w64 = wide_model()
+    llm = LLM(folder, dtype="float32", max_cache_tokens=512)
+    res = llm.generate([toks[:20]], max_tokens=4, temperature=0.0)[0]
+    assert res.token_ids == pm.greedy(wide_config(), w64, toks[:20], 4)
