@@ -18,7 +18,6 @@
 namespace pa {
 
 constexpr int kQkWaves = 4;
-constexpr int kQkGroup = 4;   // heads a wavefront of the wide kernel takes
 constexpr int kMaxHeadDim = 256;
 
 // One wavefront per (token, head) over the nh + 2*nkv heads of a token's row.
@@ -117,16 +116,22 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
   }
 }
 
+// Query and key heads a wavefront of the wide kernel takes: U loads of 64 lanes x 16 bytes.
+template <typename T, int EPL, int U>
+__host__ __device__ constexpr int wide_heads() {
+  return U * kWave / (EPL * kWave / (16 / (int)sizeof(T)));
+}
+
 // The same for head_dim 64, 128 or 256 rotated over its whole width: a lane owns EPL = head_dim / 64
 // contiguous elements, read and written as one vector; its rotation partner (element + head_dim / 2)
 // sits in lane ^ 32, so nothing goes through LDS.
 //
 // Units (one wavefront each): ceil(tokens / vgroup) x nkv groups of vgroup (1 or 8) tokens of one value head, then
-// tokens x groups of kQkGroup query and key heads.  In the transposed value page a token's elements lie
+// tokens x groups of query and key heads (see below).  In the transposed value page a token's elements lie
 // page_size apart, but eight tokens whose slots are consecutive and start at a multiple of eight (a run: the usual
 // case inside a prompt portion) lie side by side for every element, so a run is written with one vector store
 // per element by the wavefront in whose group the run starts; tokens outside runs are written one by one.
-template <typename T, int EPL>
+template <typename T, int EPL, int U>
 __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, const int* __restrict__ positions,
@@ -135,10 +140,11 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
   typedef T vec_t __attribute__((ext_vector_type(EPL)));
   typedef T run_t __attribute__((ext_vector_type(8)));
   constexpr int hd = EPL * kWave;
+  __shared__ __align__(16) T turn[kQkWaves][8][hd];   // a run of eight value rows on its way to being columns
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int heads = nh + 2 * nkv;
   const int qk_heads = nh + nkv;
-  const int head_groups = (qk_heads + kQkGroup - 1) / kQkGroup;
+  const int head_groups = (qk_heads + wide_heads<T, EPL, U>() - 1) / wide_heads<T, EPL, U>();
   const long long qk_units = (long long)tokens * head_groups;
   const long long v_units = (slots && nkv > 0) ? (long long)((tokens + vgroup - 1) / vgroup) * nkv : 0;
   long long unit = (long long)blockIdx.x * kQkWaves + wave;
@@ -185,17 +191,31 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
       const int off = slot % page_size;
       T* dst = v_cache + (page * nkv + kvh) * hd * page_size + off;
       if (in_run) {
-        vec_t v[8];
+        // the eight rows come in with 16 bytes a lane and are turned through LDS (the wavefront's own
+        // stretch of it: LDS operations of one wavefront keep their order)
+        constexpr int VEC = 16 / (int)sizeof(T);
+        constexpr int LPH = hd / VEC, TPL = kWave / LPH;   // lanes a row, rows a load
+        typedef T row_t __attribute__((ext_vector_type(VEC)));
+        const int c = lane % LPH;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          v[i] = *reinterpret_cast<const vec_t*>(qkv + ((size_t)(x + i) * heads + qk_heads + kvh) * hd + lane * EPL);
+        for (int l = 0; l < 8 / TPL; ++l) {
+          const int tok = l * TPL + lane / LPH;
+          const row_t v =
+              *reinterpret_cast<const row_t*>(qkv + ((size_t)(x + tok) * heads + qk_heads + kvh) * hd + c * VEC);
+          *reinterpret_cast<row_t*>(&turn[wave][tok][c * VEC]) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
+          const int d = e * kWave + lane;
           run_t r;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) r[i] = v[i][e];
-          *reinterpret_cast<run_t*>(dst + (size_t)(lane * EPL + e) * page_size) = r;
+          for (int i = 0; i < 8; ++i) r[i] = turn[wave][i][d];
+          *reinterpret_cast<run_t*>(dst + (size_t)d * page_size) = r;
         }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
       } else {
         const vec_t xv = *reinterpret_cast<const vec_t*>(qkv + ((size_t)x * heads + qk_heads + kvh) * hd + lane * EPL);
 #pragma unroll
@@ -206,56 +226,72 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
   }
   unit -= v_units;
   if (unit >= qk_units) return;
-  // queries and keys: kQkGroup heads of one token, loaded together so one memory round trip serves them all
-  const int t = (int)(unit / head_groups), h0 = (int)(unit % head_groups) * kQkGroup;
+  // Queries and keys: a lane owns 16 bytes of a head, LPH lanes a head, so one load of the wavefront brings
+  // 64 / LPH heads that lie side by side (1 KB), and U such loads are in flight before anything is computed.
+  // A lane's rotation partner (element + head_dim / 2) sits LPH / 2 lanes away.  Heads past the last one, and
+  // keys of tokens that are not cached, are computed on zeros and not stored, so every lane takes every shuffle.
+  constexpr int VEC = 16 / (int)sizeof(T);
+  constexpr int LPH = hd / VEC, HPL = kWave / LPH;
+  typedef T row_t __attribute__((ext_vector_type(VEC)));
+  const int t = (int)(unit / head_groups), h0 = (int)(unit % head_groups) * HPL * U;
+  const int sub = lane / LPH, c = lane % LPH;
   const long long slot = slots ? (long long)slots[t] : -1;
   const int pos = positions[t];
-  const int j0 = (lane % 32) * EPL;  // index into the cos/sin row
-  typedef float rot_t __attribute__((ext_vector_type(EPL)));
-  const rot_t c = *reinterpret_cast<const rot_t*>(cos_table + (size_t)pos * (hd / 2) + j0);
-  const rot_t sn = *reinterpret_cast<const rot_t*>(sin_table + (size_t)pos * (hd / 2) + j0);
-  vec_t xv[kQkGroup];
+  const int j0 = (c % (LPH / 2)) * VEC;  // index into the cos/sin row
+  float cs[VEC], sn[VEC], qw[VEC], kw[VEC];
 #pragma unroll
-  for (int i = 0; i < kQkGroup; ++i)
-    if (h0 + i < qk_heads) xv[i] = *reinterpret_cast<const vec_t*>(qkv + ((size_t)t * heads + h0 + i) * hd + lane * EPL);
-  rot_t qw, kw;
+  for (int e = 0; e < VEC; e += 4) {
+    const f32x4 cv = *reinterpret_cast<const f32x4*>(cos_table + (size_t)pos * (hd / 2) + j0 + e);
+    const f32x4 sv = *reinterpret_cast<const f32x4*>(sin_table + (size_t)pos * (hd / 2) + j0 + e);
+    const f32x4 one = {1.f, 1.f, 1.f, 1.f};
+    const f32x4 qv = q_weight ? *reinterpret_cast<const f32x4*>(q_weight + c * VEC + e) : one;
+    const f32x4 kv = k_weight ? *reinterpret_cast<const f32x4*>(k_weight + c * VEC + e) : one;
 #pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    qw[e] = q_weight ? q_weight[lane * EPL + e] : 1.0f;
-    kw[e] = k_weight ? k_weight[lane * EPL + e] : 1.0f;
+    for (int i = 0; i < 4; ++i) cs[e + i] = cv[i], sn[e + i] = sv[i], qw[e + i] = qv[i], kw[e + i] = kv[i];
+  }
+  row_t xv[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int h = h0 + u * HPL + sub;
+    if (h < qk_heads) {
+      xv[u] = *reinterpret_cast<const row_t*>(qkv + ((size_t)t * heads + h) * hd + c * VEC);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) xv[u][e] = from_f32<T>(0.f);
+    }
   }
 #pragma unroll
-  for (int i = 0; i < kQkGroup; ++i) {
-    const int h = h0 + i;
-    if (h >= qk_heads) break;
-    T* dst;
+  for (int u = 0; u < U; ++u) {
+    const int h = h0 + u * HPL + sub;
     const bool is_q = h < nh;
+    const bool normed = is_q ? q_weight != nullptr : k_weight != nullptr;
+    float x[VEC];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      x[e] = to_f32(xv[u][e]);
+      ss += x[e] * x[e];
+    }
+#pragma unroll
+    for (int off = LPH / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+    const float inv = rsqrtf(ss / (float)hd + eps);
+    row_t ov;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if (normed) x[e] = x[e] * inv * (is_q ? qw[e] : kw[e]);
+      const float partner = __shfl_xor(x[e], LPH / 2, kWave);
+      const float r = c < LPH / 2 ? x[e] * cs[e] - partner * sn[e] : partner * sn[e] + x[e] * cs[e];
+      ov[e] = from_f32<T>(r);
+    }
+    if (h >= qk_heads || (!is_q && slot < 0)) continue;
+    T* dst;
     if (is_q) {
       dst = q_out + ((size_t)t * nh + h) * hd;
     } else {
-      if (slot < 0) continue;
       const long long page = slot / page_size, off = slot % page_size;
       dst = k_cache + (((size_t)page * nkv + (h - nh)) * page_size + off) * hd;
     }
-    const bool normed = is_q ? q_weight != nullptr : k_weight != nullptr;
-    float x[EPL];
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      x[e] = to_f32(xv[i][e]);
-      ss += x[e] * x[e];
-    }
-    ss = wave_sum(ss);
-    const float inv = rsqrtf(ss / (float)hd + eps);
-    vec_t ov;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      if (normed) x[e] = x[e] * inv * (is_q ? qw[e] : kw[e]);
-      const float partner = __shfl_xor(x[e], 32, kWave);
-      const float r = lane < 32 ? x[e] * c[e] - partner * sn[e] : partner * sn[e] + x[e] * c[e];
-      ov[e] = from_f32<T>(r);
-    }
-    *reinterpret_cast<vec_t*>(dst + lane * EPL) = ov;
+    *reinterpret_cast<row_t*>(dst + c * VEC) = ov;
   }
 }
 
@@ -280,13 +316,25 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
   hipStream_t st = (hipStream_t)stream;
   if (rot == hd && rot > 0 && (hd == 64 || hd == 128 || hd == 256) && (dtype == kF32 || dtype == kBF16)) {
     const int vgroup = tokens >= 64 ? 8 : 1;   // runs of eight tokens pay only in prompt portions
-    const long long wide_units =
-        (long long)tokens * ((nh + nkv + kQkGroup - 1) / kQkGroup) + (long long)((tokens + vgroup - 1) / vgroup) * nkv;
-    const unsigned wide_blocks = (unsigned)((wide_units + kQkWaves - 1) / kQkWaves);
-#define PA_WIDE(T, EPL)                                                                                             \
-  hipLaunchKernelGGL((qknorm_rope_kv_wide_kernel<T, EPL>), dim3(wide_blocks), dim3(kQkWaves * kWave), 0, st, (const T*)qkv, \
-                     q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)q_out, (T*)k_cache, (T*)v_cache, \
-                     tokens, nh, nkv, page_size, eps, vgroup)
+    const long long v_units = (long long)((tokens + vgroup - 1) / vgroup) * nkv;
+    // many tokens: five loads in flight per wavefront; few: one, so that there are wavefronts enough
+#define PA_WIDE_U(T, EPL, U)                                                                                          \
+  {                                                                                                                   \
+    const int per = wide_heads<T, EPL, U>();                                                                          \
+    const long long wide_units = (long long)tokens * ((nh + nkv + per - 1) / per) + v_units;                          \
+    const unsigned wide_blocks = (unsigned)((wide_units + kQkWaves - 1) / kQkWaves);                                  \
+    hipLaunchKernelGGL((qknorm_rope_kv_wide_kernel<T, EPL, U>), dim3(wide_blocks), dim3(kQkWaves * kWave), 0, st,      \
+                       (const T*)qkv, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)q_out,          \
+                       (T*)k_cache, (T*)v_cache, tokens, nh, nkv, page_size, eps, vgroup);                            \
+  }
+#define PA_WIDE(T, EPL)          \
+  do {                           \
+    if (tokens >= 64) {          \
+      PA_WIDE_U(T, EPL, 5)       \
+    } else {                     \
+      PA_WIDE_U(T, EPL, 1)       \
+    }                            \
+  } while (0)
     if (dtype == kF32) {
       if (hd == 64) PA_WIDE(float, 1);
       else if (hd == 128) PA_WIDE(float, 2);
@@ -297,6 +345,7 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
       else PA_WIDE(bf16, 4);
     }
 #undef PA_WIDE
+#undef PA_WIDE_U
     return check_launch("qknorm_rope_kv");
   }
   if (dtype == kF32) {
