@@ -93,7 +93,7 @@ class Engine:
         # decode steps as HIP graphs: only for models whose layers keep nothing but pages (a mixer with
         # state of its own may run host code per step), and only in the serving type
         self._graphs = None
-        if config.hip_graph and not model.needs_state and self.dtype == torch.bfloat16:
+        if config.hip_graph and model.graph_safe and self.dtype == torch.bfloat16:
             from .graph import DecodeGraphs
             self._graphs = DecodeGraphs(self, config.hip_graph_max_bs)
 

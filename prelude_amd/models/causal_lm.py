@@ -111,6 +111,12 @@ class CausalLM:
     def needs_state(self) -> bool:
         return any(isinstance(c.spec, StateSpec) for c in self.cache_slots)
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step may be captured once and replayed: no state slots and no part that says no."""
+        return not self.needs_state and all(p.GRAPH_SAFE for p, _ in self._parts) \
+            and all(b.GRAPH_SAFE for b in self.blocks)
+
     # ---- forward ------------------------------------------------------------
     def forward(self, step, caches) -> torch.Tensor:
         """Runs the step's tokens; returns float32 logits [W, vocab] at ``step.want_rows``.

@@ -57,6 +57,11 @@ class StateSpec:
 class Part:
     """Base of all parts.  Subclasses take their sizes and constants as keyword parameters."""
 
+    # False for a part whose ``forward`` reads device results on the host or launches work that depends on
+    # them (rows routed by value, say): decode steps of a model with such a part are not replayed from HIP
+    # graphs.  A part that keeps state per request need not say so; its model is never captured.
+    GRAPH_SAFE = True
+
     def tensors(self) -> Dict[str, TensorReq]:
         """Local tensor name -> what is required of it."""
         return {}
