@@ -194,3 +194,38 @@ def test_overlapped_steps_change_no_token(gpu, tmp_path):
     assert all(len(o.token_ids) <= 30 and None not in o.token_ids for o in over)
     assert sync_llm.scheduler.preemptions > 0 and over_llm.scheduler.preemptions > 0
     assert over_llm.steps <= sync_llm.steps + 3
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_WORKLOADS", "6")))))   # widen for a hunt
+def test_drawn_workloads_change_no_token(gpu, seed):
+    """Requests, limits and cache sizes drawn at random: however the scheduler cuts, batches, evicts and overlaps,
+    every request gets the tokens it gets when it runs in an ample cache, greedy or with its own seeded draws."""
+    import numpy as np
+    from prelude_amd import LLM
+    from prelude_amd.sampling.sampler import SamplingParams
+    rng = np.random.default_rng(seed)
+    name = ["a", "b", "c"][seed % 3]
+    folder, cfg, _ = model_folder(name)
+    page = int(rng.choice([4, 8, 16]))
+    n = int(rng.integers(3, 11))
+    room = cfg["max_position_embeddings"]
+    lengths = [int(rng.integers(1, min(120, room - 45))) for _ in range(n)]
+    prompts = prompts_for(cfg, lengths, 50 + seed)
+    max_new = int(rng.integers(1, 41))
+    params = [SamplingParams(temperature=0.0) if rng.random() < 0.5 else
+              SamplingParams(temperature=float(rng.choice([0.6, 1.0])), top_k=int(rng.choice([0, 5])) or None,
+                             top_p=float(rng.choice([1.0, 0.9])), seed=int(rng.integers(0, 1000))) for _ in range(n)]
+    ample = LLM(folder, dtype="float32", page_size=page, max_cache_tokens=8192, overlap_steps=False)
+    want = ample.generate(prompts, max_tokens=max_new, sampling_params=params)
+    longest = -(-(max(lengths) + max_new) // page) * page
+    total = sum(-(-(m + max_new) // page) * page for m in lengths)
+    tight = LLM(folder, dtype="float32", page_size=page,
+                max_cache_tokens=int(rng.integers(longest + page, max(longest + 2 * page, total))),
+                decode_reservation_cap=int(rng.choice([0, 1, 8])), max_num_batched_tokens=int(rng.choice([16, 48, 128])),
+                long_prefill_token_threshold=int(rng.choice([0, 8, 32])), max_running_requests=int(rng.integers(2, 9)),
+                overlap_steps=bool(rng.integers(0, 2)))
+    got = tight.generate(prompts, max_tokens=max_new, sampling_params=params)
+    for i, (g, w_) in enumerate(zip(got, want)):
+        assert g.token_ids == w_.token_ids and g.finish_reason == w_.finish_reason, \
+            f"seed {seed}, request {i} of {n}: {g.token_ids} ({g.finish_reason}) against {w_.token_ids} ({w_.finish_reason})"
+    assert tight.engine.tables.audit() == "" and tight.engine.tables.num_requests() == 0
