@@ -8,7 +8,6 @@ import tempfile
 
 import numpy as np
 import pytest
-import torch
 
 import plain_model as pm
 from helpers import check
