@@ -54,8 +54,8 @@ _KERNEL_API = {
     "pa_attn_decode": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I]),
     "pa_attn_decode_fused": (I, [P, P, P, P, P, P, P, F, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I]),
     "pa_attn_decode_fused_supports": (I, [I, I, I, I, I]),
-    "pa_attn_prefill": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, F]),
-    "pa_attn_prefill_cut": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, I]),
+    "pa_attn_prefill": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F]),
+    "pa_attn_prefill_cut": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, I]),
     "pa_argmax_scratch": (I, [I, I]),
     "pa_argmax": (I, [P, P, P, P, I, I]),
     "pa_sample": (I, [P, P, P, P, P, P, P, I, I]),

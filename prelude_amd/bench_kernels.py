@@ -95,7 +95,7 @@ def bench_decode(dev, shape, page: int = 16) -> None:
 
 def bench_prefill(dev, shape, page: int = 16) -> None:
     _, _, nh, nkv, hd, _ = shape
-    for nseq, t, ctx in ((1, 512, 512), (4, 512, 512), (1, 2048, 2048), (1, 2048, 4096), (1, 8192, 8192)):
+    for nseq, t, ctx in ((1, 512, 512), (4, 512, 512), (16, 512, 512), (1, 2048, 2048), (1, 2048, 8192), (1, 8192, 8192)):
         pages = nseq * ctx // page
         kc = torch.randn(pages, nkv, page, hd, device=dev, dtype=torch.bfloat16)
         vc = torch.randn(pages, nkv, hd, page, device=dev, dtype=torch.bfloat16)
@@ -106,7 +106,7 @@ def bench_prefill(dev, shape, page: int = 16) -> None:
         lens = torch.full((nseq,), ctx, device=dev, dtype=torch.int32)
         out = torch.empty_like(q)
         scale = 1 / math.sqrt(hd)
-        us = timeit(lambda i: K.attention_prefill(q, kc, vc, table, seqs, cu, lens, out, t, 0, scale), 1, iters=20)
+        us = timeit(lambda i: K.attention_prefill(q, kc, vc, table, seqs, cu, lens, out, t, 0, scale, min_prefix=ctx - t), 1, iters=20)
         line(f"prefill attention, {nseq} x {t} tokens, context {ctx}", us, flops=2.0 * nseq * nh * hd * t * (2 * ctx - t))
 
 

@@ -72,13 +72,15 @@ int pa_attn_decode_fused(void* stream, const void* qkv, const float* q_weight, c
 int pa_attn_decode_fused_supports(int nh, int nkv, int hd, int rot, int page_size);
 int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                     int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                    int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window, float scale);
+                    int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd, int page_size, int window,
+                    float scale);
+// min_prefix: the fewest keys any sequence has before its portion (0 if unknown), a hint for the cut of the work.
 // The same with the cut of the work given (for tests and measurements): tiles in pairs, heads a wavefront (1, 2, 4),
 // head groups a workgroup (1, 2), keys staged in LDS; -1 leaves one to the launcher.
 int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                         int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                        int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window, float scale,
-                        int paired, int heads, int groups, int staged);
+                        int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd, int page_size, int window,
+                        float scale, int paired, int heads, int groups, int staged);
 
 // out[r] = index of the largest of logits[r, :], the lowest index among equals.
 // scratch: pa_argmax_scratch(rows, vocab) floats (none for narrow rows).

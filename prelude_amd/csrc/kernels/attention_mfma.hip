@@ -886,7 +886,8 @@ struct PrefillCut {
 template <int HD>
 int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
-                   int max_q_len, int nh, int nkv, int page_shift, int window, float scale, const PrefillCut& want) {
+                   int max_q_len, int min_prefix, int nh, int nkv, int page_shift, int window, float scale,
+                   const PrefillCut& want) {
   const int group = nh / nkv;
   // How the work is cut: tiles in pairs (an early and a late tile of the causal triangle, so workgroups finish
   // together) and as many heads per wavefront as share the keys and fit the registers (wider heads would not fit
@@ -895,28 +896,45 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // as 256 workgroups and 26 us as 64.
   const int gt_best = (HD <= 64 && group % 4 == 0) ? 4 : (group % 2 == 0 ? 2 : 1);
   const long tiles = (max_q_len + 63) / 64;
-  int paired = tiles >= 2, gt = gt_best;
-  auto workgroups = [&](int p, int g_) { return (p ? (tiles + 1) / 2 : tiles) * nkv * (group / g_) * nseq; };
+  const bool can_stage = page_shift >= 3 && page_shift <= 6;
+  auto workgroups = [&](int p, int g_, int h_ = 1) {
+    return (p ? (tiles + 1) / 2 : tiles) * nkv * (group / (g_ * h_)) * nseq;
+  };
   const long enough = 256;
-  if (workgroups(paired, gt) < enough) {
-    if (gt > 1 && workgroups(paired, 1) >= enough) {
-      gt = 1;
-    } else if (workgroups(0, gt) >= enough) {
-      paired = 0;
-    } else {
-      paired = 0;
-      gt = 1;
+  int paired = tiles >= 2, gt = gt_best, hw = 1;
+  // every portion has at least as many keys before it as tokens in it: its tiles see about the same number of keys
+  // and need no pairing, which doubles the workgroups there are to hand out
+  const bool level = min_prefix >= max_q_len;
+  const bool wide_ok = can_stage && group % (gt_best * 2) == 0;   // eight wavefronts: two groups of gt_best heads
+  if (wide_ok && workgroups(paired, gt_best, 2) >= enough) {
+    // the most work per staged key that still gives every compute unit a workgroup (measured at head_dim 128,
+    // 32 heads over 8: 4,096 tokens 171 against 186 us, 8,192 tokens 624 against 648)
+    hw = 2;
+  } else if (level && workgroups(0, gt_best, wide_ok ? 2 : 1) >= enough) {
+    paired = 0;   // 2,048 tokens behind 6,144: 297 against 342 us
+    hw = wide_ok ? 2 : 1;
+  } else if (level && can_stage && group % 2 == 0 && workgroups(0, 1, 2) >= enough) {
+    paired = 0, gt = 1, hw = 2;   // 1,024 tokens behind 7,168: 205 against 293 us
+  } else {
+    if (workgroups(paired, gt) < enough) {
+      if (gt > 1 && workgroups(paired, 1) >= enough) {
+        gt = 1;
+      } else if (workgroups(0, gt) >= enough) {
+        paired = 0;
+      } else {
+        paired = 0;
+        gt = 1;
+      }
+    }
+    // one workgroup per compute unit is one wavefront per SIMD, which waits for every one of its own steps: then
+    // rather eight wavefronts a workgroup, half of them on the other heads (measured at 2,048 tokens: 69 against 77 us)
+    if (can_stage && workgroups(paired, gt) >= enough && workgroups(paired, gt) < 2 * enough && gt >= 2 && gt == gt_best) {
+      gt /= 2;
+      hw = 2;
     }
   }
-  // one workgroup per compute unit is one wavefront per SIMD, which waits for every one of its own steps: then
-  // rather eight wavefronts a workgroup, half of them on the other heads (measured at 2,048 tokens: 69 against 77 us)
-  int hw = 1;
-  if (workgroups(paired, gt) >= enough && workgroups(paired, gt) < 2 * enough && gt >= 2 && gt == gt_best) {
-    gt /= 2;
-    hw = 2;
-  }
   // keys staged in LDS for pages of 8 to 64 keys; smaller and larger pages go to the kernel that reads them itself
-  bool staged = page_shift >= 3 && page_shift <= 6;
+  bool staged = can_stage;
   // a caller's own cut (tests and measurements), where it is one the kernels have
   if (want.paired >= 0) paired = want.paired != 0 && tiles >= 2;
   if (want.heads >= 0) {
@@ -1038,35 +1056,39 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
                                   max_splits, fq);
 }
 
+// min_prefix: the fewest keys any of the sequences has before its portion (0 if unknown): only a hint for how
+// the work is cut.
 // pa_attn_prefill with the cut given: paired (tiles in pairs), heads a wavefront (1, 2, 4), head groups a
 // workgroup (1, 2), staged (keys through LDS); -1 leaves one to the launcher.  A cut the shape does not take is
 // refused.  Every cut gives the same result up to rounding.
 extern "C" int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
-                                   void* out, int nseq, int max_q_len, int nh, int nkv, int hd, int page_size,
-                                   int window, float scale, int paired, int heads, int groups, int staged) {
+                                   void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
+                                   int page_size, int window, float scale, int paired, int heads, int groups,
+                                   int staged) {
   if (nseq == 0) return 0;
   if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
-  PA_REQUIRE(max_q_len >= 1, "attn_prefill: longest portion %d", max_q_len);
+  PA_REQUIRE(max_q_len >= 1 && min_prefix >= 0, "attn_prefill: longest portion %d, shortest prefix %d", max_q_len, min_prefix);
   PrefillCut cut;
   cut.paired = paired, cut.heads = heads, cut.groups = groups, cut.staged = staged;
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, nh, nkv, __builtin_ctz(page_size), window, scale, cut)
+                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, cut)
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
 
 extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                                int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
-                               void* out, int nseq, int max_q_len, int nh, int nkv, int hd, int page_size, int window,
-                               float scale) {
+                               void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
+                               int page_size, int window, float scale) {
   if (nseq == 0) return 0;
   if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
-  PA_REQUIRE(max_q_len >= 1, "attn_prefill: longest portion %d", max_q_len);
+  PA_REQUIRE(max_q_len >= 1 && min_prefix >= 0, "attn_prefill: longest portion %d, shortest prefix %d", max_q_len, min_prefix);
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, nh, nkv, __builtin_ctz(page_size), window, scale, PrefillCut{})
+                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale,           \
+                            PrefillCut{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }

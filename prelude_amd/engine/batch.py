@@ -46,6 +46,7 @@ class StepBatch:
     n_decode: int = 0
     n_prefill: int = 0
     max_prefill_q: int = 0       # longest portion among prefill_seqs
+    min_prefill_prefix: int = 0  # fewest tokens any of prefill_seqs has behind it already
     max_decode_context: int = 0  # longest context among decode_seqs
     page_size: int = 0
     graph: Optional[object] = None  # set while a step is being captured or replayed from fixed buffers

@@ -306,6 +306,7 @@ class Engine:
                          page_size=self.page_size,
                          decode_seqs=view("decode_seqs")[:len(dec)], prefill_seqs=view("prefill_seqs")[:len(pre)],
                          n_decode=len(dec), n_prefill=len(pre), max_prefill_q=max([counts[i] for i in pre], default=0),
+                         min_prefill_prefix=min([starts[i] for i in pre], default=0),
                          # with fixed buffers the launch shapes must not follow the data: bound by what the tables can hold
                          max_decode_context=(stride * self.page_size if fixed else max([ends[i] for i in dec], default=0)))
 

@@ -443,11 +443,13 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
 
 
 def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_q_len: int,
-                      window: int, scale: float, cut=None) -> None:
+                      window: int, scale: float, cut=None, min_prefix: int = 0) -> None:
     """Matrix-core attention for the sequences ``seq_ids`` (portions of several tokens); writes their rows of ``out``.
 
-    ``cut`` (tests and measurements) fixes how the launch is cut instead of leaving it to the launcher:
-    ``(paired, heads a wavefront, head groups a workgroup, staged)``, -1 for the launcher's choice."""
+    ``min_prefix`` is the fewest keys any of the sequences has before its portion: a hint for how the launcher
+    cuts the work (portions far into their contexts need no pairing of early and late tiles).
+    ``cut`` (tests and measurements) fixes the cut instead: ``(paired, heads a wavefront, head groups a
+    workgroup, staged)``, -1 for the launcher's choice."""
     _dev(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out)
     t, nh, hd = q.shape
     _check_caches(k_cache, v_cache, k_cache.shape[1], hd, torch.bfloat16, "attention_prefill")
@@ -455,8 +457,8 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_l
     if n == 0:
         return
     args = (_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_ids),
-            _ptr(cu_q), _ptr(context_lens), _ptr(out), n, int(max_q_len), nh, k_cache.shape[1], hd, k_cache.shape[2],
-            int(window), float(scale))
+            _ptr(cu_q), _ptr(context_lens), _ptr(out), n, int(max_q_len), int(min_prefix), nh, k_cache.shape[1], hd,
+            k_cache.shape[2], int(window), float(scale))
     if cut is None:
         check(kernels().pa_attn_prefill(*args))
     else:
@@ -480,7 +482,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
                              out, step.max_decode_context, window, scale)
         if step.n_prefill:
             attention_prefill(q, k_cache, v_cache, group.block_table, step.prefill_seqs, step.cu_q, step.context_lens,
-                              out, step.max_prefill_q, window, scale)
+                              out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix)
         return out
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
 

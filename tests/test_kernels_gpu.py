@@ -341,7 +341,8 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
         K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, out, max([seqs[i][0] for i in dec], default=0),
                              window, 1.0 / math.sqrt(hd))
         K().attention_prefill(qd, kd, vd, td, i32(pre), i32(cu), ctxs, out, max([seqs[i][1] for i in pre], default=0),
-                              window, 1.0 / math.sqrt(hd), cut=cut)
+                              window, 1.0 / math.sqrt(hd), cut=cut,
+                              min_prefix=min([seqs[i][0] - seqs[i][1] for i in pre], default=0))
         return out, torch.cat(refs)
     out = K().attention_generic(q.to(gpu), kc.to(dtype).to(gpu), vc.to(dtype).to(gpu), table.to(gpu),
                                 torch.tensor(seq_of, dtype=torch.int32, device=gpu),
@@ -459,6 +460,17 @@ def test_prefill_attention_every_cut(gpu, nh, nkv, hd, page, window):
                         base = out
                     # the cut moves no key to another block of 32: the same sums in the same order
                     assert torch.equal(out, base), (staged, paired, heads, groups)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page", [(32, 8, 128, 16), (16, 2, 64, 32), (4, 4, 128, 16)])
+def test_prefill_attention_far_into_its_context(gpu, nh, nkv, hd, page):
+    """Portions with long contexts behind them are cut without pairing and with wider workgroups (the launcher
+    goes by the shortest prefix and the number of workgroups); large enough here to take those branches."""
+    for seqs in ([(2304, 1024)], [(1500, 600), (3000, 1100)], [(4096, 2048)]):
+        out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, 0, seed=11, kernel="mfma")
+        close(out, ref, torch.bfloat16)
+        fixed, _ = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, 0, seed=11, kernel="mfma", cut=(1, 1, 1, 1))
+        assert torch.equal(out, fixed)
 
 
 def test_prefill_attention_refuses_a_cut_the_shape_does_not_take(gpu):
