@@ -7,10 +7,10 @@
 // over the whole vocabulary in 32-bit, keep the k largest, then keep the
 // shortest descending prefix whose mass reaches p, draw from what is left in
 // proportion to its weight.  The reference does this on the host with a
-// sorted copy; here one block per row finds the two thresholds by a bitwise
-// search over the order-preserving integer image of the floats (32 counting
-// passes each, all in cache), so nothing is sorted and nothing leaves the
-// device.  Entries equal to a threshold are all kept (a sort would keep some).
+// sorted copy; here one block per row finds the two thresholds by a search
+// over the order-preserving integer image of the floats, four bits a pass
+// (eight passes each over a row that stays in cache), so nothing is sorted
+// and nothing leaves the device.  Entries equal to a threshold are all kept (a sort would keep some).
 // The draw is the inverse CDF in index order at a uniform number the host
 // supplies per row, which makes it reproducible and testable.
 #include "common.h"
@@ -107,26 +107,127 @@ __device__ __forceinline__ unsigned order_key(float v) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-constexpr int kSampleThreads = 1024;
+// exp((x - mx) / T) as one hardware exponential: inv_t holds log2(e) / T.  (The library's expf is thirty
+// instructions; a pass over a row is bound by the vector units of the one compute unit that works on it.)
+__device__ __forceinline__ float weight_of(float x, float mx, float inv_t) {
+  return __builtin_amdgcn_exp2f((x - mx) * inv_t);
+}
 
-// Largest key t such that measure{ i : key_i >= t and key_i >= floor_key } >= target,
-// where measure counts entries (weights == false) or sums exp((x - mx) * inv_t).
+constexpr int kSampleThreads = 1024;
+constexpr int kSampleWaves = kSampleThreads / kWave;
+constexpr int kDigitBits = 4, kBuckets = 1 << kDigitBits;
+
+// What the block of a row shares.  `bins` gives every thread a column of its own per bucket, so the sums a
+// search pass takes are formed without atomics and in the same order whenever the row is the same.
+struct SampleLds {
+  float bins[kBuckets][kSampleThreads];
+  float red[kSampleWaves][kBuckets];
+  float wave_v[kSampleWaves];
+  int wave_i[kSampleWaves];
+  float scratch[16];
+  float pick_before;
+  int pick_range;
+};
+
+// f(value, index) for the entries begin + first, begin + first + stride, ... below end, `first` counted in
+// vectors of four when the stretch allows 16-byte loads (begin and the row 16-byte aligned) and in single
+// entries otherwise; eight loads are on their way before the first value is used.  One load in flight per
+// thread would make a pass over a 600 KB row 150 round trips to L2.
+template <typename F>
+__device__ __forceinline__ void walk(const float* row, int begin, int end, int first, int stride, F f) {
+  constexpr int U = 8;
+  const bool wide = (reinterpret_cast<size_t>(row + begin) & 15) == 0;
+  if (wide) {
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(row + begin);
+    const int n4 = (end - begin) / 4;
+    for (int b = first; b < n4; b += stride * U) {
+      f32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int idx = b + u * stride;
+        v[u] = idx < n4 ? r4[idx] : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int idx = b + u * stride;
+        if (idx < n4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f(v[u][e], begin + 4 * idx + e);
+        }
+      }
+    }
+    begin += 4 * n4;   // up to three entries are left
+  }
+  for (int b = begin + first; b < end; b += stride * U) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int idx = b + u * stride;
+      v[u] = idx < end ? row[idx] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int idx = b + u * stride;
+      if (idx < end) f(v[u], idx);
+    }
+  }
+}
+
+// Largest key t such that measure{ i : key_i >= t and key_i >= floor_key } >= target, where measure counts
+// entries (kWeights false) or sums the weights exp((x - mx) / T); 0 if even all entries measure less.  The key is
+// settled four bits at a time from the top: a pass over the row sorts the entries that agree with the bits
+// settled so far into the sixteen values of the next digit, and the largest digit whose entries, with all
+// above them, reach the target is taken.  Eight passes instead of one per bit.
 template <bool kWeights>
 __device__ unsigned threshold_search(const float* row, int vocab, unsigned floor_key, float target, float mx,
-                                     float inv_t, float* scratch) {
-  unsigned t = 0;
-  for (int bit = 31; bit >= 0; --bit) {
-    const unsigned cand = t | (1u << bit);
-    float acc = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-      const float x = row[i];
+                                     float inv_t, SampleLds& lds) {
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  unsigned prefix = 0;
+  float above = 0.f;   // measure of the entries whose settled bits are greater than the prefix's
+  for (int shift = 32 - kDigitBits; shift >= 0; shift -= kDigitBits) {
+#pragma unroll
+    for (int b = 0; b < kBuckets; ++b) lds.bins[b][tid] = 0.f;
+    const unsigned settled = shift + kDigitBits >= 32 ? 0u : ~0u << (shift + kDigitBits);
+    walk(row, 0, vocab, tid, kSampleThreads, [&](float x, int) {
       const unsigned k = order_key(x);
-      if (k >= cand && k >= floor_key) acc += kWeights ? expf((x - mx) * inv_t) : 1.0f;
+      if (k >= floor_key && (k & settled) == prefix)
+        lds.bins[(k >> shift) & (kBuckets - 1)][tid] += kWeights ? weight_of(x, mx, inv_t) : 1.0f;
+    });
+#pragma unroll
+    for (int b = 0; b < kBuckets; ++b) {
+      const float v = wave_sum(lds.bins[b][tid]);
+      if (lane == 0) lds.red[wave][b] = v;
     }
-    acc = block_sum(acc, scratch);
-    if (acc >= target) t = cand;
+    __syncthreads();
+    float run = above;
+    int digit = -1;
+    for (int b = kBuckets - 1; b >= 0; --b) {   // the same in every thread
+      float sb = 0.f;
+#pragma unroll
+      for (int w = 0; w < kSampleWaves; ++w) sb += lds.red[w][b];
+      if (digit < 0) {
+        if (run + sb >= target) {
+          digit = b;
+        } else {
+          run += sb;
+        }
+      }
+    }
+    __syncthreads();   // red is written again in the next pass
+    if (digit < 0) return 0u;
+    above = run;
+    prefix |= (unsigned)digit << shift;
   }
-  return t;
+  return prefix;
+}
+
+__device__ __forceinline__ float wave_scan_inclusive(float v, int lane) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const float o = __shfl_up(v, off, kWave);
+    if (lane >= off) v += o;
+  }
+  return v;
 }
 
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits, int vocab,
@@ -135,106 +236,133 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
                                                                 const float* __restrict__ top_p,
                                                                 const float* __restrict__ uniform,
                                                                 int* __restrict__ out) {
-  __shared__ float scratch[16];
-  __shared__ float sv[16];
-  __shared__ int si[16];
-  __shared__ float partial[kSampleThreads];
-  __shared__ int pick_thread;
-  __shared__ float pick_before;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  SampleLds& lds = *reinterpret_cast<SampleLds*>(lds_raw);
   const int r = blockIdx.x;
   const float* row = logits + (size_t)r * vocab;
   const float temp = temperature[r];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
 
   // maximum and its first index
   MaxIdx best{-INFINITY, 0x7fffffff};
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = row[i];
+  walk(row, 0, vocab, tid, kSampleThreads, [&](float v, int i) {
     if (v > best.v || (v == best.v && i < best.i)) best = MaxIdx{v, i};
-  }
+  });
 #pragma unroll
   for (int m = kWave / 2; m > 0; m >>= 1) {
     MaxIdx o{__shfl_xor(best.v, m, kWave), __shfl_xor(best.i, m, kWave)};
     best = better(best, o);
   }
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   if (lane == 0) {
-    sv[wave] = best.v;
-    si[wave] = best.i;
+    lds.wave_v[wave] = best.v;
+    lds.wave_i[wave] = best.i;
   }
   __syncthreads();
-  best = MaxIdx{sv[0], si[0]};
-  for (int w = 1; w < kSampleThreads / kWave; ++w) best = better(best, MaxIdx{sv[w], si[w]});
+  best = MaxIdx{lds.wave_v[0], lds.wave_i[0]};
+  for (int w = 1; w < kSampleWaves; ++w) best = better(best, MaxIdx{lds.wave_v[w], lds.wave_i[w]});
   const int arg = best.i == 0x7fffffff ? 0 : best.i;
   if (!(temp >= 1e-7f)) {  // greedy (crates/prelude-core/src/engine/model_runner/postprocess.rs:18-37)
-    if (threadIdx.x == 0) out[r] = arg;
+    if (tid == 0) out[r] = arg;
     return;
   }
-  const float mx = best.v, inv_t = 1.0f / temp;
+  const float mx = best.v, inv_t = 1.4426950408889634f / temp;
+  __syncthreads();   // wave_v and wave_i are used again below
 
   unsigned floor_key = 0;
   const int k = top_k[r];
-  if (k > 0 && k < vocab) floor_key = threshold_search<false>(row, vocab, 0u, (float)k, mx, inv_t, scratch);
+  if (k > 0 && k < vocab) floor_key = threshold_search<false>(row, vocab, 0u, (float)k, mx, inv_t, lds);
 
   const float p = top_p[r];
   if (p > 0.f && p < 1.f) {
     float z = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) z += expf((row[i] - mx) * inv_t);
-    z = block_sum(z, scratch);
-    const unsigned t = threshold_search<true>(row, vocab, floor_key, p * z, mx, inv_t, scratch);
+    walk(row, 0, vocab, tid, kSampleThreads, [&](float x, int) { z += weight_of(x, mx, inv_t); });
+    z = block_sum(z, lds.scratch);
+    const unsigned t = threshold_search<true>(row, vocab, floor_key, p * z, mx, inv_t, lds);
     // t == 0 means even everything kept so far weighs less than p: keep it all
     if (t > floor_key) floor_key = t;
   }
 
-  // inverse CDF over the kept entries in index order; each thread owns a contiguous run
-  const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
-  const int begin = threadIdx.x * chunk;
-  const int end = begin + chunk < vocab ? begin + chunk : vocab;
-  float mine = 0.f;
-  for (int i = begin; i < end; ++i) {
-    const float x = row[i];
-    if (order_key(x) >= floor_key) mine += expf((x - mx) * inv_t);
-  }
-  partial[threadIdx.x] = mine;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float total = 0.f;
-    for (int t = 0; t < kSampleThreads; ++t) total += partial[t];
-    const float target = uniform[r] * total;
-    float before = 0.f;
-    int who = -1, last_nonzero = 0;
-    for (int t = 0; t < kSampleThreads; ++t) {
-      if (partial[t] > 0.f) last_nonzero = t;
-      if (who < 0 && before + partial[t] > target) {
-        who = t;
-        pick_before = before;
+  // The draw: the first index, in index order, at which the running weight of the kept entries passes
+  // uniform * total.  The row is cut into a stretch per wavefront, then the stretch that holds the target
+  // into a stretch per wavefront again, and the last one is walked 64 entries at a time with a prefix sum.
+  auto weight = [&](float x) { return order_key(x) >= floor_key ? weight_of(x, mx, inv_t) : 0.f; };
+  constexpr int kLast = 16 * kWave;   // a stretch this short is walked by one wavefront
+  int begin = 0, end = vocab;
+  float before = 0.f, target = 0.f;
+  int fallback = arg;   // the last kept entry of the stretch in hand, for a target that rounding puts past it
+  for (int level = 0; level == 0 || end - begin > kLast; ++level) {
+    const int span = ((end - begin + kSampleWaves * kWave - 1) / (kSampleWaves * kWave)) * kWave;   // per wavefront
+    const int wb = begin + wave * span < end ? begin + wave * span : end;
+    const int we = wb + span < end ? wb + span : end;
+    float sum = 0.f;
+    int last = -1;
+    walk(row, wb, we, lane, kWave, [&](float x, int i) {
+      const float wgt = weight(x);
+      sum += wgt;
+      if (wgt > 0.f && i > last) last = i;
+    });
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) {
+      const int o = __shfl_xor(last, m, kWave);
+      last = o > last ? o : last;
+    }
+    if (lane == 0) {
+      lds.wave_v[wave] = sum;
+      lds.wave_i[wave] = last;
+    }
+    __syncthreads();
+    if (level == 0) {
+      float total = 0.f;
+      for (int w = 0; w < kSampleWaves; ++w) total += lds.wave_v[w];
+      target = uniform[r] * total;
+    }
+    int pick = -1;
+    float run = before;
+    int last_kept = -1;
+    for (int w = 0; w < kSampleWaves; ++w) {   // the same in every thread
+      if (lds.wave_i[w] > last_kept) last_kept = lds.wave_i[w];
+      if (pick < 0) {
+        if (run + lds.wave_v[w] > target) {
+          pick = w;
+        } else {
+          run += lds.wave_v[w];
+        }
       }
-      if (who < 0) before += partial[t];
     }
-    if (who < 0) {  // rounding left the target at or past the total: the last kept entry
-      who = last_nonzero;
-      pick_before = -1.f;
+    if (last_kept < 0) last_kept = fallback;
+    const int pick_last = pick >= 0 ? lds.wave_i[pick] : -1;
+    __syncthreads();   // wave_v and wave_i are written again at the next level
+    if (pick < 0) {   // rounding left the target at or past the total: the last kept entry
+      if (tid == 0) out[r] = last_kept;
+      return;
     }
-    pick_thread = who;
-    scratch[0] = target;
+    before = run;
+    fallback = pick_last >= 0 ? pick_last : fallback;
+    begin = begin + pick * span;
+    end = begin + span < end ? begin + span : end;
   }
-  __syncthreads();
-  if ((int)threadIdx.x == pick_thread) {
-    const float target = scratch[0];
-    float cum = pick_before;
-    int chosen = -1, last_kept = arg;
-    for (int i = begin; i < end; ++i) {
-      const float x = row[i];
-      if (order_key(x) < floor_key) continue;
-      last_kept = i;
-      if (pick_before < 0.f) continue;
-      cum += expf((x - mx) * inv_t);
-      if (cum > target) {
-        chosen = i;
-        break;
-      }
-    }
-    out[r] = chosen >= 0 ? chosen : last_kept;
+  if (wave != 0) return;
+  // at most sixteen groups of 64 entries, all asked for at once, then a prefix sum per group
+  float wgt[kLast / kWave];
+#pragma unroll
+  for (int j = 0; j < kLast / kWave; ++j) {
+    const int i = begin + j * kWave + lane;
+    wgt[j] = i < end ? row[i] : -INFINITY;
   }
+  float cum = before;
+#pragma unroll
+  for (int j = 0; j < kLast / kWave; ++j) {
+    if (begin + j * kWave >= end) break;
+    const float c = cum + wave_scan_inclusive(wgt[j] == -INFINITY ? 0.f : weight(wgt[j]), lane);
+    const unsigned long long hit = __ballot(c > target);
+    if (hit) {
+      if (lane == 0) out[r] = begin + j * kWave + __builtin_ctzll(hit);
+      return;
+    }
+    cum = __shfl(c, kWave - 1, kWave);
+  }
+  if (lane == 0) out[r] = fallback;
 }
 
 }  // namespace pa
@@ -245,8 +373,14 @@ extern "C" int pa_sample(void* stream, const float* logits, const float* tempera
                          const float* top_p, const float* uniform, int* out, int rows, int vocab) {
   if (rows == 0) return 0;
   PA_REQUIRE(rows > 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, (hipStream_t)stream, logits, vocab,
-                     temperature, top_k, top_p, uniform, out);
+  // the per-thread bins are more than the 64 KB a kernel may declare: asked for at launch, allowed once
+  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&sample_kernel),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                        (int)sizeof(SampleLds));
+  if (allowed != hipSuccess)
+    return pa::fail("sample: %zu bytes of LDS refused: %s", sizeof(SampleLds), hipGetErrorString(allowed));
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), sizeof(SampleLds), (hipStream_t)stream, logits,
+                     vocab, temperature, top_k, top_p, uniform, out);
   return check_launch("sample");
 }
 
