@@ -91,6 +91,11 @@ int pa_argmax(void* stream, const float* logits, int* out, float* scratch, int r
 // (0 = all) and to the shortest descending prefix of mass top_p (>= 1 = all), at the uniform number uniform[r] in [0, 1).
 int pa_sample(void* stream, const float* logits, const float* temperature, const int* top_k, const float* top_p,
               const float* uniform, int* out, int rows, int vocab);
+// The same choice for long rows with every pass spread over the chip; modes: bit 0 some row may have a top-k,
+// bit 1 some row may have a top-p.  workspace: pa_sample_wide_workspace(rows, vocab) bytes, 16-byte aligned.
+long pa_sample_wide_workspace(int rows, int vocab);
+int pa_sample_wide(void* stream, const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                   const float* uniform, int* out, void* workspace, int rows, int vocab, int modes);
 
 #ifdef __cplusplus
 }

@@ -487,13 +487,23 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
 
 
+SAMPLE_WIDE_FROM = 32768   # rows this long are sampled with every pass spread over the chip,
+SAMPLE_WIDE_ROWS = 32      # up to this many at a time (more rows fill the chip with a workgroup each)
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor) -> torch.Tensor:
+           uniform: torch.Tensor, any_top_k: bool = True, any_top_p: bool = True,
+           wide: Optional[bool] = None) -> torch.Tensor:
     """One token per row of float32 logits [R, V]; per-row float32 temperature / top_p / uniform and int32 top_k.
 
     temperature < 1e-7: argmax.  Else a draw from softmax(logits / T) kept to the
     top_k largest (0 = all) and the shortest descending prefix of mass top_p
     (>= 1 = all), by inverse CDF in index order at uniform[r] in [0, 1).
+
+    ``any_top_k`` / ``any_top_p`` false promise that no row has one, which spares long rows the passes of
+    that search.  ``wide`` picks the kernel (one workgroup a row, or rows cut into slices over many
+    workgroups); by default it follows the row length.  Both give the same token except where 32-bit
+    rounding of the sums decides between neighbours.
     """
     _dev(logits, temperature, top_k, top_p, uniform)
     _f32(logits, "logits")
@@ -505,6 +515,15 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if logits.dim() != 2 or any(t.shape != (r,) for t in (temperature, top_k, top_p, uniform)):
         raise NativeError("sample: per-row parameters do not match the rows of logits")
     out = torch.empty((r,), dtype=torch.int32, device=logits.device)
+    vocab = logits.shape[1]
+    if wide is None:
+        wide = vocab >= SAMPLE_WIDE_FROM and r <= SAMPLE_WIDE_ROWS
+    if wide and r > 0:
+        ws = torch.empty(int(kernels().pa_sample_wide_workspace(r, vocab)), dtype=torch.uint8, device=logits.device)
+        check(kernels().pa_sample_wide(_stream(), _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                       _ptr(uniform), _ptr(out), _ptr(ws), r, vocab,
+                                       (1 if any_top_k else 0) | (2 if any_top_p else 0)))
+        return out
     check(kernels().pa_sample(_stream(), _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
-                              _ptr(out), r, logits.shape[1]))
+                              _ptr(out), r, vocab))
     return out

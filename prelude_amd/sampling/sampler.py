@@ -81,7 +81,9 @@ def sample_rows_device(logits: torch.Tensor, samplers: Sequence[RequestSampler])
         kv[i] = p.top_k or 0
     dev = host.to(logits.device, non_blocking=True)
     dk = topk.to(logits.device, non_blocking=True)
-    return K.sample(logits, dev[0], dk, dev[1], dev[2])
+    return K.sample(logits, dev[0], dk, dev[1], dev[2],
+                    any_top_k=any((s.params.top_k or 0) > 0 for s in samplers if not s.params.greedy),
+                    any_top_p=any(0.0 < s.params.top_p < 1.0 for s in samplers if not s.params.greedy))
 
 
 def sample_rows(logits: torch.Tensor, samplers: Sequence[RequestSampler]) -> List[int]:

@@ -584,8 +584,9 @@ def test_argmax(gpu):
     assert K().argmax(big.to(gpu)).tolist()[2] == 7
 
 
-@pytest.mark.parametrize("vocab", [509, 151936])
-def test_sample_matches_the_plain_draw(gpu, vocab):
+@pytest.mark.parametrize("vocab,wide", [(509, False), (509, True), (151936, False), (151936, True), (40001, True)])
+def test_sample_matches_the_plain_draw(gpu, vocab, wide):
+    """Both sampling kernels (a workgroup a row; rows cut into slices over many workgroups) against the plain draw."""
     g = torch.Generator().manual_seed(3)
     rows = 24
     logits = 3.0 * torch.randn(rows, vocab, generator=g)
@@ -594,7 +595,7 @@ def test_sample_matches_the_plain_draw(gpu, vocab):
     topp = [1.0, 1.0, 1.0, 0.9, 0.5, 0.95] * 4
     u = torch.rand(rows, generator=g)
     out = K().sample(logits.to(gpu), torch.tensor(temps).to(gpu), torch.tensor(topk, dtype=torch.int32).to(gpu),
-                     torch.tensor(topp).to(gpu), u.to(gpu)).tolist()
+                     torch.tensor(topp).to(gpu), u.to(gpu), wide=wide).tolist()
     checked = 0
     for r in range(rows):
         if temps[r] < 1e-7:
@@ -609,6 +610,24 @@ def test_sample_matches_the_plain_draw(gpu, vocab):
             assert out[r] == pm.draw(prs, float(u[r])), f"row {r}"
             checked += 1
     assert checked >= rows // 2
+
+
+@pytest.mark.parametrize("rows", [1, 3, 70])
+def test_sample_wide_takes_only_the_searches_it_is_told_of(gpu, rows):
+    """Rows cut into 64, 64 and 14 slices; without top-k and top-p rows the searches are left out, and the
+    tokens are those of the one-workgroup kernel (uniform numbers away from the boundaries)."""
+    g = torch.Generator().manual_seed(rows)
+    vocab = 70001
+    logits = (2.0 * torch.randn(rows, vocab, generator=g)).to(gpu)
+    u = (0.05 + 0.9 * torch.rand(rows, generator=g)).to(gpu)
+    full = lambda v, dt=torch.float32: torch.full((rows,), v, dtype=dt).to(gpu)
+    for k, p in ((0, 1.0), (40, 1.0), (0, 0.8), (40, 0.8)):
+        args = (logits, full(0.9), full(k, torch.int32), full(p), u)
+        one = K().sample(*args, wide=False)
+        many = K().sample(*args, any_top_k=k > 0, any_top_p=p < 1.0, wide=True)
+        told_more = K().sample(*args, wide=True)
+        assert torch.equal(many, told_more)
+        assert int((one != many).sum()) <= max(1, rows // 20), (k, p, one.tolist(), many.tolist())
 
 
 def test_sample_statistics_and_limits(gpu):
