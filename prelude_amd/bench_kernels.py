@@ -1,6 +1,6 @@
 """Times single kernels against their rooflines on one MI355X.
 
-    python -m prelude_amd.bench_kernels [gemm] [decode] [prefill] [elementwise] [--shape 4b|8b|32b]
+    python -m prelude_amd.bench_kernels [gemm] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
 
 Each line gives the kernel's time (device events around repeated launches,
 operands rotated over copies larger than the caches where the kernel streams
@@ -130,9 +130,22 @@ def bench_elementwise(dev, shape, page: int = 16) -> None:
              nbytes=t * (nh * 2 + nkv * 4) * hd * 2)
 
 
+def bench_sampling(dev, shape) -> None:
+    vocab = shape[5]
+    for rows in (1, 8, 64):
+        logits = torch.randn(rows, vocab, device=dev) * 3
+        u = torch.rand(rows, device=dev)
+        full = lambda v, dt=torch.float32: torch.full((rows,), v, dtype=dt, device=dev)
+        line(f"argmax, {rows} rows of {vocab}", timeit(lambda i: K.argmax(logits), 1), nbytes=rows * vocab * 4)
+        for name, k, p in (("temperature", 0, 1.0), ("top-p 0.9", 0, 0.9), ("top-k 50", 50, 1.0), ("top-k 50, top-p 0.9", 50, 0.9)):
+            args = (logits, full(0.7), full(k, torch.int32), full(p), u)
+            us = timeit(lambda i: K.sample(*args, any_top_k=k > 0, any_top_p=p < 1.0), 1)
+            line(f"draw, {rows} rows, {name}", us)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
-    ap.add_argument("what", nargs="*", help="gemm, decode, prefill, elementwise (default: all)")
+    ap.add_argument("what", nargs="*", help="gemm, decode, prefill, elementwise, sampling (default: all)")
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -140,11 +153,12 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     shape = SHAPES[args.shape]
-    todo = args.what or ["gemm", "decode", "prefill", "elementwise"]
+    todo = args.what or ["gemm", "decode", "prefill", "elementwise", "sampling"]
     print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
           f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
     for name in todo:
-        {"gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise}[name](dev, shape)
+        {"gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
+         "sampling": bench_sampling}[name](dev, shape)
     return 0
 
 
