@@ -241,9 +241,11 @@ def main() -> int:
                     help="time a step of one --prefill-tokens portion beside 63 decoding requests at contexts up to "
                          "--context, and print its record")
     ap.add_argument("--requests", type=int, default=0,
-                    help="time this many 512-token prompts with one new token each through LLM.generate, "
-                         "--concurrency at a time, and print the record")
+                    help="time this many prompts (--prompt-len tokens, --new-tokens new tokens each) through "
+                         "LLM.generate, --concurrency at a time, and print the record")
     ap.add_argument("--concurrency", type=int, default=96)
+    ap.add_argument("--prompt-len", type=int, default=512, help="prompt length of --requests")
+    ap.add_argument("--new-tokens", type=int, default=1, help="new tokens per request of --requests")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus, flush=True)
@@ -267,11 +269,13 @@ def main() -> int:
               flush=True)
         return 0
     if args.requests:
-        total, calls = time_requests(raw, args.dtype, args.requests, 512, 1, args.concurrency)
+        total, calls = time_requests(raw, args.dtype, args.requests, args.prompt_len, args.new_tokens, args.concurrency)
         calls.sort()
-        print(json.dumps({"model": name, "workload": f"{args.requests} prompts of 512 tokens, 1 new token, "
-                          f"{args.concurrency} at a time (LLM.generate, no HTTP)",
-                          "req_per_s": round(args.requests / total, 1), "tok_per_s": round(args.requests * 512 / total, 1),
+        print(json.dumps({"model": name, "workload": f"{args.requests} prompts of {args.prompt_len} tokens, "
+                          f"{args.new_tokens} new token(s), {args.concurrency} at a time (LLM.generate, no HTTP)",
+                          "req_per_s": round(args.requests / total, 1),
+                          "prompt_tok_per_s": round(args.requests * args.prompt_len / total, 1),
+                          "new_tok_per_s": round(args.requests * args.new_tokens / total, 1),
                           "call_ms_p50": round(calls[len(calls) // 2] * 1e3, 2)}), flush=True)
         return 0
     if args.prefill_only:
