@@ -219,8 +219,14 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
 
 
 SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel itself takes up to 64) ...
-TILED_MAX_ROWS = 48    # ... except for small weights in tiles: measured at [6144, 2560] and [2560, 4096], the
-TILED_SMALL_WEIGHT = 1 << 24   # streaming kernel wins up to 48 rows (11 against 19 us at 32), loses for larger weights
+# ... except for small weights in tiles, where the library's 19 us floor is what it takes: (rows, elements) up to
+# which the streaming kernel measured faster -- [6144, 2560] and [2560, 4096] to 48 rows (11 against 19 us at 32),
+# [6144, 4096] to 32 rows (15 against 19 us); weights beyond that, and rows of 8192 columns or more, go to the library
+TILED_LIMITS = ((48, 1 << 24), (32, 1 << 25))
+
+
+def _tiled_beyond_16(m: int, n: int, k: int) -> bool:
+    return k < 8192 and k % 8 == 0 and any(m <= rows and n * k <= size for rows, size in TILED_LIMITS)
 
 
 class TiledWeight:
@@ -314,7 +320,7 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     m, k = x.shape
     if m <= SKINNY_MAX_ROWS and k % 8 == 0:
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
-    if tiles is not None and m <= TILED_MAX_ROWS and w.shape[0] * k <= TILED_SMALL_WEIGHT and k < 8192 and k % 8 == 0:
+    if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
     y = torch.matmul(x, w.t())
     if bias is not None:
