@@ -41,7 +41,7 @@ int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, cons
 
 // C[m, n] = X[m, k] W[n, k]^T for m <= 64 in bfloat16 (32-bit accumulation); out_dtype 0 = float32, 1 = bfloat16.
 // epilogue 0: (+ bias[n]); 1: C[m, n/2] = silu(gate) * up for a weight whose rows alternate gate_j, up_j.
-// tiled 1: w is the weight as pa_pack_tiles lays it out (more than 16 rows then only for k < 8192).
+// tiled 1: w is the weight as pa_pack_tiles lays it out.
 int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
                    int m, int n, int k, long ldx, long ldc, int tiled);
 // out[tile][step][half][g][r][8] = w[16 tile + r][64 step + 16 g + 8 half ..], zero-padded: ceil(n/16) * ceil(k/64) * 1024 elements.

@@ -209,6 +209,10 @@ static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* 
     if (m > 8 && tiles >= 384) *nt *= 2;
     if (mt > 1 && *nt > 2) *nt = 2;
     *waves = steps >= 128 ? 16 : 8;
+    if (mt > 1 && steps >= 128) {   // more than 16 rows of a long weight: the sums of 16 wavefronts would not fit LDS
+      *waves = 8;
+      if (tiles >= 256) *nt = 2;    // and X, as long as the weight's rows, is worth sharing over two tiles
+    }
     *depth = 1;
     return;
   }
@@ -306,7 +310,7 @@ extern "C" int pa_pack_tiles(void* stream, const void* w, void* out, int n, int 
   return check_launch("pack_tiles");
 }
 
-// tiled 1: w is the weight in tiles (pa_pack_tiles); more than 16 rows then only for k < 8192.
+// tiled 1: w is the weight in tiles (pa_pack_tiles).
 extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w,
                               const float* bias, void* c, int m, int n, int k, long ldx, long ldc, int tiled) {
   if (m == 0 || n == 0) return 0;
@@ -317,8 +321,6 @@ extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const v
   PA_REQUIRE(epilogue == kPlain || (n % 2 == 0 && !bias), "gemm_skinny: the SiLU*up epilogue needs an even n and no bias");
   PA_REQUIRE(ldc >= (epilogue == kSiluMul ? n / 2 : n), "gemm_skinny: output row stride %ld is too small", ldc);
 
-  PA_REQUIRE(!tiled || m <= 16 || k < 128 * 64,
-             "gemm_skinny: a tiled weight with %d columns takes at most 16 rows, not %d", k, m);
   hipStream_t st = (hipStream_t)stream;
   if (epilogue == kPlain && out_dtype == kBF16)
     return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);

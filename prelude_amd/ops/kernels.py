@@ -221,12 +221,19 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = 
 SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel itself takes up to 64) ...
 # ... except for small weights in tiles, where the library's 19 us floor is what it takes: (rows, elements) up to
 # which the streaming kernel measured faster -- [6144, 2560] and [2560, 4096] to 48 rows (11 against 19 us at 32),
-# [6144, 4096] to 32 rows (15 against 19 us); weights beyond that, and rows of 8192 columns or more, go to the library
+# [6144, 4096] to 32 rows (15 against 19 us); weights beyond that go to the library, as do rows of 8192 columns or
+# more -- unless they are very long: [5120, 25600] takes the library 143 to 155 us at 24 to 64 rows, the streaming
+# kernel 67 to 118
 TILED_LIMITS = ((48, 1 << 24), (32, 1 << 25))
+TILED_LONG_ROWS = 16384
 
 
 def _tiled_beyond_16(m: int, n: int, k: int) -> bool:
-    return k < 8192 and k % 8 == 0 and any(m <= rows and n * k <= size for rows, size in TILED_LIMITS)
+    if k % 8:
+        return False
+    if k >= TILED_LONG_ROWS:
+        return m <= 64
+    return k < 8192 and any(m <= rows and n * k <= size for rows, size in TILED_LIMITS)
 
 
 class TiledWeight:
@@ -283,7 +290,7 @@ def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False) -> torch.Tensor:
     """x [M <= 64, K] @ w[N, K]^T in bfloat16 on the matrix cores, streaming w once.
 
-    ``w`` is a tensor [N, K] or a ``TiledWeight`` (then more than 16 rows only for K < 8192).  With
+    ``w`` is a tensor [N, K] or a ``TiledWeight``.  With
     ``silu_mul_epilogue`` the rows of w alternate gate_j, up_j and the
     result is silu(gate) * up, [M, N/2]."""
     tiled = isinstance(w, TiledWeight)
