@@ -72,6 +72,14 @@ def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides
     return Engine(model, cfg, raw)
 
 
+def release_memory():
+    """An engine and its captured graphs refer to one another: collect the cycle before the next engine is built."""
+    import gc
+    import torch
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
 def weight_bytes(raw, el):
     h, i, v = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
     nh, nkv, hd, L = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"], raw["num_hidden_layers"]
@@ -141,7 +149,7 @@ def decode_point(raw, dtype, batch, context, steps, warmup, layers_note):
     prefill_requests(eng, batch, context - total, 2048, raw["vocab_size"], seed=batch)
     sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"])
     del eng
-    torch.cuda.empty_cache()
+    release_memory()
     return sec
 
 
@@ -163,7 +171,7 @@ def time_prefill(raw, dtype, tokens, reps):
         if r > 0:
             best = dt if best is None else min(best, dt)
     del eng
-    torch.cuda.empty_cache()
+    release_memory()
     return best
 
 
@@ -199,7 +207,7 @@ def time_mixed(raw, dtype, chunk, decoding, context, steps, warmup):
         times.append(time.perf_counter() - t0)
         eng.release(big)
     del eng
-    torch.cuda.empty_cache()
+    release_memory()
     return sum(times[warmup:]) / steps
 
 

@@ -209,9 +209,12 @@ static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* 
     if (m > 8 && tiles >= 384) *nt *= 2;
     if (mt > 1 && *nt > 2) *nt = 2;
     *waves = steps >= 128 ? 16 : 8;
-    if (mt > 1 && steps >= 128) {   // more than 16 rows of a long weight: the sums of 16 wavefronts would not fit LDS
+    if (steps >= 128 && (mt > 1 || tiles >= 320)) {
+      // long rows: 16 wavefronts' sums of more than 16 rows would not fit LDS, and where there are tiles enough,
+      // eight wavefronts on two tiles stream better than sixteen on one ([5120, 25600] at 1 / 8 / 16 rows:
+      // 52 / 51 / 57 against 55 / 60 / 83 us; [4096, 12288], 256 tiles, is still better off with sixteen on one)
       *waves = 8;
-      if (tiles >= 256) *nt = 2;    // and X, as long as the weight's rows, is worth sharing over two tiles
+      if (tiles >= 320) *nt = 2;
     }
     *depth = 1;
     return;
