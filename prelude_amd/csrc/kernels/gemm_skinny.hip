@@ -206,7 +206,7 @@ static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* 
     // (how K is split over wavefronts fixes the order of the sums and follows the weight alone; the tiles per
     // workgroup do not touch it, and more than 8 rows read X often enough that sharing it over two tiles pays)
     *nt = tiles >= 4096 ? 2 : 1;
-    if (m > 8 && tiles >= 384) *nt *= 2;
+    if (m > 8 && tiles >= 320) *nt *= 2;   // [5120, 5120] at 16 rows: 14 against 19 us
     if (mt > 1 && *nt > 2) *nt = 2;
     *waves = steps >= 128 ? 16 : 8;
     if (steps >= 128 && (mt > 1 || tiles >= 320)) {
