@@ -40,10 +40,10 @@ def build_parser() -> argparse.ArgumentParser:
     g = ap.add_mutually_exclusive_group()
     g.add_argument("--cuda-graph", "--hip-graph", dest="hip_graph", action="store_true", default=True)
     g.add_argument("--no-cuda-graph", "--no-hip-graph", dest="hip_graph", action="store_false")
-    g.add_argument("--no-weight-tiles", dest="weight_tiles", action="store_false", default=True,
-                   help="keep no second, tiled copy of the weights for decode steps (saves their memory)")
-    g.add_argument("--no-overlap-steps", dest="overlap_steps", action="store_false", default=True,
-                   help="wait for every step's token ids before scheduling the next step")
+    ap.add_argument("--no-weight-tiles", dest="weight_tiles", action="store_false", default=True,
+                    help="keep no second, tiled copy of the weights for decode steps (saves their memory)")
+    ap.add_argument("--no-overlap-steps", dest="overlap_steps", action="store_false", default=True,
+                    help="wait for every step's token ids before scheduling the next step")
     # the request
     ap.add_argument("--prompt", action="append", default=[], help="text prompt (needs tokenizer.json); repeatable")
     ap.add_argument("--prompt-ids", action="append", default=[], help="comma-separated token ids; repeatable")
@@ -55,6 +55,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--top-k", type=int, default=None)
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--stop-token-ids", default="", help="comma-separated token ids that end a request")
+    ap.add_argument("--stop", action="append", default=[], help="a string that ends a request (needs tokenizer.json); "
+                                                                 "repeatable")
     return ap
 
 
@@ -102,7 +104,7 @@ def main(argv=None) -> int:
         return 2
     stop = [int(x) for x in args.stop_token_ids.split(",") if x.strip()]
     outs = llm.generate(prompts, max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
-                        top_k=args.top_k, seed=args.seed, stop_token_ids=stop)
+                        top_k=args.top_k, seed=args.seed, stop_token_ids=stop, stop=args.stop)
     for o in outs:
         rec = {"request_id": o.request_id, "token_ids": o.token_ids, "finish_reason": o.finish_reason,
                "usage": o.usage, "metrics": {k: round(v, 3) for k, v in o.metrics.items()}}

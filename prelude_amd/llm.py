@@ -59,6 +59,7 @@ class _Live:
     sampler: RequestSampler
     stop_ids: frozenset
     t_arrive: float
+    stop_strings: tuple = ()
     t_first: Optional[float] = None
     finish_reason: Optional[str] = None
     pending_row: Optional[int] = None    # the last of ``tokens`` is still on the device: its row among the step's samples
@@ -131,19 +132,28 @@ class LLM:
     def generate(self, prompts: Union[Prompt, Sequence[Prompt]], max_tokens: int = DEFAULT_MAX_TOKENS,
                  temperature: float = 0.7, top_p: float = 1.0, top_k: Optional[int] = None,
                  seed: Optional[int] = None, stop_token_ids: Iterable[int] = (),
-                 sampling_params: Optional[Sequence[SamplingParams]] = None) -> List[GenerationResult]:
+                 sampling_params: Optional[Sequence[SamplingParams]] = None,
+                 stop: Iterable[str] = ()) -> List[GenerationResult]:
         """Runs all prompts to their end with continuous batching; results in the order of the prompts.
 
         ``sampling_params`` gives each prompt options of its own and overrides
         temperature/top_p/top_k/seed.  A request ends on an EOS id of the
-        model (``eos``), on one of ``stop_token_ids`` (``stop``), or after
-        ``max_tokens`` tokens, clamped to the positions the model has left (``length``).
+        model (``eos``), on one of ``stop_token_ids`` (``stop``), after
+        ``max_tokens`` tokens, clamped to the positions the model has left (``length``),
+        or once its text holds one of the strings ``stop`` (``stop``; needs the
+        folder's tokenizer.json; the text returned ends before the string, the
+        token ids keep the tokens that spelt it:
+        crates/prelude-core/src/engine/run/ar.rs:1560-1577,
+        crates/prelude-core/src/engine/model_runner/postprocess.rs:5-16).
         """
         single = isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int))
         plist = [prompts] if single else list(prompts)
         if sampling_params is not None and len(sampling_params) != len(plist):
             raise ValueError("sampling_params must have one entry per prompt")
-        stop = frozenset(int(t) for t in stop_token_ids)
+        stop_ids = frozenset(int(t) for t in stop_token_ids)
+        stop_strings = tuple(s for s in ([stop] if isinstance(stop, str) else stop) if s)
+        if stop_strings:
+            self.tokenizer()
         live: Dict[int, _Live] = {}
         results: List[Optional[GenerationResult]] = [None] * len(plist)
         now = time.perf_counter()
@@ -163,7 +173,7 @@ class LLM:
             rid = self._next_id
             self._next_id += 1
             self.scheduler.add_request(rid, len(ids), max_new)
-            live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop, now)
+            live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop_ids, now, stop_strings)
 
         overlap = bool(self.config.overlap_steps)
         in_flight: Optional[_InFlight] = None
@@ -239,6 +249,8 @@ class LLM:
                 reason = "stop"
             elif at + 1 - len(r.prompt) >= r.max_new:
                 reason = "length"
+            elif r.stop_strings and self._holds_stop_string(r, at):
+                reason = "stop"
             else:
                 continue
             del r.tokens[at + 1:]
@@ -250,6 +262,10 @@ class LLM:
             r.done = True
             results[r.index] = self._result(r, t, r.preemptions)
 
+    def _holds_stop_string(self, r: _Live, at: int) -> bool:
+        text = self._tokenizer.decode(r.tokens[len(r.prompt):at + 1])
+        return any(s in text for s in r.stop_strings)
+
     def _result(self, r: _Live, t_end: float, preemptions: int) -> GenerationResult:
         out = r.tokens[len(r.prompt):]
         first = r.t_first if r.t_first is not None else t_end
@@ -258,6 +274,10 @@ class LLM:
         text = None
         if self._tokenizer is not None:
             text = self._tokenizer.decode(out)
+            for s in r.stop_strings:      # cut at the first occurrence of each, in the order given
+                cut = text.find(s)
+                if cut >= 0:
+                    text = text[:cut]
         return GenerationResult(r.rid, list(r.prompt), out, r.finish_reason or "length", text, metrics, preemptions)
 
 

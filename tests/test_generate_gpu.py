@@ -229,3 +229,37 @@ def test_drawn_workloads_change_no_token(gpu, seed):
         assert g.token_ids == w_.token_ids and g.finish_reason == w_.finish_reason, \
             f"seed {seed}, request {i} of {n}: {g.token_ids} ({g.finish_reason}) against {w_.token_ids} ({w_.finish_reason})"
     assert tight.engine.tables.audit() == "" and tight.engine.tables.num_requests() == 0
+
+
+def test_text_prompts_and_stop_strings(gpu, tmp_path):
+    """A folder with a tokenizer.json takes text prompts, returns text, and ends a request once its text holds a
+    stop string (the text returned ends before it; the ids keep the tokens that spelt it)."""
+    import shutil
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    from prelude_amd import LLM
+    folder, cfg, w = model_folder("a")
+    for name in ("config.json", "model.safetensors"):
+        shutil.copy(os.path.join(folder, name), tmp_path / name)
+    vocab = {f"w{i}": i for i in range(cfg["vocab_size"])}
+    tok = Tokenizer(models.WordLevel(vocab, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(str(tmp_path / "tokenizer.json"))
+    llm = LLM(str(tmp_path), dtype="float32", page_size=8, max_cache_tokens=512)
+    prompt = "w5 w17 w3 w200 w41"
+    free = llm.generate(prompt, max_tokens=12, temperature=0.0)[0]
+    assert free.prompt_token_ids == [5, 17, 3, 200, 41]
+    assert free.token_ids == pm.greedy(cfg, w, free.prompt_token_ids, len(free.token_ids))
+    assert free.text == " ".join(f"w{t}" for t in free.token_ids)
+    words = free.text.split()
+    assert len(words) >= 6
+    # the fifth word as a stop string: the request ends with the token that completes it
+    at = next(i for i, x in enumerate(words) if x == words[4])
+    for overlap in (True, False):
+        llm2 = LLM(str(tmp_path), dtype="float32", page_size=8, max_cache_tokens=512, overlap_steps=overlap)
+        cut = llm2.generate([prompt, [5, 17, 3]], max_tokens=12, temperature=0.0, stop=[words[4], "never there"])
+        assert cut[0].finish_reason == "stop" and cut[0].token_ids == free.token_ids[:at + 1]
+        assert cut[0].text == " ".join(words[:at]) + (" " if at else "")
+        assert cut[1].finish_reason in ("length", "eos", "stop")
+        assert llm2.engine.tables.audit() == "" and llm2.engine.tables.num_requests() == 0
+    with pytest.raises(ValueError, match="tokenizer.json"):
+        LLM(folder, dtype="float32", page_size=8, max_cache_tokens=512).generate([[1, 2]], stop=["x"])
