@@ -60,6 +60,7 @@ _KERNEL_API = {
     "pa_argmax": (I, [P, P, P, P, I, I]),
     "pa_sample": (I, [P, P, P, P, P, P, P, I, I]),
     "pa_sample_wide_workspace": (c_long, [I, I]),
+    "pa_logprobs": (I, [P, P, P, P, P, P, P, I, I, I, I]),
     "pa_sample_wide": (I, [P, P, P, P, P, P, P, P, I, I, I]),
 }
 

@@ -55,6 +55,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--top-k", type=int, default=None)
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--stop-token-ids", default="", help="comma-separated token ids that end a request")
+    ap.add_argument("--logprobs", type=int, default=None, help="with every token its log-probability and the K likeliest")
+    ap.add_argument("--prompt-logprobs", action="store_true", help="the log-probability of every prompt token too")
     ap.add_argument("--stop", action="append", default=[], help="a string that ends a request (needs tokenizer.json); "
                                                                  "repeatable")
     return ap
@@ -104,12 +106,16 @@ def main(argv=None) -> int:
         return 2
     stop = [int(x) for x in args.stop_token_ids.split(",") if x.strip()]
     outs = llm.generate(prompts, max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
-                        top_k=args.top_k, seed=args.seed, stop_token_ids=stop, stop=args.stop)
+                        top_k=args.top_k, seed=args.seed, stop_token_ids=stop, stop=args.stop, logprobs=args.logprobs,
+                        prompt_logprobs=args.prompt_logprobs)
     for o in outs:
         rec = {"request_id": o.request_id, "token_ids": o.token_ids, "finish_reason": o.finish_reason,
                "usage": o.usage, "metrics": {k: round(v, 3) for k, v in o.metrics.items()}}
         if o.text is not None:
             rec["text"] = o.text
+        for key in ("token_logprobs", "top_logprobs", "prompt_logprobs"):
+            if getattr(o, key) is not None:
+                rec[key] = getattr(o, key)
         dec = max(o.metrics.get("decode_ms", 0.0), 1e-9)
         rec["decode_tok_per_s"] = round(max(len(o.token_ids) - 1, 0) / dec * 1e3, 1)
         print(json.dumps(rec), flush=True)

@@ -94,6 +94,11 @@ int pa_sample(void* stream, const float* logits, const float* temperature, const
 // The same choice for long rows with every pass spread over the chip; modes: bit 0 some row may have a top-k,
 // bit 1 some row may have a top-p.  workspace: pa_sample_wide_workspace(rows, vocab) bytes, 16-byte aligned.
 long pa_sample_wide_workspace(int rows, int vocab);
+// lp[r] = logits[r, ids[r]] - logsumexp(logits[r]) (0 where ids[r] < 0); for k > 0 also the entries among the row's
+// k largest with their log-probabilities, ties at the k-th value included, unsorted, at most cap a row:
+// top_v / top_i [rows, cap], count [rows].
+int pa_logprobs(void* stream, const float* logits, const int* ids, float* lp, float* top_v, int* top_i, int* count,
+                int rows, int vocab, int k, int cap);
 int pa_sample_wide(void* stream, const float* logits, const float* temperature, const int* top_k, const float* top_p,
                    const float* uniform, int* out, void* workspace, int rows, int vocab, int modes);
 

@@ -322,6 +322,53 @@ __device__ void draw_from(const float* row, int begin, int end, float before, fl
   if (lane == 0) *out = fallback;
 }
 
+// Log-probabilities: lp[r] = logits[r, ids[r]] - logsumexp(logits[r]) (nothing the size of the row is written:
+// crates/prelude-cuda/src/kernels/kernels_src/logprobs/gather_log_softmax.cu), and, for k > 0, the entries among
+// the k largest of the row with their log-probabilities, ties at the k-th value included, unsorted, at most `cap`
+// of them (crates/prelude-core/src/engine/model_runner/postprocess.rs:88-155 sorts a copy of the row on the host).
+// ids[r] < 0: no target, lp[r] = 0.  One workgroup a row.
+__global__ __launch_bounds__(kSampleThreads) void logprob_kernel(const float* __restrict__ logits, int vocab,
+                                                                 const int* __restrict__ ids, int k, int cap,
+                                                                 float* __restrict__ lp, float* __restrict__ top_v,
+                                                                 int* __restrict__ top_i, int* __restrict__ count) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  SampleLds& lds = *reinterpret_cast<SampleLds*>(lds_raw);
+  const int r = blockIdx.x;
+  const float* row = logits + (size_t)r * vocab;
+  const int tid = threadIdx.x;
+  float mx = -INFINITY;
+  walk(row, 0, vocab, tid, kSampleThreads, [&](float v, int) { mx = fmaxf(mx, v); });
+  mx = wave_max(mx);
+  if (tid % kWave == 0) lds.wave_v[tid / kWave] = mx;
+  __syncthreads();
+  mx = lds.wave_v[0];
+  for (int w = 1; w < kSampleWaves; ++w) mx = fmaxf(mx, lds.wave_v[w]);
+  __syncthreads();
+  float z = 0.f;
+  walk(row, 0, vocab, tid, kSampleThreads, [&](float x, int) { z += expf(x - mx); });
+  z = block_sum(z, lds.scratch);
+  const float lse = mx + logf(z);
+  if (tid == 0) {
+    const int id = ids[r];
+    lp[r] = id >= 0 && id < vocab ? row[id] - lse : 0.f;
+  }
+  if (k <= 0) return;
+  const unsigned floor_key = k < vocab ? threshold_search<false>(row, vocab, 0u, (float)k, mx, 1.0f, lds) : 0u;
+  if (tid == 0) lds.pick_range = 0;
+  __syncthreads();
+  walk(row, 0, vocab, tid, kSampleThreads, [&](float x, int i) {
+    if (order_key(x) >= floor_key) {
+      const int at = atomicAdd(&lds.pick_range, 1);
+      if (at < cap) {
+        top_v[(size_t)r * cap + at] = x - lse;
+        top_i[(size_t)r * cap + at] = i;
+      }
+    }
+  });
+  __syncthreads();
+  if (tid == 0) count[r] = lds.pick_range < cap ? lds.pick_range : cap;
+}
+
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits, int vocab,
                                                                 const float* __restrict__ temperature,
                                                                 const int* __restrict__ top_k,
@@ -782,6 +829,23 @@ extern "C" int pa_sample_wide(void* stream, const float* logits, const float* te
   launch(kWideDraw, 0, 0);
   launch(kWideFinal, 0, 0);
   return check_launch("sample_wide");
+}
+
+// lp[r] = log-probability of ids[r] in softmax(logits[r]); for k > 0 also the entries among the row's k largest
+// (ties included, unsorted, at most cap): top_v / top_i [rows, cap] and count[rows].
+extern "C" int pa_logprobs(void* stream, const float* logits, const int* ids, float* lp, float* top_v, int* top_i,
+                           int* count, int rows, int vocab, int k, int cap) {
+  if (rows == 0) return 0;
+  PA_REQUIRE(rows > 0 && vocab > 0 && k >= 0, "logprobs: bad sizes rows=%d vocab=%d k=%d", rows, vocab, k);
+  PA_REQUIRE(k == 0 || (top_v && top_i && count && cap >= k), "logprobs: no room for the %d largest (cap %d)", k, cap);
+  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&logprob_kernel),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                        (int)sizeof(SampleLds));
+  if (allowed != hipSuccess)
+    return pa::fail("logprobs: %zu bytes of LDS refused: %s", sizeof(SampleLds), hipGetErrorString(allowed));
+  hipLaunchKernelGGL(logprob_kernel, dim3(rows), dim3(kSampleThreads), sizeof(SampleLds), (hipStream_t)stream, logits,
+                     vocab, ids, k, cap, lp, top_v, top_i, count);
+  return check_launch("logprobs");
 }
 
 extern "C" int pa_argmax_scratch(int rows, int vocab) {

@@ -26,6 +26,7 @@ import torch
 from .config.engine_config import EngineConfig
 from .engine.engine import Engine, StepEntry
 from .engine.scheduler import Scheduler
+from .ops import kernels as K
 from .sampling.sampler import RequestSampler, SamplingParams, sample_rows_device
 
 DEFAULT_MAX_TOKENS = 4096   # crates/prelude-server/src/routes/generation_common.rs:9
@@ -42,6 +43,10 @@ class GenerationResult:
     text: Optional[str] = None              # when a tokenizer is at hand
     metrics: Dict[str, float] = dataclasses.field(default_factory=dict)
     preemptions: int = 0
+    # asked for with ``logprobs`` / ``prompt_logprobs`` (crates/prelude-core/src/types.rs:388-455):
+    token_logprobs: Optional[List[float]] = None                  # log P of each generated token
+    top_logprobs: Optional[List[List[tuple]]] = None              # per generated token the k likeliest (id, log P)
+    prompt_logprobs: Optional[List[Optional[float]]] = None       # log P of each prompt token given those before it
 
     @property
     def usage(self) -> Dict[str, int]:
@@ -60,6 +65,10 @@ class _Live:
     stop_ids: frozenset
     t_arrive: float
     stop_strings: tuple = ()
+    logprobs: Optional[int] = None       # None: not asked for; k >= 0: the token's own and the k likeliest
+    token_lps: List[float] = dataclasses.field(default_factory=list)
+    top_lps: List[List[tuple]] = dataclasses.field(default_factory=list)
+    prompt_lps: Optional[List[Optional[float]]] = None
     t_first: Optional[float] = None
     finish_reason: Optional[str] = None
     pending_row: Optional[int] = None    # the last of ``tokens`` is still on the device: its row among the step's samples
@@ -74,6 +83,12 @@ class _InFlight:
     sampled: torch.Tensor        # int32 [len(drawn)] on the device
     host: torch.Tensor           # pinned copy of it, valid once ``ready`` has passed
     ready: torch.cuda.Event
+    # log-probabilities asked for, as pinned copies: of the drawn tokens (with the candidates for the k likeliest),
+    # and of prompt tokens, ``prompt_at`` saying whose and where
+    lp: Optional[torch.Tensor] = None
+    top: Optional[tuple] = None
+    prompt_lp: Optional[torch.Tensor] = None
+    prompt_at: Optional[List[tuple]] = None
 
 
 class LLM:
@@ -133,7 +148,8 @@ class LLM:
                  temperature: float = 0.7, top_p: float = 1.0, top_k: Optional[int] = None,
                  seed: Optional[int] = None, stop_token_ids: Iterable[int] = (),
                  sampling_params: Optional[Sequence[SamplingParams]] = None,
-                 stop: Iterable[str] = ()) -> List[GenerationResult]:
+                 stop: Iterable[str] = (), logprobs: Optional[int] = None,
+                 prompt_logprobs: bool = False) -> List[GenerationResult]:
         """Runs all prompts to their end with continuous batching; results in the order of the prompts.
 
         ``sampling_params`` gives each prompt options of its own and overrides
@@ -145,6 +161,12 @@ class LLM:
         token ids keep the tokens that spelt it:
         crates/prelude-core/src/engine/run/ar.rs:1560-1577,
         crates/prelude-core/src/engine/model_runner/postprocess.rs:5-16).
+
+        ``logprobs`` = k >= 0 returns with every generated token its log-probability
+        under softmax of the raw logits and the k likeliest tokens with theirs
+        (postprocess.rs:88-155); ``prompt_logprobs`` the log-probability of every
+        prompt token but the first given those before it (the head then runs over
+        all prompt positions, not only the last).
         """
         single = isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int))
         plist = [prompts] if single else list(prompts)
@@ -154,6 +176,8 @@ class LLM:
         stop_strings = tuple(s for s in ([stop] if isinstance(stop, str) else stop) if s)
         if stop_strings:
             self.tokenizer()
+        if logprobs is not None and not 0 <= int(logprobs) <= 64:
+            raise ValueError(f"logprobs {logprobs} must be within 0..64")
         live: Dict[int, _Live] = {}
         results: List[Optional[GenerationResult]] = [None] * len(plist)
         now = time.perf_counter()
@@ -173,7 +197,9 @@ class LLM:
             rid = self._next_id
             self._next_id += 1
             self.scheduler.add_request(rid, len(ids), max_new)
-            live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop_ids, now, stop_strings)
+            live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop_ids, now, stop_strings,
+                              None if logprobs is None else int(logprobs),
+                              prompt_lps=[None] * len(ids) if prompt_logprobs else None)
 
         overlap = bool(self.config.overlap_steps)
         in_flight: Optional[_InFlight] = None
@@ -194,6 +220,11 @@ class LLM:
         if not portions:
             return None
         entries = []
+        draw_rows: List[int] = []        # rows of the step's logits that are sampled from, in the order of `drawn`
+        prompt_rows: List[int] = []      # rows whose log-probability of the next prompt token is asked for
+        prompt_ids: List[int] = []
+        prompt_at: List[tuple] = []
+        rows = 0
         for p in portions:
             r = live[p.id]
             toks = r.tokens[p.start:p.start + p.count]
@@ -201,7 +232,20 @@ class LLM:
             if toks[-1] is None:       # sampled by the step before, not read yet
                 toks = toks[:-1] + [0]
                 carry = r.pending_row
-            entries.append(StepEntry(p.id, toks, [p.count - 1] if p.samples else [], carry))
+            want = []
+            if r.prompt_lps is not None:
+                # position j says how likely prompt token j + 1 is
+                for j in range(p.start, min(p.start + p.count, len(r.prompt) - 1)):
+                    prompt_rows.append(rows + len(want))
+                    prompt_ids.append(r.prompt[j + 1])
+                    prompt_at.append((r, j + 1))
+                    want.append(j - p.start)
+            if p.samples:
+                if not want or want[-1] != p.count - 1:
+                    want.append(p.count - 1)
+                draw_rows.append(rows + len(want) - 1)
+            rows += len(want)
+            entries.append(StepEntry(p.id, toks, want, carry))
         try:
             logits = self.engine.run(entries, [p.start for p in portions],
                                      previous.sampled if previous is not None else None)
@@ -211,9 +255,28 @@ class LLM:
         self.scheduler.step_done()
         self.steps += 1
         drawn = [live[p.id] for p in portions if p.samples]
-        sampled = sample_rows_device(logits, [r.sampler for r in drawn])
+        device = logits.device
+        drawn_logits = logits
+        if rows != len(draw_rows):      # other rows were asked for as well: take the sampled ones out
+            drawn_logits = logits.index_select(0, torch.tensor(draw_rows, dtype=torch.int64, device=device))
+        sampled = sample_rows_device(drawn_logits, [r.sampler for r in drawn])
         host = torch.empty(len(drawn), dtype=torch.int32, pin_memory=True)
         host.copy_(sampled, non_blocking=True)
+        lp = top = prompt_lp = None
+        ks = [r.logprobs for r in drawn if r.logprobs is not None]
+        if ks:
+            lp_dev, top_dev = K.logprobs(drawn_logits, sampled, max(ks))
+            lp = torch.empty(lp_dev.shape, dtype=lp_dev.dtype, pin_memory=True)
+            lp.copy_(lp_dev, non_blocking=True)
+            if top_dev is not None:
+                top = tuple(torch.empty(t.shape, dtype=t.dtype, pin_memory=True) for t in top_dev)
+                for dst, src in zip(top, top_dev):
+                    dst.copy_(src, non_blocking=True)
+        if prompt_rows:
+            sel = logits.index_select(0, torch.tensor(prompt_rows, dtype=torch.int64, device=device))
+            plp_dev, _ = K.logprobs(sel, torch.tensor(prompt_ids, dtype=torch.int32, device=device))
+            prompt_lp = torch.empty(plp_dev.shape, dtype=plp_dev.dtype, pin_memory=True)
+            prompt_lp.copy_(plp_dev, non_blocking=True)
         ready = torch.cuda.Event()
         ready.record()
         for row, r in enumerate(drawn):
@@ -226,16 +289,27 @@ class LLM:
                 self.scheduler.finish(r.rid)
                 r.finish_reason = "length"
                 del live[r.rid]
-        return _InFlight(drawn, sampled, host, ready)
+        return _InFlight(drawn, sampled, host, ready, lp, top, prompt_lp, prompt_at)
 
     def _resolve(self, step: _InFlight, live: Dict[int, _Live], results: List[Optional[GenerationResult]]) -> None:
         """Reads a step's sampled ids and ends the requests they end."""
         step.ready.synchronize()
         toks = step.host.tolist()
         t = time.perf_counter()
-        for r, tok in zip(step.drawn, toks):
+        if step.prompt_lp is not None:
+            for (r, at), v in zip(step.prompt_at, step.prompt_lp.tolist()):
+                r.prompt_lps[at] = v
+        lps = step.lp.tolist() if step.lp is not None else None
+        for row, (r, tok) in enumerate(zip(step.drawn, toks)):
             if r.done:                 # ended by an earlier token while this step was already running
                 continue
+            if r.logprobs is not None:
+                r.token_lps.append(lps[row])
+                if r.logprobs > 0:
+                    vals, idx, count = step.top
+                    n = int(count[row])
+                    cand = sorted(zip(idx[row, :n].tolist(), vals[row, :n].tolist()), key=lambda c: (-c[1], c[0]))
+                    r.top_lps.append(cand[:r.logprobs])
             at = len(r.tokens) - 1
             if at >= 1 and r.tokens[at - 1] is None:   # the step launched since then has put its own stand-in behind
                 at -= 1
@@ -278,7 +352,13 @@ class LLM:
                 cut = text.find(s)
                 if cut >= 0:
                     text = text[:cut]
-        return GenerationResult(r.rid, list(r.prompt), out, r.finish_reason or "length", text, metrics, preemptions)
+        res = GenerationResult(r.rid, list(r.prompt), out, r.finish_reason or "length", text, metrics, preemptions)
+        if r.logprobs is not None:
+            res.token_logprobs = r.token_lps[:len(out)]
+            if r.logprobs > 0:
+                res.top_logprobs = r.top_lps[:len(out)]
+        res.prompt_logprobs = r.prompt_lps
+        return res
 
 
 def generate(model: str, prompts, dtype: str = "bfloat16", **kwargs) -> List[GenerationResult]:

@@ -500,6 +500,33 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
 
 
+def logprobs(logits: torch.Tensor, ids: torch.Tensor, k: int = 0):
+    """Log-probabilities under softmax(logits[r]) of the tokens ``ids`` [R] (int32; negative = none, gives 0).
+
+    Returns ``(lp [R] float32, top)``; with ``k`` > 0, ``top`` is ``(values [R, cap], indices [R, cap], count [R])``:
+    the entries among each row's k largest with their log-probabilities, ties at the k-th value included, in no
+    particular order (the caller sorts the few there are); else ``None``.
+    """
+    _dev(logits, ids)
+    _f32(logits, "logits")
+    _i32(ids, "ids")
+    if logits.dim() != 2 or ids.shape != (logits.shape[0],):
+        raise NativeError(f"logprobs: logits {tuple(logits.shape)} / ids {tuple(ids.shape)}")
+    r, vocab = logits.shape
+    k = int(k)
+    lp = torch.empty(r, dtype=torch.float32, device=logits.device)
+    top = None
+    cap = 0
+    if k > 0:
+        cap = min(vocab, k + 32)
+        top = (torch.empty((r, cap), dtype=torch.float32, device=logits.device),
+               torch.empty((r, cap), dtype=torch.int32, device=logits.device),
+               torch.empty(r, dtype=torch.int32, device=logits.device))
+    check(kernels().pa_logprobs(_stream(), _ptr(logits), _ptr(ids), _ptr(lp), _ptr(top[0]) if top else None,
+                                _ptr(top[1]) if top else None, _ptr(top[2]) if top else None, r, vocab, k, cap))
+    return lp, top
+
+
 SAMPLE_WIDE_FROM = 32768   # rows this long are sampled with every pass spread over the chip,
 SAMPLE_WIDE_ROWS = 32      # up to this many at a time (more rows fill the chip with a workgroup each)
 

@@ -263,3 +263,38 @@ def test_text_prompts_and_stop_strings(gpu, tmp_path):
         assert llm2.engine.tables.audit() == "" and llm2.engine.tables.num_requests() == 0
     with pytest.raises(ValueError, match="tokenizer.json"):
         LLM(folder, dtype="float32", page_size=8, max_cache_tokens=512).generate([[1, 2]], stop=["x"])
+
+
+@pytest.mark.parametrize("overlap", [True, False])
+def test_logprobs_of_generated_and_prompt_tokens(gpu, overlap):
+    """log P of every generated token with the k likeliest, and of every prompt token given those before it,
+    against log_softmax of the plain implementation's logits; prompts cut into portions, a cache tight enough to
+    evict, sampled and greedy requests side by side."""
+    from prelude_amd import LLM
+    from prelude_amd.sampling.sampler import SamplingParams
+    folder, cfg, w = model_folder("b")
+    prompts = prompts_for(cfg, [37, 9, 60, 2], 8)
+    params = [SamplingParams(temperature=0.0), SamplingParams(temperature=0.9, seed=3),
+              SamplingParams(temperature=0.0), SamplingParams(temperature=0.7, top_k=5, seed=4)]
+    llm = LLM(folder, dtype="float32", page_size=16, max_cache_tokens=128, max_num_batched_tokens=24,
+              decode_reservation_cap=1, overlap_steps=overlap)
+    outs = llm.generate(prompts, max_tokens=30, sampling_params=params, logprobs=3, prompt_logprobs=True)
+    assert llm.scheduler.preemptions > 0
+    for p, o in zip(prompts, outs):
+        ref = torch.log_softmax(pm.forward(cfg, w, p + o.token_ids), dim=-1)
+        n = len(p)
+        assert len(o.token_logprobs) == len(o.token_ids) == len(o.top_logprobs)
+        for i, tok in enumerate(o.token_ids):
+            row = ref[n - 1 + i]
+            assert abs(o.token_logprobs[i] - float(row[tok])) < 1e-4
+            want = torch.topk(row, 3)
+            assert [t for t, _ in o.top_logprobs[i]] == want.indices.tolist()
+            assert all(abs(v - float(x)) < 1e-4 for (_, v), x in zip(o.top_logprobs[i], want.values))
+        assert o.prompt_logprobs[0] is None and len(o.prompt_logprobs) == n
+        for j in range(1, n):
+            assert abs(o.prompt_logprobs[j] - float(ref[j - 1, p[j]])) < 1e-4, (j, n)
+    plain = llm.generate(prompts[:2], max_tokens=5, temperature=0.0)
+    assert plain[0].token_logprobs is None and plain[0].top_logprobs is None and plain[0].prompt_logprobs is None
+    only = llm.generate(prompts[:1], max_tokens=5, temperature=0.0, logprobs=0)[0]
+    assert len(only.token_logprobs) == 5 and only.top_logprobs is None
+    assert llm.engine.tables.audit() == "" and llm.engine.tables.num_requests() == 0

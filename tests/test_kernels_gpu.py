@@ -623,6 +623,35 @@ def test_sample_wide_takes_only_the_searches_it_is_told_of(gpu, rows):
         assert int((one != many).sum()) <= max(1, rows // 20), (k, p, one.tolist(), many.tolist())
 
 
+@pytest.mark.parametrize("vocab", [509, 151936, 40001])
+def test_logprobs(gpu, vocab):
+    """logits[id] - logsumexp(logits), and the k largest entries with ties at the k-th value
+    (crates/prelude-core/src/engine/model_runner/postprocess.rs:88-155)."""
+    g = torch.Generator().manual_seed(vocab)
+    rows = 7
+    logits = 4.0 * torch.randn(rows, vocab, generator=g)
+    logits[2, 100:104] = logits[2].max() + 1.0          # four equal entries on top
+    ids = torch.randint(0, vocab, (rows,), generator=g).to(torch.int32)
+    ids[3] = -1
+    ref = torch.log_softmax(logits.double(), dim=-1)
+    lp, top = K().logprobs(logits.to(gpu), ids.to(gpu))
+    assert top is None
+    for r in range(rows):
+        want = 0.0 if ids[r] < 0 else float(ref[r, ids[r]])
+        assert abs(float(lp[r]) - want) < 2e-5 * max(1.0, abs(want))
+    for k in (1, 3, 20):
+        lp2, (vals, idx, count) = K().logprobs(logits.to(gpu), ids.to(gpu), k)
+        assert torch.equal(lp2, lp)
+        for r in range(rows):
+            n = int(count[r])
+            got = sorted(zip(idx[r, :n].tolist(), vals[r, :n].tolist()), key=lambda t: (-t[1], t[0]))
+            kth = torch.topk(ref[r], k).values[-1]
+            want_ids = sorted(torch.nonzero(ref[r] >= kth).flatten().tolist())      # ties at the k-th value included
+            assert sorted(i for i, _ in got) == want_ids, (k, r)
+            assert all(abs(v - float(ref[r, i])) < 2e-5 * max(1.0, abs(float(ref[r, i]))) for i, v in got)
+            assert [i for i, _ in got[:k]] == torch.topk(ref[r], k).indices.tolist() or r == 2
+
+
 def test_sample_statistics_and_limits(gpu):
     logits = torch.tensor([[2.0, 1.0, 0.5, -1.0, 0.0]]).repeat(4000, 1)
     g = torch.Generator().manual_seed(0)
