@@ -126,6 +126,7 @@ class LLM:
                                    cfg.decode_priority_max_remaining_tokens, self.engine.model.needs_state)
         self._next_id = 0
         self._tokenizer = None
+        self._on_token = None
         self.steps = 0
 
     # ---- tokenizer (only when prompts are text) --------------------------------
@@ -149,7 +150,7 @@ class LLM:
                  seed: Optional[int] = None, stop_token_ids: Iterable[int] = (),
                  sampling_params: Optional[Sequence[SamplingParams]] = None,
                  stop: Iterable[str] = (), logprobs: Optional[int] = None,
-                 prompt_logprobs: bool = False) -> List[GenerationResult]:
+                 prompt_logprobs: bool = False, on_token=None) -> List[GenerationResult]:
         """Runs all prompts to their end with continuous batching; results in the order of the prompts.
 
         ``sampling_params`` gives each prompt options of its own and overrides
@@ -167,6 +168,11 @@ class LLM:
         (postprocess.rs:88-155); ``prompt_logprobs`` the log-probability of every
         prompt token but the first given those before it (the head then runs over
         all prompt positions, not only the last).
+
+        ``on_token(prompt_index, token_id)`` is called for every generated token as
+        soon as the host has read it (the reference streams text deltas the same
+        way, crates/prelude-core/src/engine/run/ar.rs:1557), in the order the
+        tokens of a request are generated.
         """
         single = isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int))
         plist = [prompts] if single else list(prompts)
@@ -201,6 +207,7 @@ class LLM:
                               None if logprobs is None else int(logprobs),
                               prompt_lps=[None] * len(ids) if prompt_logprobs else None)
 
+        self._on_token = on_token
         overlap = bool(self.config.overlap_steps)
         in_flight: Optional[_InFlight] = None
         while live or in_flight is not None:
@@ -316,6 +323,8 @@ class LLM:
             r.tokens[at] = int(tok)
             if r.t_first is None:
                 r.t_first = t
+            if self._on_token is not None:
+                self._on_token(r.index, int(tok))
             # order of checks: crates/prelude-core/src/engine/run/ar.rs:1525-1578
             if tok in self.eos_token_ids:
                 reason = "eos"

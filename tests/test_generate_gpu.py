@@ -231,6 +231,17 @@ def test_drawn_workloads_change_no_token(gpu, seed):
     assert tight.engine.tables.audit() == "" and tight.engine.tables.num_requests() == 0
 
 
+def test_tokens_are_handed_over_as_they_come(gpu):
+    from prelude_amd import LLM
+    folder, cfg, _ = model_folder("a")
+    prompts = prompts_for(cfg, [12, 40, 3], 9)
+    for overlap in (True, False):
+        seen = {i: [] for i in range(3)}
+        llm = LLM(folder, dtype="float32", page_size=8, max_cache_tokens=512, overlap_steps=overlap)
+        outs = llm.generate(prompts, max_tokens=9, temperature=0.8, seed=5, on_token=lambda i, t: seen[i].append(t))
+        assert [seen[i] for i in range(3)] == [o.token_ids for o in outs]
+
+
 def test_text_prompts_and_stop_strings(gpu, tmp_path):
     """A folder with a tokenizer.json takes text prompts, returns text, and ends a request once its text holds a
     stop string (the text returned ends before it; the ids keep the tokens that spelt it)."""
