@@ -9,12 +9,15 @@ __version__ = "0.1.0"
 
 def __getattr__(name):
     # heavy imports (torch, the native libraries) wait until something is used
-    if name in ("LLM", "GenerationResult", "generate"):
+    if name in ("LLM", "Session", "GenerationResult", "generate"):
         from . import llm
         return getattr(llm, name)
     if name in ("Engine", "StepEntry"):
         from . import engine
         return getattr(engine, name)
+    if name == "SamplingParams":
+        from .sampling.sampler import SamplingParams
+        return SamplingParams
     if name == "EngineConfig":
         from .config import EngineConfig
         return EngineConfig

@@ -1,4 +1,5 @@
-"""The Python entry point: ``LLM(model_dir).generate(prompts, ...)``.
+"""The Python entry point: ``LLM(model_dir).generate(prompts, ...)``, and ``LLM.session()`` for requests that
+arrive while others run.
 
 Modelled on the reference's ``InferenceEngine::generate`` / ``generate_batch``
 (crates/prelude-core/src/engine/mod.rs:75-132) and its request and result
@@ -126,7 +127,6 @@ class LLM:
                                    cfg.decode_priority_max_remaining_tokens, self.engine.model.needs_state)
         self._next_id = 0
         self._tokenizer = None
-        self._on_token = None
         self.steps = 0
 
     # ---- tokenizer (only when prompts are text) --------------------------------
@@ -178,48 +178,112 @@ class LLM:
         plist = [prompts] if single else list(prompts)
         if sampling_params is not None and len(sampling_params) != len(plist):
             raise ValueError("sampling_params must have one entry per prompt")
+        session = self.session(on_token=on_token)
+        for i, p in enumerate(plist):
+            sp = sampling_params[i] if sampling_params is not None else SamplingParams(temperature, top_p, top_k, seed)
+            try:
+                session.add(p, max_tokens=max_tokens, sampling=sp, stop_token_ids=stop_token_ids, stop=stop,
+                            logprobs=logprobs, prompt_logprobs=prompt_logprobs)
+            except ValueError as e:
+                session.abandon()
+                raise ValueError(f"prompt {i}: {e}") from None
+        results: List[Optional[GenerationResult]] = [None] * len(plist)
+        while session.pending:
+            for index, res in session.step():
+                results[index] = res
+        return results  # type: ignore[return-value]
+
+    def session(self, on_token=None) -> "Session":
+        """A generation loop that requests can join while others run: ``add`` a request at any time, call
+        ``step`` while ``pending``; each step returns the requests that ended in it.  One session at a time."""
+        return Session(self, on_token)
+
+
+class Session:
+    """The reference's ``ar_loop`` (crates/prelude-core/src/engine/run/ar.rs:180-396) with the request queue in
+    the caller's hands: schedule, build the step, run it, sample, finish -- one step per call."""
+
+    def __init__(self, llm: "LLM", on_token=None):
+        self.llm = llm
+        self.engine = llm.engine
+        self.scheduler = llm.scheduler
+        self._on_token = on_token
+        self._live: Dict[int, _Live] = {}
+        self._in_flight: Optional[_InFlight] = None
+        self._added = 0
+        self._ended: List[tuple] = []
+
+    @property
+    def pending(self) -> bool:
+        """Whether a request is still running or a launched step has not been read."""
+        return bool(self._live) or self._in_flight is not None
+
+    def add(self, prompt: Prompt, max_tokens: int = DEFAULT_MAX_TOKENS, sampling: Optional[SamplingParams] = None,
+            stop_token_ids: Iterable[int] = (), stop: Iterable[str] = (), logprobs: Optional[int] = None,
+            prompt_logprobs: bool = False) -> int:
+        """Queues a request; returns its index in this session (``step`` names ended requests by it)."""
+        llm = self.llm
         stop_ids = frozenset(int(t) for t in stop_token_ids)
-        stop_strings = tuple(s for s in ([stop] if isinstance(stop, str) else stop) if s)
+        stop_strings = tuple(x for x in ([stop] if isinstance(stop, str) else stop) if x)
         if stop_strings:
-            self.tokenizer()
+            llm.tokenizer()
         if logprobs is not None and not 0 <= int(logprobs) <= 64:
             raise ValueError(f"logprobs {logprobs} must be within 0..64")
-        live: Dict[int, _Live] = {}
-        results: List[Optional[GenerationResult]] = [None] * len(plist)
-        now = time.perf_counter()
-        for i, p in enumerate(plist):
-            ids = self._to_ids(p)
-            if not ids:
-                raise ValueError(f"prompt {i} is empty")
-            bad = [t for t in ids if not 0 <= t < self.engine.vocab_size]
-            if bad:
-                raise ValueError(f"prompt {i}: token id {bad[0]} is outside the vocabulary")
-            # crates/prelude-core/src/engine/model_runner/generate.rs:23-26
-            max_new = min(int(max_tokens), self.max_positions - len(ids))
-            if max_new < 1:
-                raise ValueError(f"prompt {i} has {len(ids)} tokens; the model has positions for "
-                                 f"{self.max_positions} and none is left to generate")
-            sp = sampling_params[i] if sampling_params is not None else SamplingParams(temperature, top_p, top_k, seed)
-            rid = self._next_id
-            self._next_id += 1
-            self.scheduler.add_request(rid, len(ids), max_new)
-            live[rid] = _Live(rid, i, ids, list(ids), max_new, RequestSampler(sp), stop_ids, now, stop_strings,
-                              None if logprobs is None else int(logprobs),
-                              prompt_lps=[None] * len(ids) if prompt_logprobs else None)
+        ids = llm._to_ids(prompt)
+        if not ids:
+            raise ValueError("the prompt is empty")
+        bad = [t for t in ids if not 0 <= t < self.engine.vocab_size]
+        if bad:
+            raise ValueError(f"token id {bad[0]} is outside the vocabulary")
+        # crates/prelude-core/src/engine/model_runner/generate.rs:23-26
+        max_new = min(int(max_tokens), llm.max_positions - len(ids))
+        if max_new < 1:
+            raise ValueError(f"the prompt has {len(ids)} tokens; the model has positions for "
+                             f"{llm.max_positions} and none is left to generate")
+        sp = sampling if sampling is not None else SamplingParams()
+        rid = llm._next_id
+        llm._next_id += 1
+        self.scheduler.add_request(rid, len(ids), max_new)
+        index = self._added
+        self._added += 1
+        self._live[rid] = _Live(rid, index, ids, list(ids), max_new, RequestSampler(sp), stop_ids, time.perf_counter(),
+                                stop_strings, None if logprobs is None else int(logprobs),
+                                prompt_lps=[None] * len(ids) if prompt_logprobs else None)
+        return index
 
-        self._on_token = on_token
-        overlap = bool(self.config.overlap_steps)
-        in_flight: Optional[_InFlight] = None
-        while live or in_flight is not None:
-            launched = self._launch(live, in_flight) if live else None
-            if launched is None and in_flight is None:
+    def abandon(self) -> None:
+        """Ends every request of the session without a result and gives back what they hold."""
+        if self._in_flight is not None:
+            self._in_flight.ready.synchronize()
+            self._in_flight = None
+        for rid in list(self._live):
+            self.scheduler.finish(rid)
+        self._live.clear()
+
+    def step(self) -> List[tuple]:
+        """Launches the next step (if there is anything to run) and reads the one before; returns
+        ``[(index, GenerationResult)]`` for the requests that ended."""
+        overlap = bool(self.llm.config.overlap_steps)
+        launched = self._launch(self._live, self._in_flight) if self._live else None
+        if launched is None and self._in_flight is None:
+            if self._live:
                 raise RuntimeError("the scheduler has requests but nothing to run")
-            if not overlap and launched is not None:
-                in_flight, launched = launched, None
-            if in_flight is not None:
-                self._resolve(in_flight, live, results)
-            in_flight = launched
-        return results  # type: ignore[return-value]
+            return []
+        if not overlap and launched is not None:
+            self._in_flight, launched = launched, None
+        if self._in_flight is not None:
+            self._resolve(self._in_flight, self._live)
+        self._in_flight = launched
+        ended, self._ended = self._ended, []
+        return ended
+
+    @property
+    def eos_token_ids(self):
+        return self.llm.eos_token_ids
+
+    @property
+    def _tokenizer(self):
+        return self.llm._tokenizer
 
     def _launch(self, live: Dict[int, _Live], previous: Optional[_InFlight]) -> Optional[_InFlight]:
         """Schedules and launches one step; the scheduler is told at once that its tokens exist."""
@@ -260,7 +324,7 @@ class LLM:
             self.scheduler.step_cancelled()
             raise
         self.scheduler.step_done()
-        self.steps += 1
+        self.llm.steps += 1
         drawn = [live[p.id] for p in portions if p.samples]
         device = logits.device
         drawn_logits = logits
@@ -298,7 +362,7 @@ class LLM:
                 del live[r.rid]
         return _InFlight(drawn, sampled, host, ready, lp, top, prompt_lp, prompt_at)
 
-    def _resolve(self, step: _InFlight, live: Dict[int, _Live], results: List[Optional[GenerationResult]]) -> None:
+    def _resolve(self, step: _InFlight, live: Dict[int, _Live]) -> None:
         """Reads a step's sampled ids and ends the requests they end."""
         step.ready.synchronize()
         toks = step.host.tolist()
@@ -343,7 +407,7 @@ class LLM:
                 del live[r.rid]
             r.finish_reason = reason
             r.done = True
-            results[r.index] = self._result(r, t, r.preemptions)
+            self._ended.append((r.index, self._result(r, t, r.preemptions)))
 
     def _holds_stop_string(self, r: _Live, at: int) -> bool:
         text = self._tokenizer.decode(r.tokens[len(r.prompt):at + 1])

@@ -242,6 +242,40 @@ def test_tokens_are_handed_over_as_they_come(gpu):
         assert [seen[i] for i in range(3)] == [o.token_ids for o in outs]
 
 
+def test_requests_join_a_running_session(gpu):
+    """Requests added while others are decoding get the tokens they get alone, and a session that is given up
+    leaves nothing behind in the scheduler or the cache."""
+    from prelude_amd import LLM
+    from prelude_amd.sampling.sampler import SamplingParams
+    folder, cfg, w = model_folder("c")
+    prompts = prompts_for(cfg, [30, 8, 55, 17, 3], 12)
+    llm = LLM(folder, dtype="float32", page_size=8, max_cache_tokens=1024, max_num_batched_tokens=32)
+    alone = [llm.generate([p], max_tokens=20, temperature=0.0)[0].token_ids for p in prompts]
+    s = llm.session()
+    got, ends, steps = {}, [], 0
+    arrivals = {0: [0], 3: [1, 2], 11: [3], 25: [4]}        # step -> prompts that arrive before it
+    while s.pending or steps <= max(arrivals):
+        for i in arrivals.get(steps, []):
+            assert s.add(prompts[i], max_tokens=20, sampling=SamplingParams(temperature=0.0)) == i
+        for index, res in s.step():
+            got[index] = res.token_ids
+            ends.append(index)
+        steps += 1
+    assert [got[i] for i in range(5)] == alone
+    assert ends.index(1) < ends.index(4)                      # the late arrival ends after an early one
+    assert llm.engine.tables.audit() == "" and llm.engine.tables.num_requests() == 0
+    s = llm.session()
+    s.add(prompts[2], max_tokens=50, sampling=SamplingParams(temperature=0.0))
+    for _ in range(4):
+        s.step()
+    s.abandon()
+    assert not s.pending and llm.engine.tables.num_requests() == 0 and llm.engine.tables.audit() == ""
+    assert llm.generate([prompts[1]], max_tokens=20, temperature=0.0)[0].token_ids == alone[1]
+    with pytest.raises(ValueError, match="prompt 1: the prompt is empty"):
+        llm.generate([[1, 2], []], max_tokens=4)
+    assert llm.engine.tables.num_requests() == 0
+
+
 def test_text_prompts_and_stop_strings(gpu, tmp_path):
     """A folder with a tokenizer.json takes text prompts, returns text, and ends a request once its text holds a
     stop string (the text returned ends before it; the ids keep the tokens that spelt it)."""
