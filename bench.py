@@ -212,23 +212,31 @@ def time_mixed(raw, dtype, chunk, decoding, context, steps, warmup):
 
 
 def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency):
-    """`requests` prompts of `prompt_len` random tokens, `max_tokens` new tokens each, through LLM.generate with
-    at most `concurrency` of them handed over at a time (the reference's published workload is this with one
-    new token, over HTTP).  Returns (seconds in all, list of seconds per call)."""
+    """`requests` prompts of `prompt_len` random tokens, `max_tokens` new tokens each, through an LLM session
+    that is kept at `concurrency` requests: whenever one ends the next is added, as a load generator with that
+    many clients does (the reference's published workload is this with one new token, over HTTP).
+    Returns (seconds in all, sorted list of seconds from a request's arrival to its end)."""
     import numpy as np
-    from prelude_amd import LLM
+    from prelude_amd import LLM, SamplingParams
     eng = build_engine(raw, dtype, cache_tokens=min(requests, max(concurrency, 16)) * (prompt_len + max_tokens + 64))
     llm = LLM.from_engine(eng)
     rng = np.random.default_rng(5)
     prompts = [rng.integers(0, raw["vocab_size"] - 1000, size=prompt_len).tolist() for _ in range(requests)]
     llm.generate(prompts[:min(concurrency, 8)], max_tokens=max_tokens, temperature=0.0)   # warm-up
-    calls = []
+    greedy = SamplingParams(temperature=0.0)
+    session = llm.session()
+    sent, latencies = 0, []
     t0 = time.perf_counter()
-    for s0 in range(0, requests, concurrency):
-        t1 = time.perf_counter()
-        llm.generate(prompts[s0:s0 + concurrency], max_tokens=max_tokens, temperature=0.0)
-        calls.append(time.perf_counter() - t1)
-    return time.perf_counter() - t0, calls
+    while sent < min(concurrency, requests):
+        session.add(prompts[sent], max_tokens=max_tokens, sampling=greedy)
+        sent += 1
+    while session.pending:
+        for _, res in session.step():
+            latencies.append(res.metrics["total_ms"] / 1e3)
+            if sent < requests:
+                session.add(prompts[sent], max_tokens=max_tokens, sampling=greedy)
+                sent += 1
+    return time.perf_counter() - t0, sorted(latencies)
 
 
 def main() -> int:
@@ -280,11 +288,13 @@ def main() -> int:
         total, calls = time_requests(raw, args.dtype, args.requests, args.prompt_len, args.new_tokens, args.concurrency)
         calls.sort()
         print(json.dumps({"model": name, "workload": f"{args.requests} prompts of {args.prompt_len} tokens, "
-                          f"{args.new_tokens} new token(s), {args.concurrency} at a time (LLM.generate, no HTTP)",
+                          f"{args.new_tokens} new token(s), {args.concurrency} at a time (LLM session, no HTTP)",
                           "req_per_s": round(args.requests / total, 1),
                           "prompt_tok_per_s": round(args.requests * args.prompt_len / total, 1),
                           "new_tok_per_s": round(args.requests * args.new_tokens / total, 1),
-                          "call_ms_p50": round(calls[len(calls) // 2] * 1e3, 2)}), flush=True)
+                          "latency_ms_p50": round(calls[len(calls) // 2] * 1e3, 2),
+                          "latency_ms_p95": round(calls[min(len(calls) - 1, int(len(calls) * 0.95))] * 1e3, 2)}),
+              flush=True)
         return 0
     if args.prefill_only:
         psec = time_prefill(raw, args.dtype, args.prefill_tokens, reps=3)
