@@ -40,7 +40,9 @@ QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_si
 QWEN3_8B = dict(QWEN3_4B, hidden_size=4096, intermediate_size=12288, tie_word_embeddings=False)
 QWEN3_32B = dict(QWEN3_4B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
                  max_window_layers=64, tie_word_embeddings=False)
-SHAPES = {"4b": QWEN3_4B, "8b": QWEN3_8B, "32b": QWEN3_32B}
+QWEN3_06B = dict(QWEN3_4B, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                 max_window_layers=28)
+SHAPES = {"0.6b": QWEN3_06B, "4b": QWEN3_4B, "8b": QWEN3_8B, "32b": QWEN3_32B}
 
 
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
@@ -225,7 +227,7 @@ def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency):
     llm.generate(prompts[:min(concurrency, 8)], max_tokens=max_tokens, temperature=0.0)   # warm-up
     greedy = SamplingParams(temperature=0.0)
     session = llm.session()
-    sent, latencies = 0, []
+    sent, latencies, firsts = 0, [], []
     t0 = time.perf_counter()
     while sent < min(concurrency, requests):
         session.add(prompts[sent], max_tokens=max_tokens, sampling=greedy)
@@ -233,10 +235,11 @@ def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency):
     while session.pending:
         for _, res in session.step():
             latencies.append(res.metrics["total_ms"] / 1e3)
+            firsts.append(res.metrics["ttft_ms"] / 1e3)
             if sent < requests:
                 session.add(prompts[sent], max_tokens=max_tokens, sampling=greedy)
                 sent += 1
-    return time.perf_counter() - t0, sorted(latencies)
+    return time.perf_counter() - t0, sorted(latencies), sorted(firsts)
 
 
 def main() -> int:
@@ -248,7 +251,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 8B or 32B")
+    ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 0.6B, 8B or 32B")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
@@ -285,13 +288,17 @@ def main() -> int:
               flush=True)
         return 0
     if args.requests:
-        total, calls = time_requests(raw, args.dtype, args.requests, args.prompt_len, args.new_tokens, args.concurrency)
-        calls.sort()
+        total, calls, firsts = time_requests(raw, args.dtype, args.requests, args.prompt_len, args.new_tokens,
+                                             args.concurrency)
+        mean = lambda v: sum(v) / len(v)
+        tpot = (mean(calls) - mean(firsts)) / max(args.new_tokens - 1, 1)
         print(json.dumps({"model": name, "workload": f"{args.requests} prompts of {args.prompt_len} tokens, "
                           f"{args.new_tokens} new token(s), {args.concurrency} at a time (LLM session, no HTTP)",
                           "req_per_s": round(args.requests / total, 1),
                           "prompt_tok_per_s": round(args.requests * args.prompt_len / total, 1),
                           "new_tok_per_s": round(args.requests * args.new_tokens / total, 1),
+                          "ttft_ms_mean": round(mean(firsts) * 1e3, 2), "tpot_ms_mean": round(tpot * 1e3, 3),
+                          "latency_ms_mean": round(mean(calls) * 1e3, 2),
                           "latency_ms_p50": round(calls[len(calls) // 2] * 1e3, 2),
                           "latency_ms_p95": round(calls[min(len(calls) - 1, int(len(calls) * 0.95))] * 1e3, 2)}),
               flush=True)
