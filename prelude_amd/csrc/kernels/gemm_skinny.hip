@@ -227,31 +227,52 @@ static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* 
   *depth = kDepth;
 }
 
+// The kernels that are built: the (tiles per workgroup, wavefronts) that skinny_shape can ask for with this many
+// row tiles and this layout.  Sixteen wavefronts leave 128 registers each, enough for 16 rows of one tile: a tiled
+// weight never takes them with more rows, a row-major one does (its split of K must not depend on the rows, and
+// beyond 16 rows it is not the layout that serving uses) and spills.
+template <int MT, bool TILED, int NT, int WV>
+constexpr bool skinny_built() {
+  if (TILED) return WV == 8 ? (NT <= 2 || MT == 1) : (WV == 16 && MT == 1 && NT == 1);
+  if (MT > 1) return NT == 1;
+  return NT == 1 || (NT == 2 && WV <= 8) || (NT == 4 && WV == 4);
+}
+
+template <int MT, int NT, int WV, typename TC, int EPI, bool TILED, int DEPTH>
+int launch_skinny_as(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
+                     long ldx, long ldc) {
+  if constexpr (skinny_built<MT, TILED, NT, WV>()) {
+    dim3 grid(((n + 15) / 16 + NT - 1) / NT);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED, DEPTH>), grid, dim3(WV * kWave), 0, st,
+                       (const bf16*)x, (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc);
+    return check_launch("gemm_skinny");
+  } else {
+    return pa::fail("gemm_skinny: no kernel for %d row tiles with %d tiles a workgroup on %d wavefronts (%s weight)", MT,
+                    NT, WV, TILED ? "tiled" : "row-major");
+  }
+}
+
 template <int MT, typename TC, int EPI, bool TILED, int DEPTH>
 int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                  long ldx, long ldc) {
+                        long ldx, long ldc) {
   int nt, waves, depth;
   skinny_shape(m, n, k, MT, TILED, &nt, &waves, &depth);
-  dim3 grid(((n + 15) / 16 + nt - 1) / nt);
-#define PA_W(NT, WV)                                                                                            \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED, DEPTH>), grid, dim3(WV* kWave), 0, st, (const bf16*)x, \
-                     (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc)
-#define PA_WAVES(NT)            \
-  switch (waves) {              \
-    case 16: PA_W(NT, 16); break; \
-    case 8: PA_W(NT, 8); break;   \
-    default: PA_W(NT, 4); break;  \
-  }
-  if (MT == 1 && nt == 4) {
-    PA_WAVES((MT == 1 ? 4 : 1))
-  } else if ((MT == 1 || (TILED && waves <= 8)) && nt == 2) {
-    PA_WAVES(((MT == 1 || TILED) ? 2 : 1))
-  } else {
-    PA_WAVES(1)
+#define PA_AS(NT, WV) return launch_skinny_as<MT, NT, WV, TC, EPI, TILED, DEPTH>(st, x, w, bias, c, m, n, k, ldx, ldc)
+#define PA_WAVES(NT)     \
+  switch (waves) {       \
+    case 16: PA_AS(NT, 16); \
+    case 8: PA_AS(NT, 8);   \
+    case 4: PA_AS(NT, 4);   \
+  }                      \
+  break;
+  switch (nt) {
+    case 4: PA_WAVES(4)
+    case 2: PA_WAVES(2)
+    case 1: PA_WAVES(1)
   }
 #undef PA_WAVES
-#undef PA_W
-  return check_launch("gemm_skinny");
+#undef PA_AS
+  return pa::fail("gemm_skinny: no kernel with %d tiles a workgroup on %d wavefronts", nt, waves);
 }
 
 template <int MT, typename TC, int EPI, bool TILED>
