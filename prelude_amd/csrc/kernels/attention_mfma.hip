@@ -954,10 +954,13 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
     staged = want.staged != 0;
   }
   PA_REQUIRE(staged || hw == 1, "attn_prefill: two head groups a workgroup only with staged keys");
+  PA_REQUIRE(gt <= gt_best, "attn_prefill: %d heads a wavefront, head_dim %d takes up to %d", gt, HD, gt_best);
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
                                    max_q_len, nh, nkv, page_shift, window, scale, paired, hw, staged)
-  if (gt == 4) PA_GT(4);
+  if constexpr (HD <= 64) {   // four heads' state of a wider head does not fit 256 registers: not built, never chosen
+    if (gt == 4) PA_GT(4);
+  }
   if (gt == 2) PA_GT(2);
   PA_GT(1);
 #undef PA_GT
