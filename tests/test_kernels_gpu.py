@@ -1,6 +1,8 @@
 """Each kernel alone against its plain reference, at other sizes than the tiny models use."""
 import math
+import os
 
+import numpy as np
 import pytest
 import torch
 
@@ -474,6 +476,44 @@ def test_prefill_attention_refuses_a_cut_the_shape_does_not_take(gpu):
         paged_case(gpu, torch.bfloat16, 3, 3, 64, 16, [(70, 70)], 0, kernel="mfma", cut=(-1, 1, 2, -1))
     with pytest.raises(NativeError, match="not staged"):
         paged_case(gpu, torch.bfloat16, 4, 2, 64, 4, [(70, 70)], 0, kernel="mfma", cut=(-1, -1, -1, 1))
+
+
+def draw_attention_case(seed: int):
+    rng = np.random.default_rng(seed)
+    hd = int(rng.choice([16, 32, 48, 64, 96, 128]))
+    nkv = int(rng.choice([1, 2, 3, 8]))
+    group = int(rng.choice([1, 2, 3, 4, 6, 8]))
+    page = int(rng.choice([4, 8, 16, 32, 64, 128]))
+    window = int(rng.choice([0, 0, 0, 1, 31, 64, 100, 257, int(rng.integers(2, 500))]))
+    seqs = []
+    for _ in range(int(rng.integers(1, 7))):
+        kind = int(rng.integers(0, 4))
+        if kind == 0:                                   # a decoding request
+            seqs.append((int(rng.integers(1, 1300)), 1))
+        elif kind == 1:                                 # a whole prompt
+            n = int(rng.integers(2, 800))
+            seqs.append((n, n))
+        else:                                           # a portion inside a context, long or down to two tokens
+            ctx = int(rng.integers(2, 1500))
+            seqs.append((ctx, int(rng.integers(2, min(ctx, 600 if kind == 2 else 9) + 1))))
+    return nkv * group, nkv, hd, page, window, seqs
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_ATTENTION", "10")))))   # widen for a hunt
+def test_drawn_attention(gpu, seed):
+    """Head counts, head size, page size, window and the step's requests drawn at random: decoding requests, whole
+    prompts and portions inside a context in one step.  Pages a window has passed hold NaN, so a key read from one
+    of them shows."""
+    nh, nkv, hd, page, window, seqs = draw_attention_case(seed)
+    what = f"seed {seed}: {nh} heads over {nkv}, head_dim {hd}, page {page}, window {window}, (context, new) {seqs}"
+    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=seed, kernel="mfma")
+    assert not bool(torch.isnan(out).any()), what
+    err = float((out.double().cpu() - ref).abs().max())
+    assert err <= tol(torch.bfloat16, ref), f"{what}: max error {err:.3e}"
+    out, ref = paged_case(gpu, torch.float32, nh, nkv, hd, page, seqs, window, seed=seed)
+    assert not bool(torch.isnan(out).any()), what
+    err = float((out.double().cpu() - ref).abs().max())
+    assert err <= tol(torch.float32, ref, f32=3e-6), f"{what}: 32-bit kernel, max error {err:.3e}"
 
 
 def test_mfma_attention_batch_and_page_independence(gpu):
