@@ -163,6 +163,45 @@ def test_gemm_skinny(gpu, m, n, k):
         close(K().linear(xd, K().LinearWeight(wd, tiles)), ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_PRODUCTS", "12")))))   # widen for a hunt
+def test_drawn_products(gpu, seed):
+    """Rows, outputs and inner size drawn at random, through the dispatcher and through the weight-streaming kernel
+    with the weight in rows and in tiles, with bias, 32-bit output and the SiLU*up epilogue."""
+    rng = np.random.default_rng(seed)
+    m = int(rng.choice([1, 2, 7, 8, 9, 16, 17, 31, 33, 48, 64, int(rng.integers(1, 65))]))
+    n = 2 * int(rng.choice([1, 8, 20, 160, 331, int(rng.integers(1, 1500)), int(rng.integers(1500, 12000))]))
+    k = 8 * int(rng.choice([1, 7, 8, 9, 40, 129, int(rng.integers(1, 160)), int(rng.integers(160, 1300))]))
+    if n * k > 40e6:
+        k = max(8, int(40e6 // n) // 8 * 8)
+    what = f"seed {seed}: m {m} n {n} k {k}"
+    x, w, b = rnd(m, k, dtype=torch.bfloat16, seed=seed), rnd(n, k, dtype=torch.bfloat16, seed=seed + 1, scale=0.05), rnd(n, seed=2)
+    ref = x.double() @ w.double().T
+    act = pm.silu(ref[:, 0::2]) * ref[:, 1::2]
+    xd, wd, bd = x.to(gpu), w.to(gpu), b.to(gpu)
+    tiles = K().pack_tiles(wd)
+    lw = K().LinearWeight(wd, tiles)
+    for name, got, want, dt in (
+            ("rows", K().gemm_skinny(xd, wd, out_dtype=torch.float32), ref, torch.float32),
+            ("rows, bias", K().gemm_skinny(xd, wd, bd), ref + b.double(), torch.bfloat16),
+            ("rows, SiLU*up", K().gemm_skinny(xd, wd, silu_mul_epilogue=True), act, torch.bfloat16),
+            ("tiles", K().gemm_skinny(xd, tiles, out_dtype=torch.float32), ref, torch.float32),
+            ("tiles, bias", K().gemm_skinny(xd, tiles, bd), ref + b.double(), torch.bfloat16),
+            ("tiles, SiLU*up", K().gemm_skinny(xd, tiles, silu_mul_epilogue=True), act, torch.bfloat16),
+            ("linear", K().linear(xd, lw, bd), ref + b.double(), torch.bfloat16),
+            # beyond the streaming kernel's rows the library's bfloat16 result is widened: bfloat16's rounding
+            ("linear, 32-bit out", K().linear(xd, lw, out_dtype=torch.float32), ref, torch.float32 if m <= 16 else torch.bfloat16),
+            ("linear, SiLU*up", K().linear_silu_mul(xd, lw), act, torch.bfloat16)):
+        assert tuple(got.shape) == tuple(want.shape), f"{what}, {name}: shape {tuple(got.shape)}"
+        err = float((got.double().cpu() - want).abs().max())
+        assert err <= tol(dt, want, f32=2e-5), f"{what}, {name}: max error {err:.3e} > {tol(dt, want, f32=2e-5):.3e}"
+    # many rows through the dispatcher (the library product beyond the streaming kernel's rows)
+    m2 = int(rng.integers(65, 400))
+    x2 = rnd(m2, k, dtype=torch.bfloat16, seed=seed + 3)
+    ref2 = x2.double() @ w.double().T
+    close(K().linear(x2.to(gpu), lw, bd), ref2 + b.double(), torch.bfloat16)
+    close(K().linear_silu_mul(x2.to(gpu), lw), pm.silu(ref2[:, 0::2]) * ref2[:, 1::2], torch.bfloat16)
+
+
 def test_pack_tiles_layout(gpu):
     """out[tile][step][half][g][r][j] = w[16 tile + r][64 step + 16 g + 8 half + j], zeros beyond the matrix."""
     n, k = 40, 200
@@ -643,6 +682,37 @@ def test_sample_matches_the_plain_draw(gpu, vocab, wide):
             assert out[r] == pm.draw(prs, float(u[r])), f"row {r}"
             checked += 1
     assert checked >= rows // 2
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_DRAWS", "8")))))   # widen for a hunt
+def test_drawn_draws(gpu, seed):
+    """Vocabulary, rows and every row's temperature, top-k and top-p drawn at random, through the one-workgroup
+    kernel and the wide one: the token is the plain draw's wherever 32-bit sums cannot move it over a boundary,
+    and always one of the kept set."""
+    rng = np.random.default_rng(seed)
+    vocab = int(rng.choice([2, 17, 509, 4096, 40001, 151936, int(rng.integers(2, 200000))]))
+    rows = int(rng.choice([1, 2, 8, 33, int(rng.integers(1, 70))]))
+    rows = min(rows, max(1, 400000 // vocab))      # the plain top-p walks the sorted row entry by entry
+    g = torch.Generator().manual_seed(seed)
+    logits = float(rng.choice([0.5, 3.0, 8.0])) * torch.randn(rows, vocab, generator=g)
+    temps = [float(rng.choice([0.0, 0.3, 0.8, 1.0, 1.7])) for _ in range(rows)]
+    topk = [int(rng.choice([0, 0, 1, 5, 50, vocab, 2 * vocab])) for _ in range(rows)]
+    topp = [float(rng.choice([1.0, 1.0, 0.95, 0.5, 0.05])) for _ in range(rows)]
+    u = torch.rand(rows, generator=g)
+    for wide in (False, True):
+        out = K().sample(logits.to(gpu), torch.tensor(temps).to(gpu), torch.tensor(topk, dtype=torch.int32).to(gpu),
+                         torch.tensor(topp).to(gpu), u.to(gpu), wide=wide).tolist()
+        for r in range(rows):
+            what = f"seed {seed} wide {wide}: vocabulary {vocab}, row {r} of {rows}, T {temps[r]} top-k {topk[r]} top-p {topp[r]}"
+            if temps[r] < 1e-7:
+                assert out[r] == int(torch.argmax(logits[r])), what
+                continue
+            prs = pm.sampling_probs(logits[r], temps[r], topk[r] or None, topp[r] if topp[r] < 1.0 else None)
+            assert 0 <= out[r] < vocab and prs[out[r]] > 0, f"{what}: token {out[r]} is outside the kept set"
+            cdf = torch.cumsum(prs, 0)
+            target = float(u[r]) * float(cdf[-1])
+            if float((cdf - target).abs().min()) > 1e-4 * float(cdf[-1]):
+                assert out[r] == pm.draw(prs, float(u[r])), what
 
 
 @pytest.mark.parametrize("rows", [1, 3, 70])
