@@ -199,7 +199,9 @@ def test_drawn_products(gpu, seed):
     x2 = rnd(m2, k, dtype=torch.bfloat16, seed=seed + 3)
     ref2 = x2.double() @ w.double().T
     close(K().linear(x2.to(gpu), lw, bd), ref2 + b.double(), torch.bfloat16)
-    close(K().linear_silu_mul(x2.to(gpu), lw), pm.silu(ref2[:, 0::2]) * ref2[:, 1::2], torch.bfloat16)
+    # gate and up are rounded to bfloat16 by the library product, then the activation's result: three roundings of up
+    # to 2^-8 each, the gate's weighing up to 1.2 times (x silu'(x) / silu(x)) -- 1.25 % of the largest value at worst
+    close(K().linear_silu_mul(x2.to(gpu), lw), pm.silu(ref2[:, 0::2]) * ref2[:, 1::2], torch.bfloat16, bf16=1.25e-2)
 
 
 def test_pack_tiles_layout(gpu):
