@@ -46,6 +46,7 @@ _KERNEL_API = {
     "pa_to_f32": (I, [P, I, P, P, c_long]),
     "pa_qknorm_rope_kv": (I, [P, I, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F]),
     "pa_gemm_plain": (I, [P, I, I, P, P, P, P, I, I, I, c_long, c_long, c_long]),
+    "pa_gemm_library": (I, [P, P, P, P, I, I, I, c_long, c_long, P, c_long]),
     "pa_gemm_skinny": (I, [P, I, I, P, P, P, P, I, I, I, c_long, c_long, I]),
     "pa_pack_tiles": (I, [P, P, P, I, I]),
     "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),

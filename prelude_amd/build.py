@@ -168,7 +168,12 @@ def build_kernels(force: bool = False, jobs: int | None = None) -> str:
         with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
             objs = list(ex.map(one, srcs))
         tmp = lib + f".tmp{os.getpid()}"
-        _run([hipcc, f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], "link of the kernel library")
+        # hipBLASLt for the products of many rows; a process that has loaded torch holds that library already
+        rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(hipcc))), "lib")
+        if not os.path.exists(os.path.join(rocm_lib, "libhipblaslt.so")):
+            rocm_lib = "/opt/rocm/lib"
+        _run([hipcc, f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC", "-o", tmp, *objs,
+              f"-L{rocm_lib}", "-lhipblaslt", f"-Wl,-rpath,{rocm_lib}"], "link of the kernel library")
     _finish(lib, tmp, fp)
     _log(f"kernel library ready in {time.time() - t0:.0f} s")
     return lib

@@ -35,6 +35,10 @@ int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_w
                       void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int hd, int rot,
                       int page_size, float eps);
 
+// C[m, n] = X[m, k] W[n, k]^T, bfloat16 with 32-bit accumulation, by hipBLASLt called directly; `workspace` is
+// device memory its kernels may use.  The first call with a shape makes and keeps that shape's plan in host memory.
+int pa_gemm_library(void* stream, const void* x, const void* w, void* c, int m, int n, int k, long ldx, long ldc,
+                    void* workspace, long workspace_bytes);
 // C[m, n] = A[m, k] W[n, k]^T (+ bias[n]), true 32-bit arithmetic.
 int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, const void* w, const float* bias, void* c,
                   int m, int n, int k, long lda, long ldw, long ldc);

@@ -1,10 +1,10 @@
 """Python faces of the HIP kernels: shape and type checks on the host, then one launch.
 
 Every function works on CUDA (HIP) tensors and launches on torch's current
-stream.  Nothing here computes on the CPU or through a torch operator, except
-``linear`` in bfloat16 for tall inputs, which calls the library matrix product
-(hipBLASLt through ``torch.matmul``) where the reference calls its GEMM
-libraries (crates/prelude-cuda/src/ops/gemm.rs:35-137).
+stream.  Nothing here computes on the CPU or through a torch operator;
+``linear`` in bfloat16 for tall inputs calls the library matrix product
+(hipBLASLt, directly) where the reference calls its GEMM libraries
+(crates/prelude-cuda/src/ops/gemm.rs:35-137).
 """
 from __future__ import annotations
 
@@ -311,6 +311,26 @@ def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     return out
 
 
+LIBRARY_WORKSPACE_BYTES = 76 << 20   # what the library's stream-K kernels may use for partial sums
+_library_workspaces: dict = {}
+
+
+def gemm_library(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """y = x W^T in bfloat16 with 32-bit accumulation by hipBLASLt, called directly (its plan is kept per shape:
+    a call through ``torch.matmul`` costs the host some 20 us, this one 14)."""
+    _dev(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise NativeError(f"gemm_library: x {tuple(x.shape)} {x.dtype} / w {tuple(w.shape)} {w.dtype}")
+    m, k = x.shape
+    n = w.shape[0]
+    ws = _library_workspaces.get(x.device)
+    if ws is None:
+        ws = _library_workspaces[x.device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    check(kernels().pa_gemm_library(_stream(), _ptr(x), _ptr(w), _ptr(out), m, n, k, k, n, _ptr(ws), LIBRARY_WORKSPACE_BYTES))
+    return out
+
+
 def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T (+ b), W [out, in] as a tensor or a ``LinearWeight``.  float32: our own true 32-bit product.
@@ -329,7 +349,7 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
-    y = torch.matmul(x, w.t())
+    y = gemm_library(x, w)
     if bias is not None:
         add_bias_(y, bias)
     if out_dtype is not None and out_dtype != y.dtype:
