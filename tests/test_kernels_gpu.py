@@ -519,6 +519,21 @@ def test_prefill_attention_refuses_a_cut_the_shape_does_not_take(gpu):
         paged_case(gpu, torch.bfloat16, 4, 2, 64, 4, [(70, 70)], 0, kernel="mfma", cut=(-1, -1, -1, 1))
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window,seqs", [
+    (2, 1, 128, 16, 0, [(40000, 130), (50001, 1)]),
+    (4, 2, 64, 64, 3000, [(45000, 70), (33000, 1)]),
+    (2, 2, 128, 128, 0, [(70000, 2), (131072, 1)])])
+def test_attention_long_contexts(gpu, nh, nkv, hd, page, window, seqs):
+    """Contexts of tens of thousands of tokens: thousands of pages a request, every split of a decoding request
+    at work, a window that has passed most of the pages."""
+    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=2, kernel="mfma")
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.bfloat16)
+    if max(c for c, _ in seqs) <= 50001:
+        out, ref = paged_case(gpu, torch.float32, nh, nkv, hd, page, seqs, window, seed=2)
+        close(out, ref, torch.float32, f32=3e-6)
+
+
 def draw_attention_case(seed: int):
     rng = np.random.default_rng(seed)
     hd = int(rng.choice([16, 32, 48, 64, 96, 128]))
