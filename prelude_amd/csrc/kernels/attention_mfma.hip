@@ -456,15 +456,24 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   }
 }
 
-// Merges the splits of one (sequence, head): grid (nh, sequences), a thread per head_dim column.  Every
-// wavefront keeps a split per lane (maximum, weight), sixteen splits' outputs are asked for before the weights
-// are known, and the sums run over the splits in order.
+// Merges the splits of one (sequence, head): grid (nh, sequences), groups of a thread per head_dim column.
+// Every wavefront keeps a split per lane (maximum, weight), sixteen splits' outputs are asked for before the
+// weights are known, and the sums run over the splits in order.  The splits go to the groups in runs of 64
+// (run c to group c mod kMergeGroups), and the groups' sums are added in group order: a request's result
+// depends on its own number of splits alone, and up to 64 splits (16,384 keys) it is one group's sum as it
+// stands.  The launch brings as many groups as the longest context has runs (eight at most): a merge of 512
+// splits by one group waits 32 times for memory, one after the other.
+constexpr int kMergeGroups = 8;
+
 template <int HD>
-__global__ __launch_bounds__((HD + kWave - 1) / kWave* kWave) void attn_decode_merge_kernel(
+__global__ __launch_bounds__(kMergeGroups * ((HD + kWave - 1) / kWave * kWave)) void attn_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int window,
     int split_keys, int max_splits) {
   constexpr int kBatch = 16;
+  constexpr int TPG = (HD + kWave - 1) / kWave * kWave;   // threads a group
+  __shared__ float group_acc[kMergeGroups][TPG];
+  __shared__ float group_l[kMergeGroups];
   const int h = blockIdx.x;
   const int seq = seq_ids[blockIdx.y];
   const int ctx = context_lens[seq];
@@ -473,19 +482,21 @@ __global__ __launch_bounds__((HD + kWave - 1) / kWave* kWave) void attn_decode_m
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int nsplit = (ctx + split_keys - 1) / split_keys - lo / split_keys;
   if (nsplit == 1) return;  // written by the first kernel
-  const int d = threadIdx.x, lane = threadIdx.x % kWave;
+  const int groups = blockDim.x / TPG;                     // the launch's: all runs of the longest context, or eight
+  const int grp = threadIdx.x / TPG, d = threadIdx.x % TPG, lane = threadIdx.x % kWave;
   const bool col = d < HD;
   const size_t base = ((size_t)blockIdx.y * nh + h) * max_splits;
   const float* po = part_o + base * HD + (col ? d : 0);
+  const int first = grp * kWave;                           // this group's first run
   // the first batch of outputs, on its way while the weights are worked out
   float o[kBatch];
 #pragma unroll
-  for (int i = 0; i < kBatch; ++i) o[i] = (col && i < nsplit) ? po[(size_t)i * HD] : 0.f;
+  for (int i = 0; i < kBatch; ++i) o[i] = (col && first + i < nsplit) ? po[(size_t)(first + i) * HD] : 0.f;
   float mm = -INFINITY;
   for (int s = lane; s < nsplit; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
   mm = wave_max(mm);
   float acc = 0.f, l = 0.f;
-  for (int s0 = 0; s0 < nsplit; s0 += kWave) {   // a split per lane; in order of the splits
+  for (int s0 = first; s0 < nsplit; s0 += kMergeGroups * kWave) {   // a split per lane; in order of the splits
     const int s = s0 + lane;
     float f = 0.f, ls = 0.f;
     if (s < nsplit) {
@@ -495,7 +506,7 @@ __global__ __launch_bounds__((HD + kWave - 1) / kWave* kWave) void attn_decode_m
     l += wave_sum(ls);
     const int count = nsplit - s0 < kWave ? nsplit - s0 : kWave;
     for (int b0 = 0; b0 < count; b0 += kBatch) {
-      if (s0 + b0 > 0) {
+      if (s0 + b0 > first) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) o[i] = (col && b0 + i < count) ? po[(size_t)(s0 + b0 + i) * HD] : 0.f;
       }
@@ -507,7 +518,21 @@ __global__ __launch_bounds__((HD + kWave - 1) / kWave* kWave) void attn_decode_m
       }
     }
   }
-  if (col) out[(token * nh + h) * HD + d] = (bf16)(acc / l);
+  if (groups == 1) {
+    if (col) out[(token * nh + h) * HD + d] = (bf16)(acc / l);
+    return;
+  }
+  group_acc[grp][d] = acc;
+  if (d == 0) group_l[grp] = l;
+  __syncthreads();
+  if (grp == 0 && col) {
+    float a = group_acc[0][d], ll = group_l[0];
+    for (int g = 1; g < groups; ++g) {
+      a += group_acc[g][d];
+      ll += group_l[g];
+    }
+    out[(token * nh + h) * HD + d] = (bf16)(a / ll);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -831,8 +856,12 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
                      fq);
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
-    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3((HD + kWave - 1) / kWave * kWave), 0, st,
-                       part_o, part_ml, seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys, max_splits);
+    // a group for every run of 64 splits the longest context can have, eight at most
+    const int runs = (max_splits + kWave - 1) / kWave;
+    const int groups = runs < kMergeGroups ? runs : kMergeGroups;
+    hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(groups * ((HD + kWave - 1) / kWave * kWave)),
+                       0, st, part_o, part_ml, seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys,
+                       max_splits);
     return check_launch("attn_decode_merge");
   }
   return 0;
