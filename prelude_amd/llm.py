@@ -18,6 +18,7 @@ id) has by then been fed one step too many, whose sample is dropped.
 from __future__ import annotations
 
 import dataclasses
+import numbers
 import os
 import time
 from typing import Dict, Iterable, List, Optional, Sequence, Union
@@ -174,7 +175,7 @@ class LLM:
         way, crates/prelude-core/src/engine/run/ar.rs:1557), in the order the
         tokens of a request are generated.
         """
-        single = isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int))
+        single = isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], numbers.Integral))
         plist = [prompts] if single else list(prompts)
         if sampling_params is not None and len(sampling_params) != len(plist):
             raise ValueError("sampling_params must have one entry per prompt")
