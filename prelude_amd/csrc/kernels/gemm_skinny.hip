@@ -62,16 +62,26 @@ enum Epilogue : int { kPlain = 0, kSiluMul = 1 };
 // NT tiles of 16 rows of W per workgroup: with two, every X fragment serves two products, which halves the
 // share of the loads that X makes up (X comes from L2, but the loads cost the same as any).
 // A fragment of a weight stored in tiles (see pa_pack_tiles): the wavefront's 64 lanes read 1 KB side by side.
-__device__ __forceinline__ Frag load_tiled(const bf16* tile, int step, int lane, bool ok) {
+// No load of the tiled kernel stands under a condition: a step past the end reads the last step again (its
+// product is left out), a row past m reads row 0 (its column of the result is never stored), and columns past K
+// read the row's first ones (the tiles hold zeros there, and a row is only ever mixed with itself).  Straight
+// code is a microsecond a product faster at 8 and 16 rows than loads behind lane masks, and it is what lets the
+// compiler count the loads in flight at all: after a load that may or may not have been issued it waits for all
+// of them.  (With the count right, more than one step in flight per wavefront was measured again, 2 to 4 steps
+// at the shapes of a 4B model: still slower than one, by 5 to 50 %.)
+__device__ __forceinline__ Frag load_tiled(const bf16* tile, int step, int lane) {
   Frag f;
-  if (ok) {
-    const bf16* p = tile + (size_t)step * 1024 + lane * 8;
-    f.lo = *reinterpret_cast<const bf16x8*>(p);
-    f.hi = *reinterpret_cast<const bf16x8*>(p + 512);
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f.lo[i] = f.hi[i] = (bf16)0.f;
-  }
+  const bf16* p = tile + (size_t)step * 1024 + lane * 8;
+  f.lo = *reinterpret_cast<const bf16x8*>(p);
+  f.hi = *reinterpret_cast<const bf16x8*>(p + 512);
+  return f;
+}
+
+// X for a tiled product: row + 16 g + 64 step, both halves; k_rest = K - 16 g.
+__device__ __forceinline__ Frag load_x_always(const bf16* row, int k0, int k_rest) {
+  Frag f;
+  f.lo = *reinterpret_cast<const bf16x8*>(row + (k0 + 8 <= k_rest ? k0 : 0));
+  f.hi = *reinterpret_cast<const bf16x8*>(row + (k0 + 16 <= k_rest ? k0 + 8 : 0));
   return f;
 }
 
@@ -82,7 +92,9 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
                                                                    TC* __restrict__ c, int m, int n, int k, long ldx,
                                                                    long ldc) {
   __shared__ float red[WAVES][NT * MT][kWave][4];
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  // the wavefront's number as a scalar: what depends on it (the steps it takes, the loop's end) is then uniform
+  // for the compiler too, and a branch on it is a branch, not a mask
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int n0 = blockIdx.x * 16 * NT;
   const int steps = (k + 63) / 64;
@@ -109,18 +121,20 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
     for (int t = 0; t < MT; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // DEPTH k-steps in flight per wavefront: a ring of fragments, refilled as soon as a slot has been used.
-  // Steps past the end load zeros, so the ring needs no tail handling.
+  // Steps past the end load zeros (rows) or the last step again, left out of the sums (tiles): no tail handling.
   const int kk = k - 16 * g;
+  const int last = steps - 1;
   Frag wbuf[DEPTH][NT], xbuf[DEPTH][MT];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
     const int s = wave + d * WAVES;
+    const int sc = s < steps ? s : last;
 #pragma unroll
     for (int u = 0; u < NT; ++u)
-      wbuf[d][u] = TILED ? load_tiled(wrow[u], s, lane, n_ok[u] && s < steps)
-                         : load_frag(wrow[u], s * 64, kk, n_ok[u] && s < steps);
+      wbuf[d][u] = TILED ? load_tiled(wrow[u], sc, lane) : load_frag(wrow[u], s * 64, kk, n_ok[u] && s < steps);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
+    for (int t = 0; t < MT; ++t)
+      xbuf[d][t] = TILED ? load_x_always(xrow[t], sc * 64, kk) : load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
   }
   for (int s0 = wave; s0 < steps; s0 += WAVES * DEPTH) {
 #pragma unroll
@@ -131,12 +145,15 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
       for (int t = 0; t < MT; ++t) xc[t] = xbuf[d][t];
       const int next = s0 + (d + DEPTH) * WAVES;
+      const int nc = next < steps ? next : last;
 #pragma unroll
       for (int u = 0; u < NT; ++u)
-        wbuf[d][u] = TILED ? load_tiled(wrow[u], next, lane, n_ok[u] && next < steps)
-                           : load_frag(wrow[u], next * 64, kk, n_ok[u] && next < steps);
+        wbuf[d][u] = TILED ? load_tiled(wrow[u], nc, lane) : load_frag(wrow[u], next * 64, kk, n_ok[u] && next < steps);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) xbuf[d][t] = load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
+      for (int t = 0; t < MT; ++t)
+        xbuf[d][t] = TILED ? load_x_always(xrow[t], nc * 64, kk)
+                           : load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
+      if (TILED && s0 + d * WAVES >= steps) continue;   // a step past the end: read again, not counted (no load inside)
 #pragma unroll
       for (int u = 0; u < NT; ++u)
 #pragma unroll
