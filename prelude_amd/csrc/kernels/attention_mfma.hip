@@ -651,10 +651,10 @@ struct StageLds {
 // KW = 64 / WAVES keys KW w .. of a block of 64: of K, lane (r = lane / QL, q = lane % QL; QL = 64 / KW) takes the
 // 16-byte pieces q, q + QL, .. of key KW w + r, so that the lanes of a load cover whole 64-byte stretches of a row
 // (a lane per row would ask the memory pipeline for four times as many of them); of V^T, lane (d = lane / HL, h = lane % HL; HL = KW / 8 halves)
-// takes the eight keys KW w + 8h .. + 7 of the rows d, d + 64 / HL, ...  Pages hold 8 to 64 keys here, so a block
-// starts at a page's first key, and a thread reads one page of each cache per block, at places inside the page
-// that never change.  A page outside the pages [lo_page, hi_page] that hold the tile's keys is replaced by the
-// nearest of those; the scores of its keys are masked.
+// takes the eight keys KW w + 8h .. + 7 of the rows d, d + 64 / HL, ...  Pages hold 8 keys or more here, a power of
+// two: a block of 64 starts at a page's first key or lies inside one page, so a thread reads one page of each cache
+// per block, `base` keys into it (always 0 for pages of up to 64 keys).  A page outside the pages [lo_page, hi_page]
+// that hold the tile's keys is replaced by the nearest of those; the scores of its keys are masked.
 template <int HD, int WAVES>
 struct Stage {
   static_assert(WAVES == 4 || WAVES == 8, "four or eight wavefronts stage a block");
@@ -667,9 +667,10 @@ struct Stage {
   static constexpr int NV = (HD + DL - 1) / DL;
   bf16x8 k[NK];
   bf16x8 v[NV];
-  int kpage, vpage;
+  int kpage, vpage, base;
 
   __device__ __forceinline__ void load_pages(const KeyWalk& w, int key0, int wave, int lane, int lo_page, int hi_page) {
+    base = key0 & w.page_mask;
     int kp = (key0 + KW * wave + lane / QL) >> w.page_shift;
     int vp = (key0 + KW * wave + 8 * (lane % HL)) >> w.page_shift;
     kp = kp < lo_page ? lo_page : (kp > hi_page ? hi_page : kp);
@@ -683,13 +684,13 @@ struct Stage {
     const unsigned head_off = ((unsigned)w.kvh * HD) << w.page_shift;
     const int r = lane / QL, q = lane % QL;
     const bf16* kp = w.kc + ((unsigned long long)(unsigned)kpage * page_elems + head_off +
-                             (unsigned)((KW * wave + r) & w.page_mask) * HD + 8 * q);
+                             (unsigned)((base + KW * wave + r) & w.page_mask) * HD + 8 * q);
 #pragma unroll
     for (int j = 0; j < NK; ++j)
       if (CPK % QL == 0 || QL * j + q < CPK) k[j] = *reinterpret_cast<const bf16x8*>(kp + 8 * QL * j);
     const int d = lane / HL, h = lane % HL;
     const bf16* vp = w.vc + ((unsigned long long)(unsigned)vpage * page_elems + head_off + ((unsigned)d << w.page_shift) +
-                             (unsigned)((KW * wave + 8 * h) & w.page_mask));
+                             (unsigned)((base + KW * wave + 8 * h) & w.page_mask));
 #pragma unroll
     for (int j = 0; j < NV; ++j)
       if (HD % DL == 0 || d + DL * j < HD) v[j] = *reinterpret_cast<const bf16x8*>(vp + ((size_t)(DL * j) << w.page_shift));
@@ -925,7 +926,7 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // as 256 workgroups and 26 us as 64.
   const int gt_best = (HD <= 64 && group % 4 == 0) ? 4 : (group % 2 == 0 ? 2 : 1);
   const long tiles = (max_q_len + 63) / 64;
-  const bool can_stage = page_shift >= 3 && page_shift <= 6;
+  const bool can_stage = page_shift >= 3;
   auto workgroups = [&](int p, int g_, int h_ = 1) {
     return (p ? (tiles + 1) / 2 : tiles) * nkv * (group / (g_ * h_)) * nseq;
   };
@@ -962,7 +963,7 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
       hw = 2;
     }
   }
-  // keys staged in LDS for pages of 8 to 64 keys; smaller and larger pages go to the kernel that reads them itself
+  // keys staged in LDS for pages of 8 keys or more; pages of 4 go to the kernel that reads them itself
   bool staged = can_stage;
   // a caller's own cut (tests and measurements), where it is one the kernels have
   if (want.paired >= 0) paired = want.paired != 0 && tiles >= 2;

@@ -473,7 +473,8 @@ def test_mfma_attention_far_key_and_edges(gpu):
             assert (float(out[-1].float().abs().max()) > 50.0) == seen
 
 
-@pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0)])
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0),
+                                                   (8, 2, 128, 128, 0), (4, 2, 64, 256, 100)])
 def test_prefill_attention_every_cut(gpu, nh, nkv, hd, page, window):
     """The launcher cuts a prefill by the size of the step (tiles in pairs, 1, 2 or 4 heads a wavefront, one or two
     head groups a workgroup, keys staged in LDS or not); small cases would only ever see one cut, so each is
