@@ -459,14 +459,19 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
 // Merges the splits of one (sequence, head): grid (nh, sequences), groups of a thread per head_dim column.
 // Every wavefront keeps a split per lane (maximum, weight), sixteen splits' outputs are asked for before the
 // weights are known, and the sums run over the splits in order.  The splits go to the groups in runs of 64
-// (run c to group c mod kMergeGroups), and the groups' sums are added in group order: a request's result
+// (run c to group c mod merge_groups_of(HD)), and the groups' sums are added in group order: a request's result
 // depends on its own number of splits alone, and up to 64 splits (16,384 keys) it is one group's sum as it
 // stands.  The launch brings as many groups as the longest context has runs (eight at most): a merge of 512
 // splits by one group waits 32 times for memory, one after the other.
 constexpr int kMergeGroups = 8;
+// ... as far as a workgroup's 1,024 threads go: heads wider than 128 get fewer groups
+constexpr int merge_groups_of(int hd) {
+  const int threads = (hd + kWave - 1) / kWave * kWave;
+  return kMergeGroups * threads <= 1024 ? kMergeGroups : 1024 / threads;
+}
 
 template <int HD>
-__global__ __launch_bounds__(kMergeGroups * ((HD + kWave - 1) / kWave * kWave)) void attn_decode_merge_kernel(
+__global__ __launch_bounds__(merge_groups_of(HD) * ((HD + kWave - 1) / kWave * kWave)) void attn_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int window,
     int split_keys, int max_splits) {
@@ -496,7 +501,7 @@ __global__ __launch_bounds__(kMergeGroups * ((HD + kWave - 1) / kWave * kWave)) 
   for (int s = lane; s < nsplit; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
   mm = wave_max(mm);
   float acc = 0.f, l = 0.f;
-  for (int s0 = first; s0 < nsplit; s0 += kMergeGroups * kWave) {   // a split per lane; in order of the splits
+  for (int s0 = first; s0 < nsplit; s0 += merge_groups_of(HD) * kWave) {   // a split per lane; in order of the splits
     const int s = s0 + lane;
     float f = 0.f, ls = 0.f;
     if (s < nsplit) {
@@ -859,7 +864,7 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   if (max_splits > 1) {
     // a group for every run of 64 splits the longest context can have, eight at most
     const int runs = (max_splits + kWave - 1) / kWave;
-    const int groups = runs < kMergeGroups ? runs : kMergeGroups;
+    const int groups = runs < merge_groups_of(HD) ? runs : merge_groups_of(HD);
     hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(groups * ((HD + kWave - 1) / kWave * kWave)),
                        0, st, part_o, part_ml, seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys,
                        max_splits);

@@ -77,11 +77,13 @@ __device__ __forceinline__ Frag load_tiled(const bf16* tile, int step, int lane)
   return f;
 }
 
-// X for a tiled product: row + 16 g + 64 step, both halves; k_rest = K - 16 g.
-__device__ __forceinline__ Frag load_x_always(const bf16* row, int k0, int k_rest) {
+// X for a tiled product: columns at, at + 8 .. of a row of k columns, both halves.  A half that would pass the
+// row's end reads the row's first eight columns instead (k is a multiple of 8 and at least 8): memory of the same
+// row, always there, and finite where the row is; the tile holds zeros at those places.
+__device__ __forceinline__ Frag load_x_always(const bf16* row, int at, int k) {
   Frag f;
-  f.lo = *reinterpret_cast<const bf16x8*>(row + (k0 + 8 <= k_rest ? k0 : 0));
-  f.hi = *reinterpret_cast<const bf16x8*>(row + (k0 + 16 <= k_rest ? k0 + 8 : 0));
+  f.lo = *reinterpret_cast<const bf16x8*>(row + (at + 8 <= k ? at : 0));
+  f.hi = *reinterpret_cast<const bf16x8*>(row + (at + 16 <= k ? at + 8 : 0));
   return f;
 }
 
@@ -112,7 +114,8 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     m_ok[t] = 16 * t + r < m;
-    xrow[t] = x + (size_t)(m_ok[t] ? 16 * t + r : 0) * ldx + 16 * g;
+    // a tiled product addresses X from the row's start (its loads stand under no condition and must stay inside the row)
+    xrow[t] = x + (size_t)(m_ok[t] ? 16 * t + r : 0) * ldx + (TILED ? 0 : 16 * g);
   }
   f32x4 acc[NT][MT];
 #pragma unroll
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
       wbuf[d][u] = TILED ? load_tiled(wrow[u], sc, lane) : load_frag(wrow[u], s * 64, kk, n_ok[u] && s < steps);
 #pragma unroll
     for (int t = 0; t < MT; ++t)
-      xbuf[d][t] = TILED ? load_x_always(xrow[t], sc * 64, kk) : load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
+      xbuf[d][t] = TILED ? load_x_always(xrow[t], sc * 64 + 16 * g, k) : load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
   }
   for (int s0 = wave; s0 < steps; s0 += WAVES * DEPTH) {
 #pragma unroll
@@ -151,7 +154,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
         wbuf[d][u] = TILED ? load_tiled(wrow[u], nc, lane) : load_frag(wrow[u], next * 64, kk, n_ok[u] && next < steps);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
-        xbuf[d][t] = TILED ? load_x_always(xrow[t], nc * 64, kk)
+        xbuf[d][t] = TILED ? load_x_always(xrow[t], nc * 64 + 16 * g, k)
                            : load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
       if (TILED && s0 + d * WAVES >= steps) continue;   // a step past the end: read again, not counted (no load inside)
 #pragma unroll

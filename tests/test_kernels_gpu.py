@@ -163,6 +163,24 @@ def test_gemm_skinny(gpu, m, n, k):
         close(K().linear(xd, K().LinearWeight(wd, tiles)), ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("m,n,k", [(30, 24, 16), (4, 76, 24), (16, 48, 40), (1, 32, 8), (39, 2304, 24), (64, 40, 72)])
+def test_gemm_skinny_stays_inside_its_rows(gpu, m, n, k):
+    """Rows shorter than a step of 64 columns, or ending inside one: what lies behind a row of X is not the
+    product's to read.  X is the head of a buffer whose rest is NaN (and a row stride wider than k keeps NaN behind
+    every row): a read past a row's end, even one multiplied by the tile's zeros, would show in the result."""
+    w = rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05)
+    x = rnd(m, k, dtype=torch.bfloat16)
+    ref = x.double() @ w.double().T
+    wd = w.to(gpu)
+    tiles = K().pack_tiles(wd)
+    behind = torch.full((m + 8, k), float("nan"), dtype=torch.bfloat16, device=gpu)
+    behind[:m] = x.to(gpu)
+    for weight in (tiles, wd):
+        got = K().gemm_skinny(behind[:m], weight, out_dtype=torch.float32)
+        assert bool(torch.isfinite(got).all()), f"read behind X with a {'tiled' if weight is tiles else 'row-major'} weight"
+        close(got, ref, torch.float32, f32=2e-5)
+
+
 @pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_PRODUCTS", "12")))))   # widen for a hunt
 def test_drawn_products(gpu, seed):
     """Rows, outputs and inner size drawn at random, through the dispatcher and through the weight-streaming kernel
