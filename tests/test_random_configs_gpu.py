@@ -32,7 +32,7 @@ def draw_config(seed: int) -> tuple:
                tie_word_embeddings=bool(rng.integers(0, 2)), rope_theta=float(rng.choice([100.0, 10000.0, 1e6])),
                rms_norm_eps=float(rng.choice([1e-6, 1e-5, 3e-4])), use_sliding_window=bool(window),
                hidden_act="silu", eos_token_id=0)
-    page = int(rng.choice([4, 8, 16, 32, 64]))
+    page = int(rng.choice([4, 8, 16, 32, 64, 128]))
     return cfg, page
 
 
