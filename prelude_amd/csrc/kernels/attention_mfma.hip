@@ -376,7 +376,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   const int group = nh / nkv;
   const int qtiles = (group + 15) / 16;
   const int kvh = blockIdx.y / qtiles, qt = blockIdx.y % qtiles;
-  const int seq = seq_ids[blockIdx.z];
+  const int seq = seq_ids ? seq_ids[blockIdx.z] : (int)blockIdx.z;   // no list: every sequence of the step
   const int ctx = context_lens[seq];
   const int pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(merge_groups_of(HD) * ((HD + kWave - 1) / kWave * k
   __shared__ float group_acc[kMergeGroups][TPG];
   __shared__ float group_l[kMergeGroups];
   const int h = blockIdx.x;
-  const int seq = seq_ids[blockIdx.y];
+  const int seq = seq_ids ? seq_ids[blockIdx.y] : (int)blockIdx.y;
   const int ctx = context_lens[seq];
   const size_t token = cu_q[seq];
   const int pos = ctx - 1;

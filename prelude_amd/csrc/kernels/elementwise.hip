@@ -93,12 +93,18 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const f
   vec_t* orow = reinterpret_cast<vec_t*>(out + (size_t)r * hidden);
   const int nvec = hidden / VEC;
   float s[NV][VEC];
+  float wv[NV][VEC];   // the scale, asked for with the row: its way from memory is not waited for after the sum
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int v = threadIdx.x + j * blockDim.x;
     if (v < nvec) {
       const vec_t xv = xr[v];
+#pragma unroll
+      for (int e = 0; e < VEC; e += 4) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + (size_t)v * VEC + e);
+        wv[j][e] = w4.x, wv[j][e + 1] = w4.y, wv[j][e + 2] = w4.z, wv[j][e + 3] = w4.w;
+      }
       if (rr) {
         const vec_t rv = rr[v];
 #pragma unroll
@@ -121,7 +127,7 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const f
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         sv[e] = from_f32<T>(s[j][e]);
-        ov[e] = from_f32<T>(s[j][e] * inv * w[v * VEC + e]);
+        ov[e] = from_f32<T>(s[j][e] * inv * wv[j][e]);
       }
       if (rr && !rows) rr[v] = sv;
       orow[v] = ov;

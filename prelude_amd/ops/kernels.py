@@ -418,8 +418,10 @@ def mfma_attention_supported(head_dim: int, page_size: int) -> bool:
 
 
 def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_context: int,
-                     window: int, scale: float) -> None:
-    """Matrix-core attention for the sequences ``seq_ids`` (each feeding one token); writes their rows of ``out``."""
+                     window: int, scale: float, every_seq: bool = False) -> None:
+    """Matrix-core attention for the sequences ``seq_ids`` (each feeding one token); writes their rows of ``out``.
+    ``every_seq``: ``seq_ids`` is 0, 1, .. (a step of single tokens only); the kernels then count for themselves
+    instead of reading it, which is one trip to memory less before their first key."""
     _dev(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out)
     t, nh, hd = q.shape
     _check_caches(k_cache, v_cache, k_cache.shape[1], hd, torch.bfloat16, "attention_decode")
@@ -431,7 +433,8 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_le
     words = kernels().pa_attn_decode_workspace(n, nh, hd, max_splits)
     ws = torch.empty((max(words, 1),), dtype=torch.float32, device=q.device)
     check(kernels().pa_attn_decode(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
-                                   block_table.shape[1], _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out),
+                                   block_table.shape[1], None if every_seq else _ptr(seq_ids), _ptr(cu_q),
+                                   _ptr(context_lens), _ptr(out),
                                    _ptr(ws), n, nh, k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale),
                                    DECODE_SPLIT_KEYS, max_splits))
 
@@ -442,7 +445,7 @@ def attention_decode_fused_supported(nh: int, nkv: int, hd: int, rot: int, page_
 
 def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float, k_cache, v_cache,
                            block_table, seq_ids, cu_q, context_lens, nh: int, max_context: int, window: int,
-                           scale: float) -> torch.Tensor:
+                           scale: float, every_seq: bool = False) -> torch.Tensor:
     """``qknorm_rope_kv`` and ``attention_decode`` in one kernel, for a step in which every sequence feeds one
     token: takes the merged projection [T, (nh + 2 nkv) * hd], writes the tokens' keys and values into the caches
     and returns the attention output [T, nh, hd].  A token's position is its sequence's context length less one."""
@@ -469,7 +472,8 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
     ws = torch.empty((max(words, 1),), dtype=torch.float32, device=qkv.device)
     check(kernels().pa_attn_decode_fused(_stream(), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin),
                                          _ptr(slots), float(eps), _ptr(k_cache), _ptr(v_cache),
-                                         _ptr(block_table), block_table.shape[1], _ptr(seq_ids), _ptr(cu_q),
+                                         _ptr(block_table), block_table.shape[1],
+                                         None if every_seq else _ptr(seq_ids), _ptr(cu_q),
                                          _ptr(context_lens), _ptr(out), _ptr(ws), n, nh, nkv, hd, page, int(window),
                                          float(scale), DECODE_SPLIT_KEYS, max_splits))
     return out
@@ -512,7 +516,8 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
         out = torch.empty_like(q)
         if step.n_decode:
             attention_decode(q, k_cache, v_cache, group.block_table, step.decode_seqs, step.cu_q, step.context_lens,
-                             out, step.max_decode_context, window, scale)
+                             out, step.max_decode_context, window, scale,
+                             every_seq=step.n_prefill == 0 and step.n_decode == step.num_seqs)
         if step.n_prefill:
             attention_prefill(q, k_cache, v_cache, group.block_table, step.prefill_seqs, step.cu_q, step.context_lens,
                               out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix)

@@ -90,7 +90,7 @@ class GQAAttention(Mixer):
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
             o = K.attention_decode_fused(qkv, self.q_norm, self.k_norm, cos, sin, g.slots, self.norm_eps,
                                          cache.k, cache.v, g.block_table, step.decode_seqs, step.cu_q, step.context_lens,
-                                         nh, step.max_decode_context, self.window, self.scale)
+                                         nh, step.max_decode_context, self.window, self.scale, every_seq=True)
             return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o)
         if write_cache:
             qkv = K.linear(x, self.w_qkv, self.b_qkv)

@@ -394,6 +394,11 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
         ctxs = i32([c for c, _ in seqs])
         K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, out, max([seqs[i][0] for i in dec], default=0),
                              window, 1.0 / math.sqrt(hd))
+        if dec and not pre:   # a step of single tokens: the kernels may count the sequences themselves, same bits
+            again = torch.full_like(qd, float("nan"))
+            K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, again, max(seqs[i][0] for i in dec), window,
+                                 1.0 / math.sqrt(hd), every_seq=True)
+            assert torch.equal(again, out)
         K().attention_prefill(qd, kd, vd, td, i32(pre), i32(cu), ctxs, out, max([seqs[i][1] for i in pre], default=0),
                               window, 1.0 / math.sqrt(hd), cut=cut,
                               min_prefix=min([seqs[i][0] - seqs[i][1] for i in pre], default=0))
@@ -551,6 +556,18 @@ def test_attention_long_contexts(gpu, nh, nkv, hd, page, window, seqs):
     if max(c for c, _ in seqs) <= 50001:
         out, ref = paged_case(gpu, torch.float32, nh, nkv, hd, page, seqs, window, seed=2)
         close(out, ref, torch.float32, f32=3e-6)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [(32, 8, 128, 16, 0), (8, 2, 64, 8, 0), (4, 1, 96, 32, 100),
+                                                   (6, 3, 128, 128, 0), (2, 2, 32, 4, 0)])
+def test_decode_attention_of_single_tokens_only(gpu, nh, nkv, hd, page, window):
+    """A step of single tokens: contexts that end at, just before and just behind the edge of a split and of a page
+    (the pages of a split are looked up before the length is known, and a key past the end is read from the last
+    one there is); table entries behind a sequence's last page are -1."""
+    seqs = [(1, 1), (255, 1), (256, 1), (257, 1), (1000, 1), (4097, 1), (31, 1), (33, 1), (512, 1), (769, 1)]
+    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=4, kernel="mfma")
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.bfloat16)
 
 
 def draw_attention_case(seed: int):
