@@ -255,6 +255,44 @@ def test_graph_replays_equal_eager_steps(gpu):
         assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
 
 
+def test_graph_replays_with_library_products_equal_eager_steps(gpu):
+    """A decode step of more than 48 requests multiplies through the library product, also inside a captured
+    graph (with its workspace): every replay, with eager steps of other shapes between them, gives the eager
+    step's logits bit for bit."""
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    folder, cfg, _ = model_folder("b")
+    rng = np.random.default_rng(5)
+    n = 56
+    seqs = [rng.integers(0, cfg["vocab_size"], size=40).tolist() for _ in range(n)]
+
+    def play(hip_graph):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=n * 48,
+                                                         hip_graph=hip_graph))
+        outs, at = [], [0] * n
+
+        def feed(parts):
+            entries = []
+            for r, k in parts:
+                entries.append(StepEntry(r, seqs[r][at[r]:at[r] + k], [k - 1]))
+                at[r] += k
+            outs.append(eng.step(entries).cpu())
+        feed([(r, 7 + r % 5) for r in range(n)])
+        for i in range(4):
+            feed([(r, 1) for r in range(n)])      # the graph of 56 single tokens: capture, then replays
+            feed([(i, 2), (n - 1 - i, 3)])        # eager work between the replays
+            torch.cuda.synchronize()
+        for _ in range(3):
+            feed([(r, 1) for r in range(n)])
+        return eng, outs
+
+    eager_eng, eager = play(False)
+    graph_eng, graphed = play(True)
+    assert graph_eng._graphs.captures >= 1 and graph_eng._graphs.replays >= 6
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
+
+
 @pytest.mark.parametrize("dtype,hip_graph", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
 def test_tokens_carried_on_the_device(gpu, dtype, hip_graph):
     """A step whose last tokens are taken from a device tensor (the previous step's samples, never read by the
