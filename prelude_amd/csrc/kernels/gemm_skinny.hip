@@ -156,6 +156,11 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
       for (int t = 0; t < MT; ++t)
         xbuf[d][t] = TILED ? load_x_always(xrow[t], nc * 64 + 16 * g, k)
                            : load_frag(xrow[t], next * 64, kk, m_ok[t] && next < steps);
+      // with two tiles or more, every load of the next step is on its way before this step's products: left to
+      // itself the compiler moves the loads of a second tile behind the products of the first (fewer registers, and
+      // half the bytes in flight: [5120, 25600] at 8 rows took 69 us so, 49 with the loads held together); with one
+      // tile its own order is the faster one by half a microsecond
+      if (TILED && NT > 1) __builtin_amdgcn_sched_barrier(0);
       if (TILED && s0 + d * WAVES >= steps) continue;   // a step past the end: read again, not counted (no load inside)
 #pragma unroll
       for (int u = 0; u < NT; ++u)
@@ -234,7 +239,9 @@ static void skinny_shape(int m, int n, int k, int mt, bool tiled, int* nt, int* 
       // eight wavefronts on two tiles stream better than sixteen on one ([5120, 25600] at 1 / 8 / 16 rows:
       // 52 / 51 / 57 against 55 / 60 / 83 us; [4096, 12288], 256 tiles, is still better off with sixteen on one)
       *waves = 8;
-      if (tiles >= 320) *nt = 2;
+      // ... two tiles except for up to 4 rows of rows shorter than 256 steps ([5120, 8192] at 1 / 4 / 8 rows:
+      // 17 / 17 / 20 us on one tile against 19 to 20 on two)
+      if (tiles >= 320 && (m > 4 || steps >= 256)) *nt = 2;
     }
     *depth = 1;
     return;
