@@ -295,6 +295,13 @@ __device__ __forceinline__ void fused_write_kv(const FusedQkv& f, bf16* kc, bf16
   const bf16* vrow = f.qkv + (token * heads + nh + nkv + kvh) * HD;
   const vec_t kv = *reinterpret_cast<const vec_t*>(krow + lane * EPL);
   const vec_t vv = *reinterpret_cast<const vec_t*>(vrow + lane * EPL);
+  // the scale and the angles of the lane's elements, asked for with the rows (not one by one after the sum)
+  typedef float fvec_t __attribute__((ext_vector_type(EPL)));
+  const int j0 = (lane % 32) * EPL;
+  fvec_t kw;
+  if (f.k_weight) kw = *reinterpret_cast<const fvec_t*>(f.k_weight + lane * EPL);
+  const fvec_t csv = *reinterpret_cast<const fvec_t*>(f.cos_table + (size_t)pos * (HD / 2) + j0);
+  const fvec_t snv = *reinterpret_cast<const fvec_t*>(f.sin_table + (size_t)pos * (HD / 2) + j0);
   bf16* vdst = vc + ((((size_t)page * nkv + kvh) * HD) << page_shift) + off;
 #pragma unroll
   for (int e = 0; e < EPL; ++e) vdst[(size_t)(lane * EPL + e) << page_shift] = vv[e];
@@ -306,18 +313,20 @@ __device__ __forceinline__ void fused_write_kv(const FusedQkv& f, bf16* kc, bf16
   }
   ss = wave_sum(ss);
   const float inv = rsqrtf(ss / (float)HD + f.eps);
-  const int j0 = (lane % 32) * EPL;
   vec_t ov;
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
-    if (f.k_weight) x[e] = x[e] * inv * f.k_weight[lane * EPL + e];
+    if (f.k_weight) x[e] = x[e] * inv * kw[e];
     const float partner = __shfl_xor(x[e], 32, kWave);
-    const float cs = f.cos_table[(size_t)pos * (HD / 2) + j0 + e], sn = f.sin_table[(size_t)pos * (HD / 2) + j0 + e];
+    const float cs = csv[e], sn = snv[e];
     ov[e] = (bf16)(lane < 32 ? x[e] * cs - partner * sn : partner * sn + x[e] * cs);
   }
   bf16* kdst = kc + ((((size_t)page * nkv + kvh) << page_shift) + off) * HD;
   *reinterpret_cast<vec_t*>(kdst + lane * EPL) = ov;
 }
+
+// Element i of a float4 (i known when the loops around it are unrolled).
+__device__ __forceinline__ float f4(const float4& v, int i) { return i == 0 ? v.x : (i == 1 ? v.y : (i == 2 ? v.z : v.w)); }
 
 // Q^T of one head as B operands from the raw projection: normed and rotated in the lane.  Lane (g, r) holds
 // head_dim 32 ks + 8g .. + 7 of its head; the element head_dim / 2 further on, its rotation partner, is in
@@ -326,15 +335,37 @@ template <int HD>
 __device__ __forceinline__ void fused_load_q(const FusedQkv& f, const bf16* qrow, bool valid, int pos, int g, bf16x8* qf) {
   constexpr int KS = HD / 32;
   static_assert(HD == 64 || HD == 128, "the rotation partner must sit in the same lane");
+  // Everything the lane needs is asked for at once, in 16-byte pieces: its elements of the row, and for each of
+  // its KS / 2 first-half stretches of eight elements the two stretches of the norm's scale and the angles' cosines
+  // and sines.  (Element by element, under the test for a scale, the loads had been issued and waited for one
+  // pair at a time: sixteen trips to the cache in a row.)
+  bf16x8 raw[KS];
+  float4 wa[KS / 2][2], wb[KS / 2][2], cs4[KS / 2][2], sn4[KS / 2][2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    raw[ks] = zero8();
+    if (valid) raw[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * g);
+  }
+#pragma unroll
+  for (int ks = 0; ks < KS / 2; ++ks) {
+    const int d = 32 * ks + 8 * g;   // the first-half element; its partner is d + HD / 2
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (f.q_weight) {
+        wa[ks][h] = *reinterpret_cast<const float4*>(f.q_weight + d + 4 * h);
+        wb[ks][h] = *reinterpret_cast<const float4*>(f.q_weight + d + HD / 2 + 4 * h);
+      }
+      cs4[ks][h] = *reinterpret_cast<const float4*>(f.cos_table + (size_t)pos * (HD / 2) + d + 4 * h);
+      sn4[ks][h] = *reinterpret_cast<const float4*>(f.sin_table + (size_t)pos * (HD / 2) + d + 4 * h);
+    }
+  }
   float x[KS][8];
   float ss = 0.f;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    bf16x8 raw = zero8();
-    if (valid) raw = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * g);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      x[ks][j] = (float)raw[j];
+      x[ks][j] = (float)raw[ks][j];
       ss += x[ks][j] * x[ks][j];
     }
   }
@@ -342,16 +373,15 @@ __device__ __forceinline__ void fused_load_q(const FusedQkv& f, const bf16* qrow
   const float inv = rsqrtf(ss / (float)HD + f.eps);
 #pragma unroll
   for (int ks = 0; ks < KS / 2; ++ks) {
-    const int d = 32 * ks + 8 * g;   // the first-half element; its partner is d + HD / 2
     bf16x8 lo, hi;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float a = x[ks][j], b = x[ks + KS / 2][j];
       if (f.q_weight) {
-        a = a * inv * f.q_weight[d + j];
-        b = b * inv * f.q_weight[d + HD / 2 + j];
+        a = a * inv * f4(wa[ks][j / 4], j % 4);
+        b = b * inv * f4(wb[ks][j / 4], j % 4);
       }
-      const float cs = f.cos_table[(size_t)pos * (HD / 2) + d + j], sn = f.sin_table[(size_t)pos * (HD / 2) + d + j];
+      const float cs = f4(cs4[ks][j / 4], j % 4), sn = f4(sn4[ks][j / 4], j % 4);
       lo[j] = (bf16)(a * cs - b * sn);
       hi[j] = (bf16)(a * sn + b * cs);
     }
