@@ -80,6 +80,27 @@ def test_whole_then_decoded_then_mixed(gpu, dtype):
     assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
 
 
+def test_twenty_requests_decode_together(gpu):
+    """Twenty requests at different places of the same sequence feed one token each, step after step: the decode
+    attention that takes the raw projection (QK-norm, rotation and the cache write inside it) with more sequences
+    than the products of few rows take, so the streaming and the library products feed it in turn."""
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref, _ = wide_model()
+    r = TraceRunner(folder, "bfloat16", 20 * 96, page_size=16)
+    starts = [3 + 4 * i for i in range(20)]
+    for i, s in enumerate(starts):
+        r.step([{"id": f"r{i}", "tokens": toks[:s], "want": []}])
+    rows = [[] for _ in starts]
+    for k in range(5):
+        out = r.step([{"id": f"r{i}", "tokens": [toks[s + k]], "want": [0]} for i, s in enumerate(starts)])
+        for i in range(len(starts)):
+            rows[i].append(out[i:i + 1])
+    for i, s in enumerate(starts):
+        check(np.concatenate(rows[i]), ref[s:s + 5], "bfloat16", f"request {i} from position {s}")
+    r.step([], [f"r{i}" for i in range(20)])
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
 def test_greedy_generation_at_real_widths(gpu):
     from prelude_amd import LLM
     folder, toks, _, w64 = wide_model()
