@@ -60,6 +60,7 @@ int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache,
 // seq_ids lists the sequences of the step a call handles; cu_q[s] is the first packed token row of sequence s,
 // context_lens[s] its tokens in the cache after the step.  Decode takes sequences that feed one token and cuts
 // each one's keys into splits of split_keys; workspace must hold pa_attn_decode_workspace(...) floats.
+// The two decode entry points take seq_ids = null for the sequences 0 .. nseq - 1 (a step of single tokens only).
 int pa_attn_mfma_supports(int hd, int page_size);
 long pa_attn_decode_workspace(int nseq, int nh, int hd, int max_splits);
 int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,

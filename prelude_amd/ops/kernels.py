@@ -466,7 +466,8 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
                            scale: float, every_seq: bool = False) -> torch.Tensor:
     """``qknorm_rope_kv`` and ``attention_decode`` in one kernel, for a step in which every sequence feeds one
     token: takes the merged projection [T, (nh + 2 nkv) * hd], writes the tokens' keys and values into the caches
-    and returns the attention output [T, nh, hd].  A token's position is its sequence's context length less one."""
+    and returns the attention output [T, nh, hd].  A token's position is its sequence's context length less one.
+    ``every_seq``: as in ``attention_decode``."""
     _dev(qkv, q_weight, k_weight, cos, sin, slots, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens)
     nkv, page, hd = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     _check_caches(k_cache, v_cache, nkv, hd, torch.bfloat16, "attention_decode_fused")
