@@ -59,6 +59,8 @@ _KERNEL_API = {
     "pa_attn_prefill_cut": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, I]),
     "pa_argmax_scratch": (I, [I, I]),
     "pa_argmax": (I, [P, P, P, P, I, I]),
+    "pa_argmax_static_capacity": (I, []),
+    "pa_argmax_static": (I, [P, P, P, I, I]),
     "pa_sample": (I, [P, P, P, P, P, P, P, I, I]),
     "pa_sample_wide_workspace": (c_long, [I, I]),
     "pa_logprobs": (I, [P, P, P, P, P, P, P, I, I, I, I]),

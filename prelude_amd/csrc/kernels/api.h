@@ -91,6 +91,16 @@ int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, const void*
 // scratch: pa_argmax_scratch(rows, vocab) floats (none for narrow rows).
 int pa_argmax_scratch(int rows, int vocab);
 int pa_argmax(void* stream, const float* logits, int* out, float* scratch, int rows, int vocab);
+// pa_argmax without a scratch argument and without any allocation, for callers that cannot allocate (code under
+// HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+// reference.  The candidates of wide rows go to an array inside the library, pa_argmax_static_capacity() floats
+// (65,536 = 256 KB) on every GPU the library runs on, held until the process ends; rows * ceil(vocab / 2048) * 2
+// must fit it (64 rows of 151,936 entries take 9,600), else the call is refused.  The first call on a GPU looks
+// up where that GPU's copy lies (make it before a capture begins).  Nothing in the array has to be cleared between
+// calls: what the second launch reads the first has written.  All calls on a GPU share the one array: calls
+// that overlap there (two streams, two threads) race, calls in order on one stream do not.
+int pa_argmax_static_capacity();
+int pa_argmax_static(void* stream, const float* logits, int* out, int rows, int vocab);
 
 // Per row: temperature < 1e-7 -> argmax; else a draw from softmax(logits / T) kept to the top_k largest
 // (0 = all) and to the shortest descending prefix of mass top_p (>= 1 = all), at the uniform number uniform[r] in [0, 1).

@@ -16,6 +16,8 @@
 #include "common.h"
 #include "api.h"
 
+#include <mutex>
+
 namespace pa {
 
 struct MaxIdx {
@@ -767,7 +769,6 @@ extern "C" int pa_sample(void* stream, const float* logits, const float* tempera
   return check_launch("sample");
 }
 
-// Floats of scratch pa_argmax needs for rows of this width (0: none).
 // Slices a row of `vocab` entries is cut into when `rows` rows are sampled by pa_sample_wide, and their length.
 static void wide_shape(int rows, int vocab, int* slices, int* slice_len) {
   int want = 1024 / rows;
@@ -848,15 +849,17 @@ extern "C" int pa_logprobs(void* stream, const float* logits, const int* ids, fl
   return check_launch("logprobs");
 }
 
+// Floats of scratch pa_argmax needs for rows of this width (0: none).
 extern "C" int pa_argmax_scratch(int rows, int vocab) {
   return vocab <= 8192 ? 0 : rows * ((vocab + 2047) / 2048) * 2;
 }
 
-extern "C" int pa_argmax(void* stream, const float* logits, int* out, float* scratch, int rows, int vocab) {
-  if (rows == 0) return 0;
-  PA_REQUIRE(rows > 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
+// The launches of an argmax: a workgroup a row for narrow rows; for wide ones a candidate per 2,048-entry chunk
+// into `scratch` (values, then indices), and a second launch that picks among them.  Every word of `scratch`
+// the second launch reads has been written by the first, so it need not start at any value.
+static int argmax_launch(hipStream_t st, const float* logits, int* out, float* scratch, int rows, int vocab) {
   if (vocab <= 8192) {
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, out, vocab);
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, st, logits, out, vocab);
     return check_launch("argmax");
   }
   PA_REQUIRE(scratch, "argmax: rows of %d need scratch", vocab);
@@ -864,9 +867,59 @@ extern "C" int pa_argmax(void* stream, const float* logits, int* out, float* scr
   PA_REQUIRE(chunks <= 65535, "argmax: %d columns exceed the grid", vocab);
   float* cand_v = scratch;
   int* cand_i = reinterpret_cast<int*>(scratch + (size_t)rows * chunks);
-  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(rows, chunks), dim3(256), 0, (hipStream_t)stream, logits, cand_v, cand_i,
-                     vocab, 2048);
+  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(rows, chunks), dim3(256), 0, st, logits, cand_v, cand_i, vocab, 2048);
   if (int rc = check_launch("argmax")) return rc;
-  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, (hipStream_t)stream, cand_v, cand_i, out, chunks);
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, st, cand_v, cand_i, out, chunks);
   return check_launch("argmax");
+}
+
+extern "C" int pa_argmax(void* stream, const float* logits, int* out, float* scratch, int rows, int vocab) {
+  if (rows == 0) return 0;
+  PA_REQUIRE(rows > 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
+  return argmax_launch((hipStream_t)stream, logits, out, scratch, rows, vocab);
+}
+
+// ---------------------------------------------------------------------------
+// pa_argmax for callers that cannot allocate: the candidates of wide rows go to an array that is part of the
+// library's image on every GPU.  In host code the array's name is only a stand-in for the symbol; the address
+// of a GPU's copy comes from hipGetSymbolAddress with that GPU current, once per GPU, and only that address is
+// ever handed to a kernel.
+// ---------------------------------------------------------------------------
+constexpr int kStaticArgmaxWords = 1 << 16;   // 256 KB a GPU
+static __device__ __align__(256) float scratch[kStaticArgmaxWords];
+
+constexpr int kStaticMaxDevices = 64;
+static float* g_static_scratch[kStaticMaxDevices];   // per GPU: where its copy of `scratch` lies
+static std::mutex g_static_lock;
+
+static int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return pa::fail("argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+  PA_REQUIRE(dev >= 0 && dev < kStaticMaxDevices, "argmax_static: device %d is beyond the %d this library keeps track of",
+             dev, kStaticMaxDevices);
+  std::lock_guard<std::mutex> hold(g_static_lock);
+  if (!g_static_scratch[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return pa::fail("argmax_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+    g_static_scratch[dev] = static_cast<float*>(p);
+  }
+  *out = g_static_scratch[dev];
+  return 0;
+}
+
+extern "C" int pa_argmax_static_capacity() { return kStaticArgmaxWords; }
+
+extern "C" int pa_argmax_static(void* stream, const float* logits, int* out, int rows, int vocab) {
+  if (rows == 0) return 0;
+  PA_REQUIRE(rows > 0 && vocab > 0, "argmax_static: bad sizes rows=%d vocab=%d", rows, vocab);
+  const long words = (long)rows * ((vocab + 2047) / 2048) * 2;
+  PA_REQUIRE(vocab <= 8192 || words <= kStaticArgmaxWords,
+             "argmax_static: %d rows of %d entries need %ld words of scratch, the built-in array holds %d "
+             "(use pa_argmax with a workspace of the caller's)", rows, vocab, words, kStaticArgmaxWords);
+  float* ptr = nullptr;
+  if (int rc = static_scratch(&ptr)) return rc;
+  return argmax_launch((hipStream_t)stream, logits, out, ptr, rows, vocab);
 }
