@@ -46,32 +46,11 @@ SHAPES = {"0.6b": QWEN3_06B, "4b": QWEN3_4B, "8b": QWEN3_8B, "32b": QWEN3_32B}
 
 
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
-    """The engine's own model with weights drawn on the device (no 8 GB file is written)."""
-    import torch
-    from prelude_amd import models  # noqa: F401
-    from prelude_amd.config import EngineConfig, resolve_architecture
+    """The engine in its random-weights mode: the product's own loader, tensors drawn on the device."""
+    from prelude_amd.config import EngineConfig
     from prelude_amd.engine import Engine
-    from prelude_amd.models.causal_lm import CausalLM
-    from prelude_amd.parts.base import MATRIX, NORM
-
-    arch = resolve_architecture(raw)
-    model = CausalLM(arch.build_spec(arch.parse_config(raw)))
-    device = torch.device("cuda:0")
-    tdtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
-    gen = torch.Generator(device=device).manual_seed(seed)
-    cache = {}
-
-    def fetch(name, req):
-        if name not in cache:
-            t = torch.randn(req.shape, generator=gen, device=device, dtype=torch.float32)
-            t = (1.0 + 0.01 * t) if req.kind == NORM else 0.02 * t
-            cache[name] = t.to(tdtype if req.kind == MATRIX else torch.float32).contiguous()
-        return cache[name]
-
-    model.load(fetch, tdtype, device)
-    cache.clear()
     cfg = EngineConfig(dtype=dtype, page_size=page_size, max_cache_tokens=cache_tokens, **cfg_overrides)
-    return Engine(model, cfg, raw)
+    return Engine.from_config(raw, cfg, seed=seed)
 
 
 def release_memory():

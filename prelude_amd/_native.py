@@ -39,6 +39,7 @@ _KERNEL_API = {
     "pa_num_compute_units": (I, []),
     "pa_embed_gather": (I, [P, I, P, P, P, I, I, I]),
     "pa_carry_tokens": (I, [P, P, P, P, P, I, I, I]),
+    "pa_zero_fresh_rows": (I, [P, P, c_long, P, P, I, I]),
     "pa_rmsnorm": (I, [P, I, P, P, P, P, P, I, I, F]),
     "pa_silu_mul": (I, [P, I, P, P, I, I]),
     "pa_gather_rows": (I, [P, I, P, P, P, I, I]),
@@ -93,7 +94,7 @@ _HOST_API = {
     "pa_cache_error": (c_char_p, [P]),
     "pa_sched_create": (P, [P, I, I, I, I, I, I, I]),
     "pa_sched_destroy": (None, [P]),
-    "pa_sched_add": (I, [P, c_longlong, I, I]),
+    "pa_sched_add": (I, [P, c_longlong, I, I, I, I]),
     "pa_sched_schedule": (I, [P, P, P, P, P, I]),
     "pa_sched_step_done": (I, [P]),
     "pa_sched_step_cancelled": (None, [P]),

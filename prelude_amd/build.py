@@ -26,7 +26,7 @@ GPU_ARCH = "gfx950"
 
 HIPCC_FLAGS = [
     f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
-    # packed 32-bit float instructions have given wrong results on this hardware pool
+    # no packed 32-bit float instructions: some of their forms have been seen to give wrong results on gfx950
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 HOST_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra"]

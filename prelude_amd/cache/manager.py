@@ -194,9 +194,22 @@ class StateLayerCache:
     """What a mixer with state of fixed size gets: per name a tensor [slots, *shape]."""
     tensors: Dict[str, torch.Tensor]
 
-    def zero_slots(self, slots: torch.Tensor) -> None:
+    def snapshot(self, state_slots: torch.Tensor) -> Dict[str, torch.Tensor]:
+        """Copies of the slots' rows (``state_slots`` int32 on the device, all >= 0)."""
+        idx = state_slots.to(torch.int64)
+        return {name: t.index_select(0, idx) for name, t in self.tensors.items()}
+
+    def restore(self, state_slots: torch.Tensor, saved: Dict[str, torch.Tensor]) -> None:
+        idx = state_slots.to(torch.int64)
+        for name, t in self.tensors.items():
+            t.index_copy_(0, idx, saved[name])
+
+    def zero_fresh(self, state_slots: torch.Tensor, fresh: torch.Tensor) -> None:
+        """Clears the slots of the step's sequences that start their request; both index arrays are the
+        step's own on the device, so a captured step can carry this."""
+        from ..ops import kernels as K
         for t in self.tensors.values():
-            t.index_fill_(0, slots, 0)
+            K.zero_fresh_rows(t, state_slots, fresh)
 
 
 def plan_groups(cache_specs: Sequence[object]) -> Tuple[List[KVCacheSpec], List[Optional[int]]]:
@@ -217,6 +230,43 @@ def plan_groups(cache_specs: Sequence[object]) -> Tuple[List[KVCacheSpec], List[
 def bytes_per_token(cache_specs: Sequence[object], dtype: torch.dtype) -> int:
     el = torch.empty((), dtype=dtype).element_size()
     return sum(2 * cs.num_kv_heads * cs.head_dim * el for cs in cache_specs if isinstance(cs, KVCacheSpec))
+
+
+def state_bytes_per_slot(cache_specs: Sequence[object]) -> int:
+    """Bytes one request's state of fixed size takes, over all cache slots that keep such state."""
+    total = 0
+    for cs in cache_specs:
+        if isinstance(cs, StateSpec):
+            for _name, shape, dt in cs.tensors:
+                n = 1
+                for d in shape:
+                    n *= int(d)
+                total += n * torch.empty((), dtype=dt).element_size()
+    return total
+
+
+def peak_pages(total: int, chunk: int, window: int, page_size: int) -> int:
+    """Pages of a group with this window that a request of ``total`` tokens holds at most when it is fed in
+    portions of at most ``chunk`` tokens (the rule of ``CacheManager::peak_pages``)."""
+    pages = lambda n: -(-n // page_size)
+    if window <= 0:
+        return pages(total)
+    return min(pages(total), pages(max(1, chunk) + window - 1) + 1)
+
+
+def pages_per_group(tokens: int, group_specs: Sequence[KVCacheSpec], page_size: int, max_requests: int,
+                    max_request_tokens: int, chunk: int) -> List[int]:
+    """Pages each group needs so that live requests can hold ``tokens`` tokens between them: a group that
+    sees every key holds them all; one with a window holds per request what the window and a portion span,
+    so it needs no more than that for as many requests as may run."""
+    full = max(1, -(-tokens // page_size))
+    out = []
+    for g in group_specs:
+        if g.window > 0:
+            out.append(max(1, min(full, max_requests * peak_pages(max_request_tokens, chunk, g.window, page_size))))
+        else:
+            out.append(full)
+    return out
 
 
 def allocate_storage(cache_specs: Sequence[object], of_slot: Sequence[Optional[int]], pages_per_group: Sequence[int],

@@ -8,7 +8,9 @@ Option names and meanings are the reference server's where it has them
 --cuda-graph/--no-cuda-graph).  The request fields the reference takes per
 HTTP request are options here: --max-tokens, --temperature, --top-p, --top-k,
 --seed, --stop-token-ids (crates/prelude-core/src/types.rs:63-96, :388-413).
---random-weights is ours: it needs only a config.json.
+--random-weights is ours: it needs only a config.json, and draws the tensors
+on the device; with --write-model DIR the drawn model is written out as a
+folder (config.json, model.safetensors) and loaded from there.
 """
 from __future__ import annotations
 
@@ -16,7 +18,6 @@ import argparse
 import json
 import os
 import sys
-import tempfile
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -28,6 +29,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--random-weights", action="store_true", help="draw weights from --seed instead of loading them")
     ap.add_argument("--weights-seed", type=int, default=0)
+    ap.add_argument("--write-model", metavar="DIR", help="with --random-weights: write the model folder (config.json, "
+                                                         "model.safetensors) there and load it from there")
     ap.add_argument("--max-running-requests", type=int, default=256)
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--long-prefill-token-threshold", type=int, default=0)
@@ -77,17 +80,6 @@ def main(argv=None) -> int:
     from .config.engine_config import EngineConfig
     from .llm import LLM
 
-    tmp = None
-    if args.random_weights:
-        from .weights.random_init import write_random_model
-        cfg_path = os.path.join(model, "config.json") if os.path.isdir(model) else model
-        with open(cfg_path, "r", encoding="utf-8") as f:
-            raw = json.load(f)
-        tmp = tempfile.TemporaryDirectory(prefix="prelude_amd_random_")
-        dt = torch.float32 if _dtype(args.dtype) == "float32" else torch.bfloat16
-        print(f"writing random weights (seed {args.weights_seed}) to {tmp.name}", file=sys.stderr, flush=True)
-        model = write_random_model(raw, tmp.name, seed=args.weights_seed, dtype=dt)
-
     cfg = EngineConfig(dtype=_dtype(args.dtype), device=args.device, page_size=args.page_size,
                        max_cache_tokens=args.max_cache_tokens, gpu_memory_utilization=args.gpu_memory_utilization,
                        max_num_batched_tokens=args.max_num_batched_tokens,
@@ -96,7 +88,19 @@ def main(argv=None) -> int:
                        decode_reservation_cap=args.decode_reservation_cap,
                        decode_priority_max_remaining_tokens=args.decode_priority_max_remaining_tokens,
                        hip_graph=args.hip_graph, overlap_steps=args.overlap_steps, weight_tiles=args.weight_tiles)
-    llm = LLM(model, config=cfg)
+    if args.random_weights:
+        cfg_path = os.path.join(model, "config.json") if os.path.isdir(model) else model
+        with open(cfg_path, "r", encoding="utf-8") as f:
+            raw = json.load(f)
+        if args.write_model:
+            from .weights.random_init import write_random_model
+            dt = torch.float32 if _dtype(args.dtype) == "float32" else torch.bfloat16
+            print(f"writing random weights (seed {args.weights_seed}) to {args.write_model}", file=sys.stderr, flush=True)
+            llm = LLM(write_random_model(raw, args.write_model, seed=args.weights_seed, dtype=dt), config=cfg)
+        else:
+            llm = LLM.from_config(raw, config=cfg, seed=args.weights_seed)
+    else:
+        llm = LLM(model, config=cfg)
     prompts = list(args.prompt)
     prompts += [[int(x) for x in s.split(",") if x.strip()] for s in args.prompt_ids]
     rng = np.random.default_rng(0 if args.seed is None else args.seed)
@@ -111,6 +115,8 @@ def main(argv=None) -> int:
     for o in outs:
         rec = {"request_id": o.request_id, "token_ids": o.token_ids, "finish_reason": o.finish_reason,
                "usage": o.usage, "metrics": {k: round(v, 3) for k, v in o.metrics.items()}}
+        if o.error is not None:
+            rec["error"] = o.error
         if o.text is not None:
             rec["text"] = o.text
         for key in ("token_logprobs", "top_logprobs", "prompt_logprobs"):
@@ -119,8 +125,6 @@ def main(argv=None) -> int:
         dec = max(o.metrics.get("decode_ms", 0.0), 1e-9)
         rec["decode_tok_per_s"] = round(max(len(o.token_ids) - 1, 0) / dec * 1e3, 1)
         print(json.dumps(rec), flush=True)
-    if tmp is not None:
-        tmp.cleanup()
     return 0
 
 

@@ -29,6 +29,7 @@ class EngineConfig:
     # decode steps replayed from HIP graphs
     hip_graph: bool = True
     hip_graph_max_bs: int = 64
+    hip_graph_cache_size: int = 32          # captured graphs kept (one per batch size and table width); the least recently used goes
     # a second copy of every bfloat16 weight matrix, in the tiles the few-row product streams fastest
     # (decode steps run about a tenth faster for twice the weight memory)
     weight_tiles: bool = True

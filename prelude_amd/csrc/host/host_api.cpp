@@ -98,8 +98,8 @@ void* pa_sched_create(void* cache, int max_num_batched_tokens, int long_prefill_
 void pa_sched_destroy(void* h) { delete static_cast<SchedHandle*>(h); }
 static Scheduler& S(void* h) { return static_cast<SchedHandle*>(h)->sched; }
 
-int pa_sched_add(void* h, long long id, int prompt_len, int max_new) {
-  return S(h).add_request(id, prompt_len, max_new) ? 0 : -1;
+int pa_sched_add(void* h, long long id, int prompt_len, int max_new, int atomic, int max_chunk) {
+  return S(h).add_request(id, prompt_len, max_new, atomic != 0, max_chunk) ? 0 : -1;
 }
 // Decides a step; writes up to cap entries and returns their number (or -1 if cap is too small).
 int pa_sched_schedule(void* h, long long* ids, int* starts, int* counts, int* samples, int cap) {

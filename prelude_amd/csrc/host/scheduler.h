@@ -55,6 +55,10 @@ struct Sequence {
   uint64_t arrival = 0;
   int preempt_count = 0;
   bool finished = false;
+  // A request whose mixers cannot continue a prompt from a cut (their state does not carry across portions):
+  // what it still has to feed is fed whole in one step or not at all.  Single decode tokens are not meant.
+  bool atomic = false;
+  int max_chunk = 0;  // cap on this request's portion (0 = none), beside the scheduler's own
   int remaining() const { return max_new - generated; }
 };
 
@@ -64,8 +68,9 @@ class Scheduler {
 
   const SchedulerConfig& config() const { return cfg_; }
   // False (with error()) if the id is in use, the prompt is empty, or the
-  // request could never fit the cache even alone.
-  bool add_request(int64_t id, int prompt_len, int max_new);
+  // request could never fit the cache (or, fed whole, the step's token budget) even alone.
+  // `atomic`: feed what is known whole or not at all; `max_chunk`: cap on its portions, 0 = none.
+  bool add_request(int64_t id, int prompt_len, int max_new, bool atomic = false, int max_chunk = 0);
   // Decides one step and reserves its pages.  Empty when nothing can run.
   const std::vector<StepEntry>& schedule();
   // The step just scheduled has run: what it fed is cached now.
@@ -94,6 +99,7 @@ class Scheduler {
  private:
   int chunk_for(const Sequence& s, int budget) const;
   int shrink_to_pages(const Sequence& s, int chunk) const;
+  int portion_for(const Sequence& s, int budget) const;
   bool tail_priority(const std::vector<StepEntry>& entries) const;
   void admit_waiting(int& budget);
   void preempt(size_t idx);

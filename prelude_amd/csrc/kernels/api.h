@@ -17,6 +17,10 @@ int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, 
 // ids[dst[i]] = sampled[src[i]] for i < n with src[i] >= 0 (token ids handed from one step to the next on the device).
 int pa_carry_tokens(void* stream, const int* sampled, const int* src, const int* dst, int* ids, int n, int sampled_rows,
                     int tokens);
+// Clears row slots[i] of data [num_rows, row_bytes] for every sequence i < nseq with fresh[i] != 0 and slots[i] >= 0:
+// per-request state of fixed size starts from zero, decided on the device (so a captured step can do it).
+int pa_zero_fresh_rows(void* stream, void* data, long row_bytes, const int* slots, const int* fresh, int nseq,
+                       int num_rows);
 // RMSNorm of x (+ residual, which then receives the sum) with a 32-bit weight;
 // with `rows`, output row r comes from input row rows[r] and the residual is left alone.
 int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out, const int* rows,

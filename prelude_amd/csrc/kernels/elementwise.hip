@@ -46,6 +46,18 @@ __global__ void carry_tokens_kernel(const int* __restrict__ sampled, const int* 
   ids[d] = sampled[s];
 }
 
+// ---- state of fixed size per request, started from zero ------------------
+// Row slots[i] of `data` (rows of `row_words` 32-bit words) is cleared for every sequence i of the step that
+// starts its request (fresh[i] != 0) and has a slot.  Grid (sequences, pieces of a row).
+__global__ void zero_fresh_rows_kernel(uint32_t* __restrict__ data, long row_words, const int* __restrict__ slots,
+                                       const int* __restrict__ fresh, int num_rows) {
+  const int i = blockIdx.x;
+  const int slot = slots[i];
+  if (!fresh[i] || slot < 0 || slot >= num_rows) return;
+  uint32_t* row = data + (size_t)slot * row_words;
+  for (long w = (long)blockIdx.y * blockDim.x + threadIdx.x; w < row_words; w += (long)gridDim.y * blockDim.x) row[w] = 0u;
+}
+
 // ---- RMSNorm, optionally fused with the residual add --------------------
 //   s = x (+ residual)                         in 32-bit
 //   residual <- round(s)                       (only when `residual` is given and `rows` is not)
@@ -221,6 +233,19 @@ extern "C" int pa_carry_tokens(void* stream, const int* sampled, const int* src,
   hipLaunchKernelGGL(carry_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, sampled, src, dst,
                      ids, n, sampled_rows, tokens);
   return check_launch("carry_tokens");
+}
+
+extern "C" int pa_zero_fresh_rows(void* stream, void* data, long row_bytes, const int* slots, const int* fresh, int nseq,
+                                  int num_rows) {
+  if (nseq == 0 || row_bytes == 0) return 0;
+  PA_REQUIRE(nseq > 0 && num_rows > 0 && row_bytes > 0 && row_bytes % 4 == 0,
+             "zero_fresh_rows: bad sizes sequences=%d rows=%d row_bytes=%ld (a multiple of 4)", nseq, num_rows, row_bytes);
+  PA_REQUIRE(data && slots && fresh, "zero_fresh_rows: a null operand");
+  const long words = row_bytes / 4;
+  const int pieces = (int)((words + 4095) / 4096 < 64 ? (words + 4095) / 4096 : 64);
+  hipLaunchKernelGGL(zero_fresh_rows_kernel, dim3(nseq, pieces), dim3(256), 0, (hipStream_t)stream, (uint32_t*)data, words,
+                     slots, fresh, num_rows);
+  return check_launch("zero_fresh_rows");
 }
 
 extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out,

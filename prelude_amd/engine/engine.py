@@ -18,7 +18,8 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache.manager import (CacheError, OutOfPages, PageTables, allocate_storage, bytes_per_token, plan_groups)
+from ..cache.manager import (CacheError, OutOfPages, PageTables, allocate_storage, bytes_per_token, pages_per_group,
+                             plan_groups, state_bytes_per_slot)
 from ..config.engine_config import EngineConfig
 from ..config.model_config import read_config_json
 from ..config.registry import resolve_architecture
@@ -81,21 +82,37 @@ class Engine:
         self.page_size = int(config.page_size)
         specs = [c.spec for c in model.cache_slots]
         self.group_specs, self._group_of_slot = plan_groups(specs)
-        tokens = self._decide_cache_tokens(specs)
-        pages = max(1, -(-tokens // self.page_size))
-        self.cache_tokens = pages * self.page_size
-        state_slots = config.max_state_slots if model.needs_state else 0
-        self.tables = PageTables(self.page_size, [(pages, g.window) for g in self.group_specs], state_slots)
-        self.caches = allocate_storage(specs, self._group_of_slot, [pages] * len(self.group_specs), self.page_size,
-                                       state_slots, self.dtype, self.device)
         self._staging = _Staging()
         self._live: Dict[int, int] = {}   # request id -> tokens fed so far
-        # decode steps as HIP graphs: only for models whose layers keep nothing but pages (a mixer with
-        # state of its own may run host code per step), and only in the serving type
         self._graphs = None
+        state_slots = config.max_state_slots if model.needs_state else 0
+        self.memory_plan: Dict[str, int] = {}
+        tokens = self._decide_cache_tokens(specs, state_slots)
+        pages = self._pages_for(tokens)
+        self.cache_tokens = max(pages) * self.page_size if pages else self.page_size
+        self._set_cache(pages, state_slots)
+        # decode steps as HIP graphs, in the serving type, for models none of whose parts says it cannot be replayed
         if config.hip_graph and model.graph_safe and self.dtype == torch.bfloat16:
             from .graph import DecodeGraphs
-            self._graphs = DecodeGraphs(self, config.hip_graph_max_bs)
+            self._graphs = DecodeGraphs(self, config.hip_graph_max_bs, config.hip_graph_cache_size)
+
+    def _chunk_cap(self) -> int:
+        """The most tokens of one request a step may bring."""
+        cap = int(self.config.max_num_batched_tokens)
+        if self.config.long_prefill_token_threshold > 0:
+            cap = min(cap, int(self.config.long_prefill_token_threshold))
+        return max(1, cap)
+
+    def _pages_for(self, tokens: int) -> List[int]:
+        return pages_per_group(tokens, self.group_specs, self.page_size, max(1, int(self.config.max_running_requests)),
+                               self.max_positions, self._chunk_cap())
+
+    def _set_cache(self, pages: List[int], state_slots: int) -> None:
+        specs = [c.spec for c in self.model.cache_slots]
+        self.tables = PageTables(self.page_size, [(n, g.window) for n, g in zip(pages, self.group_specs)], state_slots)
+        self.caches = allocate_storage(specs, self._group_of_slot, pages, self.page_size, state_slots, self.dtype,
+                                       self.device)
+        self.pages_per_group = list(pages)
 
     # ---- construction -------------------------------------------------------
     @classmethod
@@ -115,20 +132,101 @@ class Engine:
         load_into(model, model_dir, config.torch_dtype(), device)
         return cls(model, config, raw)
 
-    def _decide_cache_tokens(self, specs) -> int:
+    @classmethod
+    def from_config(cls, raw_config: dict, config: Optional[EngineConfig] = None, seed: int = 0, std: float = 0.02,
+                    norm_std: float = 0.01) -> "Engine":
+        """The random-weights mode without a folder: the architecture ``raw_config`` (a config.json's content)
+        names, with every tensor drawn on the device from (seed, tensor name)."""
+        from .. import models  # noqa: F401
+        from ..weights.random_init import load_random
+        config = config or EngineConfig()
+        if not torch.cuda.is_available():
+            raise RuntimeError("prelude_amd needs a GPU: torch sees no HIP device, and there is no CPU path")
+        arch = resolve_architecture(raw_config)
+        model = CausalLM(arch.build_spec(arch.parse_config(raw_config)))
+        device = torch.device(config.device)
+        torch.cuda.set_device(device)
+        from ..ops import kernels as K
+        K.set_weight_tiles(config.weight_tiles)
+        load_random(model, config.torch_dtype(), device, seed, std, norm_std)
+        return cls(model, config, dict(raw_config))
+
+    def _cache_bytes(self, tokens: int, specs) -> int:
+        """Bytes the pages take when live requests may hold ``tokens`` tokens (windowed groups are bounded)."""
+        el = torch.empty((), dtype=self.dtype).element_size()
+        pages = self._pages_for(tokens)
+        total = 0
+        for cs, g in zip(specs, self._group_of_slot):
+            if g is not None:
+                total += pages[g] * self.page_size * 2 * cs.num_kv_heads * cs.head_dim * el
+        return total
+
+    def _decide_cache_tokens(self, specs, state_slots: int) -> int:
+        """How many tokens the page pools hold.  Given (``max_cache_tokens``), or what the device has left after
+        the weights, one step's activations as measured by running one, and stated reserves -- the reference's
+        rule, crates/prelude-core/src/scheduler/components/cache/manager.rs:240-280 with the dummy forward of
+        crates/prelude-core/src/engine/loading.rs:283-368:
+
+            pages = total * gpu_memory_utilization - in use (weights) - peak of a step - reserves
+
+        The reserves are what is allocated only later: the library product's workspace, the state slots, and for
+        captured decode steps a logits tensor per kept graph plus their shared activation pool."""
         if self.config.max_cache_tokens is not None:
             return max(int(self.config.max_cache_tokens), self.page_size)
         per_token = bytes_per_token(specs, self.dtype)
         if per_token == 0:
             return self.page_size
-        free, _total = torch.cuda.mem_get_info(self.device)
-        # room for one step's activations: a dozen hidden-sized rows, the widest projection, float32 logits rows
-        spec = self.model.spec
-        el = torch.empty((), dtype=self.dtype).element_size()
-        act = self.config.max_num_batched_tokens * spec.hidden_size * el * 48 + 256 * spec.vocab_size * 4 * 2
-        usable = int(free * self.config.gpu_memory_utilization) - act
-        tokens = max(usable // per_token, 16 * self.page_size)
-        return int(min(tokens, self.max_positions * max(1, self.config.max_running_requests)))
+        from ..ops import kernels as K
+        peak = self._probe_step_bytes(specs, state_slots)
+        torch.cuda.synchronize(self.device)
+        torch.cuda.empty_cache()
+        free, total = torch.cuda.mem_get_info(self.device)
+        in_use = total - free
+        reserve_state = state_slots * state_bytes_per_slot(specs)
+        reserve_library = 0 if self.dtype != torch.bfloat16 else K.library_workspace_reserve(self.device)
+        reserve_graphs = 0
+        if self.config.hip_graph and self.model.graph_safe and self.dtype == torch.bfloat16:
+            logits = int(self.config.hip_graph_max_bs) * self.vocab_size * 4
+            reserve_graphs = int(self.config.hip_graph_cache_size) * logits + (256 << 20)
+        budget = int(total * self.config.gpu_memory_utilization) - in_use - peak - reserve_state - reserve_library \
+            - reserve_graphs
+        self.memory_plan = dict(total=total, in_use=in_use, step_peak=peak, state=reserve_state,
+                                library_workspace=reserve_library, graphs=reserve_graphs, cache=max(budget, 0))
+        ceiling = self.max_positions * max(1, int(self.config.max_running_requests))
+        floor = 16 * self.page_size
+        if budget <= self._cache_bytes(floor, specs):
+            return floor
+        lo, hi = floor, ceiling          # the most tokens whose pages fit the budget (the cost grows with the tokens)
+        if self._cache_bytes(hi, specs) <= budget:
+            return hi
+        while hi - lo > self.page_size:
+            mid = (lo + hi) // 2
+            if self._cache_bytes(mid, specs) <= budget:
+                lo = mid
+            else:
+                hi = mid
+        return lo // self.page_size * self.page_size
+
+    def _probe_step_bytes(self, specs, state_slots: int) -> int:
+        """Runs one step of as many tokens as a step may bring (one request, its last rows wanted) over a cache
+        just large enough for it, and returns the peak of device memory the step took beyond what was
+        allocated before it; the cache is given back."""
+        n = max(1, min(self._chunk_cap(), self.max_positions))
+        rows = min(n, max(512, int(self.config.max_running_requests)))
+        pages = [max(1, -(-n // self.page_size))] * len(self.group_specs)
+        self._set_cache(pages, 1 if state_slots else 0)
+        torch.cuda.synchronize(self.device)
+        before = torch.cuda.memory_allocated(self.device)
+        torch.cuda.reset_peak_memory_stats(self.device)
+        try:
+            self.step([StepEntry(-1, [0] * n, list(range(n - rows, n)))])
+            torch.cuda.synchronize(self.device)
+            peak = torch.cuda.max_memory_allocated(self.device) - before
+        finally:
+            self.release(-1)
+            self.tables = None
+            self.caches = None
+        return max(int(peak), 0)
 
     # ---- requests ---------------------------------------------------------------
     def has(self, rid: int) -> bool:
@@ -190,6 +288,10 @@ class Engine:
         if not entries:
             raise StepError("a step needs at least one entry")
         self._validate_carried(entries, carried)
+        total = sum(len(e.tokens) for e in entries)
+        if total > self.config.max_num_batched_tokens:
+            raise StepError(f"the step brings {total} tokens; max_num_batched_tokens is "
+                            f"{self.config.max_num_batched_tokens} (pools and activation memory are sized for that)")
         seen = set()
         for e in entries:
             if e.id in seen:
@@ -321,11 +423,14 @@ class Engine:
         if self._graphs is not None and self._graphs.eligible(entries):
             return self._graphs.run(entries, starts, carried)
         batch = self.build_batch(entries, starts, carried=carried)
-        if self.model.needs_state:
-            fresh = [s for s, f in zip(batch.state_slots_host, batch.fresh_host) if f and s >= 0]
-            if fresh:
-                idx = torch.tensor(fresh, dtype=torch.int64, device=self.device)
-                for c in self.caches:
-                    if hasattr(c, "zero_slots"):
-                        c.zero_slots(idx)
+        return self.forward(batch, any(batch.fresh_host))
+
+    def forward(self, batch: StepBatch, maybe_fresh: bool = True) -> torch.Tensor:
+        """The model over a built batch.  State of fixed size starts from zero for the sequences that start their
+        request, decided on the device from the step's own arrays (``maybe_fresh`` false spares the launches
+        when the host knows that none does; a captured step always carries them)."""
+        if self.model.needs_state and maybe_fresh:
+            for c in self.caches:
+                if hasattr(c, "zero_fresh"):
+                    c.zero_fresh(batch.state_slots, batch.fresh)
         return self.model.forward(batch, self.caches)

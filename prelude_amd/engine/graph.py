@@ -11,7 +11,11 @@ The reference does the same with CUDA graphs, one per batch size up to 32,
 with fixed input buffers refreshed before each replay
 (crates/prelude-cuda/src/cuda_graph.rs:45-332, buffers.rs:11-30).  Here the
 block-table width is part of the key (rounded up, so few graphs cover all
-context lengths) and graphs are captured when first needed.
+context lengths) and graphs are captured when first needed.  At most
+``cache_size`` graphs are kept: each owns its logits tensor [B, vocab], so
+the number is part of the memory the engine sets aside; when one more is
+needed the least recently used is dropped (after the device has finished
+with it) and captured again if its shape comes back.
 
 A graph may be launched again while its previous launch still runs (the host
 prepares one step ahead): launches on one stream run in order, and the index
@@ -24,8 +28,9 @@ hold; workgroups beyond a sequence's length leave at once).
 """
 from __future__ import annotations
 
+import collections
 import dataclasses
-from typing import Dict, Sequence, Tuple
+from typing import Sequence, Tuple
 
 import torch
 
@@ -41,13 +46,15 @@ class _Captured:
 class DecodeGraphs:
     STRIDE_STEP_TOKENS = 1024   # table widths are rounded up to this many tokens
 
-    def __init__(self, engine, max_batch: int):
+    def __init__(self, engine, max_batch: int, cache_size: int = 32):
         self.engine = engine
         self.max_batch = int(max_batch)
-        self._graphs: Dict[Tuple[int, int], _Captured] = {}
+        self.cache_size = max(1, int(cache_size))
+        self._graphs: "collections.OrderedDict[Tuple[int, int], _Captured]" = collections.OrderedDict()
         self._pool = None
         self.replays = 0
         self.captures = 0
+        self.evictions = 0
 
     def eligible(self, entries: Sequence) -> bool:
         if not 1 <= len(entries) <= self.max_batch:
@@ -70,9 +77,15 @@ class DecodeGraphs:
         key = (n, stride)
         cap = self._graphs.get(key)
         if cap is None:
+            while len(self._graphs) >= self.cache_size:
+                # the device may still be replaying it (the host runs a step ahead): wait, then let it go
+                torch.cuda.synchronize(eng.device)
+                self._graphs.popitem(last=False)
+                self.evictions += 1
             cap = self._capture(entries, starts, stride, carried)
             self._graphs[key] = cap
         else:
+            self._graphs.move_to_end(key)
             eng.build_batch(entries, starts, stride=stride, device_buffer=cap.buffer, carried=carried)
         cap.graph.replay()
         self.replays += 1
@@ -85,17 +98,22 @@ class DecodeGraphs:
         buffer = torch.empty(size, dtype=torch.int32, device=eng.device)
         batch = eng.build_batch(entries, starts, stride=stride, device_buffer=buffer, carried=carried)
         # once outside a capture, on a side stream, so that whatever libraries set up lazily exists already;
-        # it writes the same keys and values the replay will write
+        # it writes the same keys and values the replay will write.  State of fixed size is not written twice to
+        # the same effect (a recurrence would advance two steps): the slots' rows are put back afterwards.
+        stateful = [c for c in eng.caches if hasattr(c, "snapshot")] if eng.model.needs_state else []
+        saved = [c.snapshot(batch.state_slots) for c in stateful]
         side = torch.cuda.Stream(device=eng.device)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            eng.model.forward(batch, eng.caches)
+            eng.forward(batch)
         torch.cuda.current_stream().wait_stream(side)
+        for c, rows in zip(stateful, saved):
+            c.restore(batch.state_slots, rows)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         if self._pool is None:
             self._pool = torch.cuda.graph_pool_handle()
         with torch.cuda.graph(graph, pool=self._pool):
-            logits = eng.model.forward(batch, eng.caches)
+            logits = eng.forward(batch)
         self.captures += 1
         return _Captured(graph, buffer, logits, stride)

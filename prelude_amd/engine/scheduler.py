@@ -65,8 +65,10 @@ class Scheduler:
     def _err(self) -> str:
         return self._lib.pa_sched_error(self._h).decode()
 
-    def add_request(self, rid: int, prompt_len: int, max_new: int) -> None:
-        if self._lib.pa_sched_add(self._h, rid, prompt_len, max_new) != 0:
+    def add_request(self, rid: int, prompt_len: int, max_new: int, atomic: bool = False, max_chunk: int = 0) -> None:
+        """``atomic``: what the request has to feed is fed whole in one step or not at all (for mixers that
+        cannot continue a prompt from a cut); ``max_chunk``: a cap on its portions, 0 = none."""
+        if self._lib.pa_sched_add(self._h, rid, prompt_len, max_new, int(bool(atomic)), int(max_chunk)) != 0:
             raise SchedulerError(self._err())
 
     def schedule(self) -> List[Portion]:

@@ -5,8 +5,9 @@ Modelled on the reference's ``InferenceEngine::generate`` / ``generate_batch``
 (crates/prelude-core/src/engine/mod.rs:75-132) and its request and result
 types (crates/prelude-core/src/types.rs:388-455): per request a prompt (text
 or token ids), ``max_tokens``, sampling options, stop token ids and a seed;
-per result the generated ids, why it finished (``stop`` | ``length`` | ``eos``),
-token counts and the four timings ``ttft_ms, prefill_ms, decode_ms, total_ms``.
+per result the generated ids, why it finished (``stop`` | ``length`` | ``eos`` |
+``cancelled``, crates/prelude-core/src/scheduler/state.rs:35-52; ``error`` for a
+request whose step failed), token counts and the four timings ``ttft_ms, prefill_ms, decode_ms, total_ms``.
 The loop is the reference's ``ar_loop`` (crates/prelude-core/src/engine/run/ar.rs:180-396):
 schedule, build the step, run it, sample, finish.  With ``overlap_steps`` the
 host runs one step ahead of the device: step N+1 is scheduled and launched
@@ -27,11 +28,12 @@ import torch
 
 from .config.engine_config import EngineConfig
 from .engine.engine import Engine, StepEntry
-from .engine.scheduler import Scheduler
+from .engine.scheduler import Scheduler, SchedulerError
 from .ops import kernels as K
 from .sampling.sampler import RequestSampler, SamplingParams, sample_rows_device
 
 DEFAULT_MAX_TOKENS = 4096   # crates/prelude-server/src/routes/generation_common.rs:9
+PROMPT_LOGPROBS_CHUNK = 512
 
 Prompt = Union[str, Sequence[int]]
 
@@ -41,8 +43,9 @@ class GenerationResult:
     request_id: int
     prompt_token_ids: List[int]
     token_ids: List[int]
-    finish_reason: str                      # "stop" | "length" | "eos"
+    finish_reason: str                      # "stop" | "length" | "eos" | "cancelled" | "error"
     text: Optional[str] = None              # when a tokenizer is at hand
+    error: Optional[str] = None             # with "error": what failed in the step that ended the request
     metrics: Dict[str, float] = dataclasses.field(default_factory=dict)
     preemptions: int = 0
     # asked for with ``logprobs`` / ``prompt_logprobs`` (crates/prelude-core/src/types.rs:388-455):
@@ -76,6 +79,7 @@ class _Live:
     pending_row: Optional[int] = None    # the last of ``tokens`` is still on the device: its row among the step's samples
     done: bool = False
     preemptions: int = 0
+    error: Optional[str] = None
 
 
 @dataclasses.dataclass
@@ -105,6 +109,19 @@ class LLM:
             setattr(cfg, k, v)
         self.model_dir = model
         self._attach(Engine.from_model_dir(model, cfg))
+
+    @classmethod
+    def from_config(cls, raw_config: dict, dtype: str = "bfloat16", config: Optional[EngineConfig] = None,
+                    seed: int = 0, std: float = 0.02, norm_std: float = 0.01, **overrides) -> "LLM":
+        """The random-weights mode: the model ``raw_config`` (a config.json's content) describes, every tensor
+        drawn on the device from (seed, tensor name); no folder is read or written."""
+        cfg = config or EngineConfig()
+        cfg.dtype = dtype if config is None else cfg.dtype
+        for k, v in overrides.items():
+            if not hasattr(cfg, k):
+                raise TypeError(f"unknown engine option {k!r}")
+            setattr(cfg, k, v)
+        return cls.from_engine(Engine.from_config(raw_config, cfg, seed, std, norm_std))
 
     @classmethod
     def from_engine(cls, engine: Engine, model_dir: Optional[str] = None) -> "LLM":
@@ -244,7 +261,10 @@ class Session:
         sp = sampling if sampling is not None else SamplingParams()
         rid = llm._next_id
         llm._next_id += 1
-        self.scheduler.add_request(rid, len(ids), max_new)
+        # every prompt position's logits are asked for with prompt_logprobs: the head then runs over portions of
+        # at most PROMPT_LOGPROBS_CHUNK rows, as in crates/prelude-core/src/engine/model_runner/paged_mixed.rs:172-270
+        self.scheduler.add_request(rid, len(ids), max_new, atomic=self.engine.model.atomic_prefill,
+                                   max_chunk=PROMPT_LOGPROBS_CHUNK if prompt_logprobs else 0)
         index = self._added
         self._added += 1
         self._live[rid] = _Live(rid, index, ids, list(ids), max_new, RequestSampler(sp), stop_ids, time.perf_counter(),
@@ -261,15 +281,60 @@ class Session:
             self.scheduler.finish(rid)
         self._live.clear()
 
+    def cancel(self, index: int) -> Optional[GenerationResult]:
+        """Ends one request now, whatever it was doing (the reference's ``abort_request``,
+        crates/prelude-core/src/engine/run/ar.rs:436-446, crates/prelude-core/src/scheduler/state.rs:357-470):
+        what it holds goes back and its result, with the tokens generated so far and the reason ``cancelled``,
+        is returned.  The other requests go on.  ``None`` if no live request has this index."""
+        r = next((x for x in self._live.values() if x.index == index), None)
+        if r is None:
+            return None
+        if self._in_flight is not None and any(x is r for x in self._in_flight.drawn):
+            # a launched step holds a token of it that the host has not read: read it first, so that the
+            # result has every token that was generated (this may end the request by itself)
+            self._resolve(self._in_flight, self._live)
+            self._in_flight = None
+            for i, (idx, res) in enumerate(self._ended):
+                if idx == index:
+                    del self._ended[i]
+                    return res
+        return self._end_now(r, "cancelled")
+
+    def _end_now(self, r: _Live, reason: str, error: Optional[str] = None) -> GenerationResult:
+        """Takes a live request out of the scheduler and the session and makes its result."""
+        if r.rid in self._live:
+            r.preemptions = self.scheduler.info(r.rid).preempt_count
+            self.scheduler.finish(r.rid)
+            del self._live[r.rid]
+        while r.tokens and r.tokens[-1] is None:      # stand-ins of tokens that were never read
+            r.tokens.pop()
+        r.finish_reason, r.error, r.done = reason, error, True
+        return self._result(r, time.perf_counter(), r.preemptions)
+
+    def _fail(self, rids: Sequence[int], error: BaseException) -> None:
+        """A step could not be run: every request of it ends with the reason ``error`` and gives back what it
+        holds (the reference's ``fail_step``, crates/prelude-core/src/engine/run/ar.rs:1647-1665); the others go on."""
+        if self._in_flight is not None:     # what the step before sampled is still wanted
+            self._resolve(self._in_flight, self._live)
+            self._in_flight = None
+        msg = f"{type(error).__name__}: {error}"
+        for rid in rids:
+            r = self._live.get(rid)
+            if r is not None:
+                self._ended.append((r.index, self._end_now(r, "error", msg)))
+
     def step(self) -> List[tuple]:
         """Launches the next step (if there is anything to run) and reads the one before; returns
-        ``[(index, GenerationResult)]`` for the requests that ended."""
+        ``[(index, GenerationResult)]`` for the requests that ended.  A step that cannot be run ends its own
+        requests with ``finish_reason == "error"`` (``error`` says why); nothing is raised for it."""
         overlap = bool(self.llm.config.overlap_steps)
+        ended_before = len(self._ended)
         launched = self._launch(self._live, self._in_flight) if self._live else None
         if launched is None and self._in_flight is None:
-            if self._live:
+            if self._live and len(self._ended) == ended_before:
                 raise RuntimeError("the scheduler has requests but nothing to run")
-            return []
+            ended, self._ended = self._ended, []
+            return ended
         if not overlap and launched is not None:
             self._in_flight, launched = launched, None
         if self._in_flight is not None:
@@ -288,7 +353,12 @@ class Session:
 
     def _launch(self, live: Dict[int, _Live], previous: Optional[_InFlight]) -> Optional[_InFlight]:
         """Schedules and launches one step; the scheduler is told at once that its tokens exist."""
-        portions = self.scheduler.schedule()
+        try:
+            portions = self.scheduler.schedule()
+        except SchedulerError as e:
+            # no running request can move and none can be evicted: those that run end here, the queue goes on
+            self._fail([rid for rid in list(live) if self.scheduler.info(rid).running], e)
+            return None
         if not portions:
             return None
         entries = []
@@ -321,9 +391,10 @@ class Session:
         try:
             logits = self.engine.run(entries, [p.start for p in portions],
                                      previous.sampled if previous is not None else None)
-        except Exception:
+        except Exception as e:
             self.scheduler.step_cancelled()
-            raise
+            self._fail([p.id for p in portions], e)
+            return None
         self.scheduler.step_done()
         self.llm.steps += 1
         drawn = [live[p.id] for p in portions if p.samples]
@@ -426,7 +497,8 @@ class Session:
                 cut = text.find(s)
                 if cut >= 0:
                     text = text[:cut]
-        res = GenerationResult(r.rid, list(r.prompt), out, r.finish_reason or "length", text, metrics, preemptions)
+        res = GenerationResult(r.rid, list(r.prompt), out, r.finish_reason or "length", text, r.error, metrics,
+                               preemptions)
         if r.logprobs is not None:
             res.token_logprobs = r.token_lps[:len(out)]
             if r.logprobs > 0:

@@ -113,9 +113,13 @@ class CausalLM:
 
     @property
     def graph_safe(self) -> bool:
-        """Whether a decode step may be captured once and replayed: no state slots and no part that says no."""
-        return not self.needs_state and all(p.GRAPH_SAFE for p, _ in self._parts) \
-            and all(b.GRAPH_SAFE for b in self.blocks)
+        """Whether a decode step may be captured once and replayed: no part says no."""
+        return all(p.GRAPH_SAFE for p, _ in self._parts) and all(b.GRAPH_SAFE for b in self.blocks)
+
+    @property
+    def atomic_prefill(self) -> bool:
+        """Whether some mixer cannot continue a prompt from a cut: requests are then fed whole or not at all."""
+        return any(getattr(p, "ATOMIC_PREFILL", False) for p, _ in self._parts)
 
     # ---- forward ------------------------------------------------------------
     def forward(self, step, caches) -> torch.Tensor:

@@ -16,8 +16,8 @@ from .spec import LayerSpec, ModelSpec, PartSpec, RunSpec
 def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
     if cfg.hidden_act != "silu":
         raise ConfigError(f"failed to parse Qwen3 config: `hidden_act` {cfg.hidden_act!r} is not supported (silu)")
-    if cfg.head_dim % 16 or cfg.head_dim > 256:
-        raise ConfigError(f"failed to parse Qwen3 config: `head_dim` {cfg.head_dim} must be a multiple of 16, at most 256")
+    if cfg.head_dim > 256:
+        raise ConfigError(f"failed to parse Qwen3 config: `head_dim` {cfg.head_dim} is more than the 256 the kernels take")
     h, hd = cfg.hidden_size, cfg.head_dim
     layers = []
     for i in range(cfg.num_hidden_layers):
@@ -47,7 +47,10 @@ def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
         head=PartSpec("linear_head", dict(vocab_size=cfg.vocab_size, hidden_size=h),
                       {"weight": embed_name if cfg.tie_word_embeddings else "lm_head.weight"}),
         positions={"rope": PartSpec("rope", dict(rotary_dim=hd, max_positions=cfg.max_position_embeddings,
-                                                 theta=cfg.rope_theta))})
+                                                 theta=cfg.rope_theta))},
+        # a tied checkpoint may still carry the head it does not use (the reference never reads it,
+        # crates/prelude-core/src/models/qwen3.rs:637-643), and old exports the rotary frequencies as a buffer
+        ignored_tensors=("*.rotary_emb.inv_freq",) + (("lm_head.weight",) if cfg.tie_word_embeddings else ()))
 
 
 QWEN3 = register_architecture(Architecture(

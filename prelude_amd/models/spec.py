@@ -50,6 +50,9 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     positions: Dict[str, PartSpec] = dataclasses.field(default_factory=dict)  # shared position encodings by name
+    # checkpoint names (shell patterns) that files of this architecture may hold and the model does not read:
+    # they are passed over; any other tensor nothing asks for is an error
+    ignored_tensors: Tuple[str, ...] = ()
 
     def validate(self) -> None:
         if not self.order:

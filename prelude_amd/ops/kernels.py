@@ -83,6 +83,21 @@ def carry_tokens(sampled: torch.Tensor, src: torch.Tensor, dst: torch.Tensor, id
                                     sampled.numel(), ids.numel()))
 
 
+def zero_fresh_rows(data: torch.Tensor, slots: torch.Tensor, fresh: torch.Tensor) -> None:
+    """data[slots[i]] = 0 for every sequence i with fresh[i] != 0 and slots[i] >= 0; data [rows, ...] of a
+    4-byte-multiple row size, slots / fresh int32 [B] on the device."""
+    _dev(data, slots, fresh)
+    _i32(slots, "slots")
+    _i32(fresh, "fresh")
+    if data.dim() < 1 or slots.shape != fresh.shape or slots.dim() != 1:
+        raise NativeError(f"zero_fresh_rows: data {tuple(data.shape)} / slots {tuple(slots.shape)} / fresh {tuple(fresh.shape)}")
+    if data.shape[0] == 0 or slots.shape[0] == 0:
+        return
+    row_bytes = data[0].numel() * data.element_size()
+    check(kernels().pa_zero_fresh_rows(_stream(), _ptr(data), row_bytes, _ptr(slots), _ptr(fresh), slots.shape[0],
+                                       data.shape[0]))
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None,
             rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """RMSNorm over the last axis of x [T, H] with a float32 weight [H].
@@ -315,6 +330,11 @@ LIBRARY_WORKSPACE_BYTES = 76 << 20   # what the library's stream-K kernels may u
 _library_workspaces: dict = {}
 
 
+def library_workspace_reserve(device) -> int:
+    """Bytes the library product will still allocate on ``device`` at its first call (0 once it has)."""
+    return 0 if torch.device(device) in _library_workspaces else LIBRARY_WORKSPACE_BYTES
+
+
 def gemm_library(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """y = x W^T in bfloat16 with 32-bit accumulation by hipBLASLt, called directly (its plan is kept per shape:
     a call through ``torch.matmul`` costs the host some 20 us, this one 14)."""
@@ -349,6 +369,10 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
+    if k % 8:
+        # rows that are no multiple of 16 bytes: neither the streaming kernel's loads nor the library's fast
+        # kernels take them; the plain product does (bfloat16 in, 32-bit sums), and only odd toy sizes come here
+        return gemm_plain(x, w, bias, out_dtype)
     y = gemm_library(x, w)
     if bias is not None:
         add_bias_(y, bias)

@@ -27,8 +27,10 @@ class GQAAttention(Mixer):
                  rotary_dim: Optional[int] = None, scale: Optional[float] = None):
         if num_heads % num_kv_heads:
             raise PartError(f"gqa_attention: {num_heads} heads are not a multiple of {num_kv_heads} KV heads")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
-            raise PartError(f"gqa_attention: head_dim {head_dim} is not a multiple of 16 in 16..256")
+        # what the kernels take: the matrix-core attention has head sizes of its own (others go to the generic
+        # kernel), the generic kernel and the norm + rotation kernel any size up to 256
+        if not 1 <= head_dim <= 256:
+            raise PartError(f"gqa_attention: head_dim {head_dim} is outside 1..256")
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
         self.norm_eps, self.qk_norm, self.bias, self.window = float(norm_eps), bool(qk_norm), bool(bias), int(window or 0)
         self.position = position

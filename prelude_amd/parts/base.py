@@ -57,9 +57,12 @@ class StateSpec:
 class Part:
     """Base of all parts.  Subclasses take their sizes and constants as keyword parameters."""
 
-    # False for a part whose ``forward`` reads device results on the host or launches work that depends on
-    # them (rows routed by value, say): decode steps of a model with such a part are not replayed from HIP
-    # graphs.  A part that keeps state per request need not say so; its model is never captured.
+    # False for a part whose ``forward``, in a step of single tokens, reads device results on the host, launches
+    # work that depends on them (rows routed by value, say) or works from the step's host-side lists
+    # (``StepBatch.q_lens``, ``state_slots_host``): decode steps of a model with such a part are not replayed
+    # from HIP graphs.  A part that keeps state per request can be replayed if in such steps it reaches its
+    # slots through the device array ``StepBatch.state_slots`` alone; the slots of starting requests are
+    # cleared on the device before it runs.
     GRAPH_SAFE = True
 
     def tensors(self) -> Dict[str, TensorReq]:
@@ -74,6 +77,10 @@ class Part:
 
 
 class Mixer(Part):
+    # True for a mixer that cannot pick a prompt up again where a step left it (nothing carries its state across
+    # a cut): the scheduler then feeds a request's known tokens whole in one step or not at all.
+    ATOMIC_PREFILL = False
+
     def cache_spec(self):
         return None
 

@@ -16,14 +16,29 @@ from .engine.engine import Engine, StepEntry
 
 
 class TraceRunner:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: Optional[int] = None,
-                 device: str = "cuda:0"):
+    def __init__(self, model_dir: Optional[str], dtype: str, max_tokens: Optional[int] = None,
+                 page_size: Optional[int] = None, device: str = "cuda:0", num_pages: Optional[int] = None,
+                 random_config: Optional[dict] = None, weights_seed: int = 0):
+        """``model_dir``: a folder with config.json and safetensors; or ``random_config`` (a config.json's
+        content): that model with weights drawn on the device from ``weights_seed``.  The pool holds
+        ``max_tokens`` tokens, or ``num_pages`` pages of ``page_size`` tokens: exactly what live requests may
+        hold, so pages are used again."""
         cfg = EngineConfig(dtype=dtype, device=device)
         if page_size is not None:
-            cfg.page_size = page_size
-        # the pool holds exactly what live requests may hold, so pages are used again
-        cfg.max_cache_tokens = max(int(max_tokens), cfg.page_size)
-        self.engine = Engine.from_model_dir(model_dir, cfg)
+            cfg.page_size = int(page_size)
+        if num_pages is not None:
+            tokens = int(num_pages) * cfg.page_size
+        elif max_tokens is not None:
+            tokens = int(max_tokens)
+        else:
+            raise ValueError("trace replay needs the pool's size: max_tokens or num_pages")
+        cfg.max_cache_tokens = max(tokens, cfg.page_size)
+        # a step may bring as much as the pool holds (a whole request at once)
+        cfg.max_num_batched_tokens = max(cfg.max_num_batched_tokens, cfg.max_cache_tokens)
+        if random_config is not None:
+            self.engine = Engine.from_config(random_config, cfg, seed=weights_seed)
+        else:
+            self.engine = Engine.from_model_dir(model_dir, cfg)
         self._ids: Dict[object, int] = {}
         self._next = 0
 

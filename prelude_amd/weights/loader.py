@@ -4,6 +4,11 @@ What the reference does per tensor (fetch by dotted name, cast to the engine's
 type, then check the shape: crates/prelude-core/src/engine/weight_loader.rs:200-285,
 :379-404) is done here for the whole model at once, before anything is copied:
 one error lists every missing tensor, every unexpected one and every wrong shape.
+The reference passes over whatever it does not fetch; here only the names an
+architecture declares it may meet and does not read (``ModelSpec.ignored_tensors``:
+the unused head of a tied checkpoint, exported rotary frequencies) are passed
+over, and anything else nothing asks for is reported, since it most often
+means the wrong architecture or a renamed tensor.
 
 Element types on the device: matrices take the engine's type (bfloat16 for
 serving, float32 for the 32-bit path); norm scales and biases are always
@@ -12,7 +17,8 @@ exactly; integer tensors become int32.
 """
 from __future__ import annotations
 
-from typing import Dict, Mapping, Tuple
+import fnmatch
+from typing import Dict, Mapping, Sequence, Tuple
 
 import torch
 
@@ -24,7 +30,9 @@ class WeightError(ValueError):
     pass
 
 
-def check_tensors(requests: Mapping[str, TensorReq], files: WeightFiles, where: str) -> None:
+def check_tensors(requests: Mapping[str, TensorReq], files: WeightFiles, where: str,
+                  ignored: Sequence[str] = ()) -> None:
+    """``ignored``: shell patterns of names the files may hold although nothing asks for them."""
     missing, wrong = [], []
     for name, req in requests.items():
         if name not in files:
@@ -35,7 +43,7 @@ def check_tensors(requests: Mapping[str, TensorReq], files: WeightFiles, where: 
             wrong.append(f"{name}: expected {list(req.shape)}, got {list(shape)}")
         elif not (dt.is_floating_point or dt in (torch.int32, torch.int64)):
             wrong.append(f"{name}: element type {dt} cannot be used")
-    unexpected = [n for n in files.names() if n not in requests]
+    unexpected = [n for n in files.names() if n not in requests and not any(fnmatch.fnmatchcase(n, p) for p in ignored)]
     if missing or wrong or unexpected:
         def part(title, items):
             if not items:
@@ -58,7 +66,7 @@ def load_into(model, model_dir: str, dtype: torch.dtype, device: torch.device) -
     files = WeightFiles(model_dir)
     try:
         requests = model.tensor_requests()
-        check_tensors(requests, files, model_dir)
+        check_tensors(requests, files, model_dir, model.spec.ignored_tensors)
         cache: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
 
         def fetch(name: str, req: TensorReq) -> torch.Tensor:

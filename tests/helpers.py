@@ -9,7 +9,7 @@ import torch
 import plain_model as pm
 
 CONFIGS = {"a": pm.tiny_config_a, "b": pm.tiny_config_b, "c": pm.tiny_config_c}
-# weights as BASELINE names them for A and B; C is ours
+# (seed, matrix std, norm-scale std) of each configuration's weights
 WEIGHT_STATS = {"a": (0, 0.02, 0.01), "b": (1, 0.05, 0.05), "c": (2, 0.05, 0.03)}
 PAGE = {"a": 8, "b": 16, "c": 8}
 _keep = []
@@ -43,10 +43,15 @@ def reference_logits(name: str, seed: int, length: int, stored: str = "float32")
 
 
 def tolerance(dtype: str, ref: torch.Tensor) -> float:
-    """Largest allowed |engine - plain| over a tensor of logits.  float32: rounding of a few
-    hundred 32-bit operations per logit; bfloat16: the 2^-8 rounding of every activation."""
-    scale = max(1.0, float(ref.abs().max()))
-    return (1e-5 if dtype == "float32" else 3e-2) * scale
+    """Largest allowed |engine - plain| over a tensor of logits.  float32: rounding of a few hundred 32-bit
+    operations per logit.  bfloat16: a tenth of the logits' spread (their standard deviation).  Every activation
+    is rounded to 8 bits of mantissa, which adds up to a few hundredths of the spread by the last layer: over the
+    three tiny configurations and sixty drawn ones the largest error measured was 0.03 to 0.063 of it.  A key
+    that is lost, misplaced or taken from another request moves a logit by a quarter of the spread or more, in
+    every configuration; a bound tied to the largest logit instead would let that pass where logits are small."""
+    if dtype == "float32":
+        return 1e-5 * max(1.0, float(ref.abs().max()))
+    return 0.1 * float(ref.double().std())
 
 
 def check(got, ref, dtype, what=""):

@@ -195,3 +195,22 @@ def test_random_orders_lose_nothing(seed):
     for rid in list(live):
         t.close(rid)
     assert [t.free_pages(g) for g in range(2)] == [g[0] for g in groups] and t.free_state_slots() == 3
+
+
+def test_pool_sizes_per_group():
+    """A group with a window needs pages for what a window and a portion span, per request that may run; the
+    Python rule used to size the pools is the manager's own."""
+    from prelude_amd.cache.manager import pages_per_group, peak_pages
+    from prelude_amd.parts.base import KVCacheSpec
+    t = PageTables(8, [(100, 0), (100, 24), (100, 5)])
+    for total in (1, 7, 8, 9, 63, 64, 500):
+        for chunk in (1, 2, 8, 13, 64, 1000):
+            for g, w in enumerate((0, 24, 5)):
+                assert peak_pages(total, chunk, w, 8) == t.peak_pages(total, chunk, g), (total, chunk, w)
+    groups = [KVCacheSpec(2, 16, 0), KVCacheSpec(2, 16, 24), KVCacheSpec(1, 32, 5)]
+    # 4,096 tokens for at most 4 requests fed 16 tokens at a time: 512 pages where every key is kept,
+    # 4 * (ceil((16 + 23) / 8) + 1) = 24 and 4 * (ceil((16 + 4) / 8) + 1) = 16 where a window passes
+    assert pages_per_group(4096, groups, 8, max_requests=4, max_request_tokens=2048, chunk=16) == [512, 24, 16]
+    # never more than the tokens asked for, never less than a page
+    assert pages_per_group(40, groups, 8, max_requests=4, max_request_tokens=2048, chunk=16) == [5, 5, 5]
+    assert pages_per_group(1, groups, 8, max_requests=1, max_request_tokens=8, chunk=1) == [1, 1, 1]

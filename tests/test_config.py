@@ -82,7 +82,8 @@ def test_spec_is_data_from_the_config():
     tied = qwen3_spec(Qwen3Config.from_dict(pm.tiny_config_a()))
     assert tied.head.weights["weight"] == tied.embedding.weights["weight"] == "model.embed_tokens.weight"
     with pytest.raises(ConfigError, match="head_dim"):
-        qwen3_spec(Qwen3Config.from_dict(dict(pm.tiny_config_a(), head_dim=24)))
+        qwen3_spec(Qwen3Config.from_dict(dict(pm.tiny_config_a(), head_dim=258)))
+    assert qwen3_spec(Qwen3Config.from_dict(dict(pm.tiny_config_a(), head_dim=24))).layers[0].parts["mixer"].params["head_dim"] == 24
     with pytest.raises(ConfigError, match="hidden_act"):
         qwen3_spec(Qwen3Config.from_dict(dict(pm.tiny_config_a(), hidden_act="gelu")))
 

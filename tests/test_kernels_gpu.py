@@ -125,7 +125,10 @@ def test_linear_bf16(gpu, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 2560, 4096), (8, 6144, 2560), (8, 2560, 9728), (13, 509, 96), (16, 331, 80),
                                    (17, 64, 64), (33, 192, 160), (24, 9728, 2560), (32, 200, 72), (64, 2560, 2560), (5, 19456, 2560), (2, 40, 8),
-                                   (3, 151936, 256), (40, 336, 8256), (64, 4112, 8192), (9, 48, 8320)])
+                                   (3, 151936, 256), (40, 336, 8256), (64, 4112, 8192), (9, 48, 8320),
+                                   # the launch shapes that only the weights of larger models reach: 320 tiles or more with
+                                   # rows of 128 steps or more (eight wavefronts on two tiles, or on one for few short rows)
+                                   (8, 5120, 25600), (1, 5120, 8192), (5, 5120, 8192), (16, 5120, 5120), (24, 24576, 4096)])
 def test_gemm_skinny(gpu, m, n, k):
     x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
     ref = x.double() @ w.double().T

@@ -73,3 +73,37 @@ def test_drawn_configuration(gpu, seed):
             check(np.concatenate(outs), ref[56:70], dtype, "decoding alone: " + what)
             r.step([], ["p", "d"])
             assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
+@pytest.mark.parametrize("hd,nh,nkv,hidden", [(8, 4, 2, 40), (20, 3, 1, 50), (24, 6, 2, 72), (40, 2, 2, 100), (250, 2, 1, 36)])
+def test_head_sizes_outside_steps_of_16(gpu, hd, nh, nkv, hidden):
+    """Head sizes that are no multiple of 16 (and widths that are no multiple of 8) are not refused: the generic
+    kernels take them, in 32-bit and in bfloat16, whole and in portions beside a decoding request."""
+    from prelude_amd.trace import TraceRunner
+    from prelude_amd.weights import write_safetensors
+    cfg = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=203, hidden_size=hidden,
+               intermediate_size=60, num_hidden_layers=2, num_attention_heads=nh, num_key_value_heads=nkv, head_dim=hd,
+               attention_bias=False, max_position_embeddings=128, sliding_window=None, max_window_layers=2,
+               tie_word_embeddings=True, rope_theta=10000.0, rms_norm_eps=1e-6, use_sliding_window=False,
+               hidden_act="silu", eos_token_id=0)
+    w = pm.random_weights(cfg, seed=hd, std=0.08, norm_std=0.05)
+    toks = np.random.default_rng(hd).integers(0, 203, size=70).tolist()
+    refs = {"float32": pm.forward(cfg, w, toks),
+            "bfloat16": pm.forward(cfg, {k: v.to(torch.bfloat16).float() for k, v in w.items()}, toks)}
+    with tempfile.TemporaryDirectory(prefix="prelude_amd_hd_") as folder:
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        write_safetensors(os.path.join(folder, "model.safetensors"), w)
+        for dtype in ("float32", "bfloat16"):
+            r = TraceRunner(folder, dtype, 256, page_size=16)
+            got = r.step([{"id": "w", "tokens": toks, "want": list(range(70))}], ["w"])
+            check(got, refs[dtype], dtype, f"whole, head_dim {hd} {dtype}")
+            r.step([{"id": "d", "tokens": toks[:40], "want": []}])
+            at, a, b = 0, [], []
+            for k, n in enumerate((19, 2, 30, 1, 18)):
+                out = r.step([{"id": "p", "tokens": toks[at:at + n], "want": list(range(n))},
+                              {"id": "d", "tokens": [toks[40 + k]], "want": [0]}])
+                a.append(out[:n]), b.append(out[n:])
+                at += n
+            check(np.concatenate(a), refs[dtype], dtype, f"portions, head_dim {hd} {dtype}")
+            check(np.concatenate(b), refs[dtype][40:45], dtype, f"decoding, head_dim {hd} {dtype}")

@@ -107,3 +107,53 @@ def test_greedy_generation_at_real_widths(gpu):
     llm = LLM(folder, dtype="float32", max_cache_tokens=512)
     res = llm.generate([toks[:20]], max_tokens=4, temperature=0.0)[0]
     assert res.token_ids == pm.greedy(wide_config(), w64, toks[:20], 4)
+
+
+@functools.lru_cache(maxsize=None)
+def long_model():
+    """The same layer widths under a small vocabulary, for a sequence of 700 tokens.  With these weights a split
+    of 256 keys that is left out of one layer's attention moves the logits of the positions behind it by 0.34 to
+    0.92 of their spread (second layer) or 2.7 to 4.7 (first layer), measured with the plain implementation; the
+    bound for bfloat16 is a tenth of the spread and the engine's error 0.06 of it."""
+    from prelude_amd.weights import write_safetensors
+    cfg = dict(wide_config(), vocab_size=4099, eos_token_id=4098)
+    w = pm.random_weights(cfg, seed=9, std=0.02, norm_std=0.02)
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    tmp = tempfile.TemporaryDirectory(prefix="prelude_amd_test_long_")
+    _keep.append(tmp)
+    with open(os.path.join(tmp.name, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(tmp.name, "model.safetensors"), w)
+    toks = torch.randint(0, cfg["vocab_size"], (700,), generator=torch.Generator().manual_seed(33)).tolist()
+    return tmp.name, toks, pm.forward(cfg, {k: v.double() for k, v in w.items()}, toks)
+
+
+def test_decoding_far_into_a_context_from_graphs(gpu):
+    """What serving runs at this width -- the decode attention that takes the raw projection, over several splits
+    of 256 keys with their merge, replayed from a captured graph -- against the plain implementation: 560 tokens
+    in one step and the next 32 one by one, then three requests decoding together while their contexts pass 256
+    and 512 keys (one split becomes two, two become three)."""
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref = long_model()
+    r = TraceRunner(folder, "bfloat16", 2048, page_size=16)
+    assert r.engine._graphs is not None
+    outs = [r.step([{"id": "d", "tokens": toks[:560], "want": [0, 255, 256, 559]}])]
+    check(outs[0], ref[[0, 255, 256, 559]], "bfloat16", "the portion")
+    rows = [r.step([{"id": "d", "tokens": [toks[i]], "want": [0]}]) for i in range(560, 592)]
+    check(np.concatenate(rows), ref[560:592], "bfloat16", "decoded from position 560")
+    replays = r.engine._graphs.replays
+    assert replays == 32 and r.engine._graphs.captures == 1
+    r.step([], ["d"])
+    starts = {"x": 250, "y": 505, "z": 660}
+    for rid, s0 in starts.items():
+        r.step([{"id": rid, "tokens": toks[:s0], "want": []}])
+    got = {rid: [] for rid in starts}
+    for k in range(14):
+        out = r.step([{"id": rid, "tokens": [toks[s0 + k]], "want": [0]} for rid, s0 in starts.items()])
+        for j, rid in enumerate(starts):
+            got[rid].append(out[j:j + 1])
+    assert r.engine._graphs.replays == replays + 14
+    for rid, s0 in starts.items():
+        check(np.concatenate(got[rid]), ref[s0:s0 + 14], "bfloat16", f"request decoding from position {s0}")
+    r.step([], list(starts))
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0

@@ -185,13 +185,8 @@ def test_errors_leave_the_cache_intact(gpu):
     assert r.engine.length(0) == 40
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_trace_run_program(gpu, dtype, tmp_path):
-    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and `done <step>` lines out."""
-    folder, cfg, _ = model_folder("b")
-    toks, ref = reference_logits("b", 0, 180)
-    toks2, ref2 = reference_logits("b", 1, 180)
-    steps = [
+def _trace_steps(toks, toks2):
+    return [
         {"step": 0, "entries": [{"id": "a", "tokens": toks[:50], "want": [0, 49]}], "end": []},
         {"step": 1, "entries": [{"id": "a", "tokens": toks[50:52], "want": []},
                                 {"id": "b", "tokens": toks2[:30], "want": [29]}], "end": []},
@@ -199,12 +194,26 @@ def test_trace_run_program(gpu, dtype, tmp_path):
                                 {"id": "b", "tokens": toks2[30:31], "want": [0]}], "end": ["a"]},
         {"step": 5, "entries": [{"id": "b", "tokens": toks2[31:40], "want": [8]}], "end": ["b"]},
     ]
-    out = tmp_path / "out"
-    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
-                        "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
-                       capture_output=True, text=True, timeout=300)
+
+
+def _run_program(args, steps, out):
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), *args, "--out", str(out)],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
     assert p.returncode == 0, p.stderr[-2000:]
-    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 5"]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,pool", [("a", ["--page-size", "8", "--num-pages", "13"]), ("b", ["--max-tokens", "128"])])
+def test_trace_run_program(gpu, dtype, name, pool, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and `done <step>` lines out; Tiny A with
+    its pages of 8 given as a number of pages, Tiny B with pages of 16 and the pool given in tokens."""
+    folder, cfg, _ = model_folder(name)
+    n = LENGTHS[name]
+    toks, ref = reference_logits(name, 0, n)
+    toks2, ref2 = reference_logits(name, 1, n)
+    out = tmp_path / "out"
+    _run_program(["--model", folder, "--dtype", dtype, *pool], _trace_steps(toks, toks2), out)
     v = cfg["vocab_size"]
     load = lambda s: np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(-1, v)
     check(load(0), ref[[0, 49]], dtype, "step 0")
@@ -212,6 +221,31 @@ def test_trace_run_program(gpu, dtype, tmp_path):
     check(load(2), torch.stack([ref[52], ref2[30]]), dtype, "step 2")
     check(load(5), ref2[[39]], dtype, "step 5")
     assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "2.f32", "5.f32"]
+
+
+def test_trace_run_program_from_a_bare_config(gpu, tmp_path):
+    """--random-weights: only a config.json is there; the weights are drawn on the device from the seed, the
+    same ones ``random_tensors_on_device`` gives, which the plain implementation is run on here."""
+    from prelude_amd.weights import random_tensors_on_device
+    import plain_model as pm
+    cfg = pm.tiny_config_a()
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    w = {k: v.float().cpu() for k, v in random_tensors_on_device(cfg, 5, gpu, dtype=torch.float32).items()}
+    g = torch.Generator().manual_seed(77)
+    toks, toks2 = (torch.randint(0, cfg["vocab_size"], (60,), generator=g).tolist() for _ in range(2))
+    ref, ref2 = pm.forward(cfg, w, toks), pm.forward(cfg, w, toks2)
+    out = tmp_path / "out"
+    _run_program(["--random-weights", str(tmp_path / "config.json"), "--weights-seed", "5", "--dtype", "float32",
+                  "--page-size", "8", "--num-pages", "13"], _trace_steps(toks, toks2), out)
+    load = lambda s: np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])
+    check(load(0), ref[[0, 49]], "float32", "step 0")
+    check(load(2), torch.stack([ref[52], ref2[30]]), "float32", "step 2")
+    check(load(5), ref2[[39]], "float32", "step 5")
+    # another seed, other weights
+    out2 = tmp_path / "out2"
+    _run_program(["--random-weights", str(tmp_path), "--weights-seed", "6", "--dtype", "float32", "--max-tokens", "128"],
+                 _trace_steps(toks, toks2)[:1], out2)
+    assert float(np.abs(np.fromfile(out2 / "0.f32", dtype="<f4").reshape(-1, cfg["vocab_size"]) - load(0)).max()) > 1e-3
 
 
 def test_graph_replays_equal_eager_steps(gpu):

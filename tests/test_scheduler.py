@@ -69,6 +69,50 @@ def test_per_request_cap():
     assert [(p.id, p.count) for p in ps] == [(1, 64), (2, 30)]
 
 
+def test_a_request_of_its_own_portion_cap():
+    # a cap that holds for one request only (its logits are wanted at every prompt position, say)
+    _, s = make(max_num_batched_tokens=100)
+    s.add_request(1, 70, 2, max_chunk=32)
+    s.add_request(2, 70, 2)
+    ps = run_step(s)
+    assert [(p.id, p.start, p.count) for p in ps] == [(1, 0, 32), (2, 0, 68)]
+    ps = run_step(s)
+    assert [(p.id, p.start, p.count) for p in ps] == [(1, 32, 32), (2, 68, 2)]
+    ps = run_step(s)
+    assert [(p.id, p.start, p.count, p.samples) for p in ps] == [(1, 64, 6, True), (2, 70, 1, True)]
+
+
+def test_a_request_fed_whole_or_not_at_all():
+    """A request whose mixers cannot continue a prompt from a cut is never given a part of its prompt: it waits
+    for a step that takes all of it, and after an eviction it is fed prompt and generated tokens whole again."""
+    _, s = make(max_num_batched_tokens=64)
+    s.add_request(1, 40, 30)
+    run_step(s)                                   # 1 is decoding
+    s.add_request(2, 62, 2, atomic=True)          # 62 + 1 decode token of request 1 = 63 <= 64: fits whole
+    s.add_request(3, 30, 2, atomic=True)          # only 1 token of the budget is left: not cut, waits
+    ps = run_step(s)
+    assert [(p.id, p.start, p.count, p.samples) for p in ps] == [(1, 40, 1, True), (2, 0, 62, True)]
+    ps = run_step(s)
+    assert [(p.id, p.start, p.count) for p in ps] == [(1, 41, 1), (2, 62, 1), (3, 0, 30)]
+    # what could never be fed whole is refused when it is added, with what a step takes
+    with pytest.raises(SchedulerError, match="must be fed whole .70 tokens.*a step takes 64"):
+        s.add_request(4, 60, 11, atomic=True)
+    with pytest.raises(SchedulerError, match="a step takes 16"):
+        s.add_request(5, 20, 1, atomic=True, max_chunk=16)
+    # pages: a whole portion that the free pages cannot hold is not shortened
+    tables, s = make(pages=6, page=16, max_num_batched_tokens=128, decode_reservation_cap=0)
+    s.add_request(1, 60, 4)
+    run_step(s)                                   # 4 pages held by request 1
+    s.add_request(2, 50, 2, atomic=True)          # needs 4 pages, 2 are free: waits, whole
+    ps = run_step(s)
+    assert [(p.id, p.count) for p in ps] == [(1, 1)]
+    for _ in range(2):
+        assert [(p.id, p.count) for p in run_step(s)] == [(1, 1)]   # request 1 ends and gives its pages back
+    ps = run_step(s)
+    assert [(p.id, p.start, p.count, p.samples) for p in ps] == [(2, 0, 50, True)]
+    assert tables.audit() == ""
+
+
 def test_running_cap_and_fcfs():
     _, s = make(max_running_requests=2)
     for i in range(4):

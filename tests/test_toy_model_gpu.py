@@ -25,6 +25,8 @@ def register_toy():
     class ToyDecay(Mixer):
         """s_t = decay * s_{t-1} + x_t per request; y_t = W s_t.  The state s lives in a slot of the cache manager."""
 
+        GRAPH_SAFE = False     # it walks the step's host-side lists
+
         def __init__(self, hidden_size, decay):
             self.hidden_size, self.decay = hidden_size, decay
             self.w = None
@@ -52,6 +54,21 @@ def register_toy():
                 t += n
             return K.linear(out, self.w)
 
+    @register_part("mixer", "toy_decay_device")
+    class ToyDecayDevice(ToyDecay):
+        """The same mixer with its decode step written on the device alone: it finds its slots through
+        ``step.state_slots``, so a step of single tokens can be captured once and replayed."""
+        GRAPH_SAFE = True
+
+        def forward(self, x, step, cache, write_cache=True):
+            if not step.all_decode:
+                return super().forward(x, step, cache, write_cache)
+            s_all = cache.tensors["s"]
+            slots = step.state_slots.to(torch.int64)
+            s = self.decay * s_all.index_select(0, slots) + x.float()
+            s_all.index_copy_(0, slots, s)
+            return K.linear(s.to(x.dtype), self.w)
+
     @dataclasses.dataclass
     class ToyConfig:
         vocab_size: int
@@ -66,12 +83,12 @@ def register_toy():
     def parse(raw):
         return ToyConfig(**{f.name: raw[f.name] for f in dataclasses.fields(ToyConfig)})
 
-    def spec(c):
+    def spec(c, mixer="toy_decay"):
         norm = lambda name: PartSpec("rms_norm", dict(size=c.hidden_size, eps=c.eps), {"weight": name})
         ffn = lambda p: PartSpec("gated_mlp", dict(hidden_size=c.hidden_size, intermediate_size=c.inter),
                                  {f"{x}_proj.weight": f"{p}.ffn.{x}" for x in ("gate", "up", "down")})
         toy = LayerSpec("prenorm", {"input_norm": norm("l0.n1"), "post_mixer_norm": norm("l0.n2"), "ffn": ffn("l0"),
-                                    "mixer": PartSpec("toy_decay", dict(hidden_size=c.hidden_size, decay=c.decay),
+                                    "mixer": PartSpec(mixer, dict(hidden_size=c.hidden_size, decay=c.decay),
                                                       {"proj.weight": "l0.mix.proj"})})
         attn = LayerSpec("prenorm", {"input_norm": norm("l1.n1"), "post_mixer_norm": norm("l1.n2"), "ffn": ffn("l1"),
                                      "mixer": PartSpec("gqa_attention", dict(
@@ -87,6 +104,8 @@ def register_toy():
                          {"rope": PartSpec("rope", dict(rotary_dim=c.head_dim, max_positions=c.max_positions, theta=100.0))})
 
     register_architecture(Architecture("toy", ("Toy",), ("toy",), parse, spec))
+    register_architecture(Architecture("toydevice", ("ToyDevice",), ("toydevice",), parse,
+                                       lambda c: spec(c, "toy_decay_device")))
 
 
 RAW = dict(architectures=["ToyForCausalLM"], vocab_size=97, hidden_size=48, inter=80, heads=3, head_dim=16, decay=0.7,
@@ -195,3 +214,49 @@ def test_toy_model_generates_through_the_entry_point(gpu, tmp_path):
             seq.append(tok)
         assert o.finish_reason in ("length", "eos")
     assert llm.engine.tables.audit() == "" and llm.engine.tables.free_state_slots() == 2
+
+
+def test_toy_model_with_state_decodes_from_graphs(gpu, tmp_path):
+    """A model whose mixer keeps state per request is captured and replayed like any other once its decode step
+    stays on the device: slots come through ``step.state_slots``, and the slot of a request that starts inside a
+    captured step (a prompt of one token, in a slot another request has used) is cleared on the device."""
+    register_toy()
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    from prelude_amd.weights import WeightFiles, write_random_model
+    raw = dict(RAW, architectures=["ToyDeviceForCausalLM"])
+    folder = write_random_model(raw, str(tmp_path / "toydev"), seed=6, std=0.2, norm_std=0.1, dtype=torch.bfloat16)
+    files = WeightFiles(folder)
+    w = {n: files.tensor(n).float() for n in files.names()}
+    g = torch.Generator().manual_seed(3)
+    seqs = [torch.randint(0, 97, (n,), generator=g).tolist() for n in (40, 33, 25)]
+    refs = [plain_toy(w, s) for s in seqs]
+
+    def play(hip_graph):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=8, max_cache_tokens=256,
+                                                         max_state_slots=2, hip_graph=hip_graph))
+        assert eng.model.needs_state and eng.model.graph_safe
+        rows = {0: [], 1: [], 2: []}
+        eng.step([StepEntry(0, seqs[0][:20], [])])
+        eng.step([StepEntry(1, seqs[1][:9], [])])
+        for k in range(12):                               # both slots in use, a batch of two, replayed
+            out = eng.step([StepEntry(0, [seqs[0][20 + k]], [0]), StepEntry(1, [seqs[1][9 + k]], [0])])
+            rows[0].append(out[0:1].cpu()), rows[1].append(out[1:2].cpu())
+        eng.release(1)                                    # its slot holds what request 1 left there
+        for k in range(8):                                # request 2 starts inside the captured step of two
+            out = eng.step([StepEntry(0, [seqs[0][32 + k]], [0]), StepEntry(2, [seqs[2][k]], [0])])
+            rows[0].append(out[0:1].cpu()), rows[2].append(out[1:2].cpu())
+        return eng, {r: torch.cat(v) for r, v in rows.items()}
+
+    eager_eng, eager = play(False)
+    eng, replayed = play(True)
+    assert eager_eng._graphs is None and eng._graphs.captures == 1 and eng._graphs.replays == 20
+    for r in rows_of(eager):
+        assert torch.equal(eager[r], replayed[r])
+    from helpers import check
+    for r, lo, hi in ((0, 20, 40), (1, 9, 21), (2, 0, 8)):
+        check(replayed[r], refs[r][lo:hi], "bfloat16", f"request {r}")
+
+
+def rows_of(d):
+    return sorted(d)

@@ -88,14 +88,28 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     assert "wrong shape (2)" in msg and "expected [32], got [16]" in msg and "expected [32, 96], got [32, 95]" in msg
 
 
-def test_tied_model_refuses_a_stray_head(tmp_path):
+def test_tensors_an_architecture_knows_of_and_does_not_read_are_passed_over(tmp_path):
+    """A tied checkpoint that still carries its unused head, and exported rotary frequencies, load (the reference
+    fetches by name and never looks at them: crates/prelude-core/src/models/qwen3.rs:637-643,
+    crates/prelude-core/src/engine/weight_loader.rs:200-285); anything else nothing asks for is still reported."""
     raw = pm.tiny_config_a()
     t = random_tensors(raw, seed=0)
     assert "lm_head.weight" not in t
     t["lm_head.weight"] = torch.zeros(256, 64)
+    t["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
     write_safetensors(str(tmp_path / "model.safetensors"), t)
-    with pytest.raises(WeightError, match="unexpected"):
-        check_tensors(_model(raw).tensor_requests(), WeightFiles(str(tmp_path)), "X")
+    model = _model(raw)
+    assert model.spec.ignored_tensors == ("*.rotary_emb.inv_freq", "lm_head.weight")
+    check_tensors(model.tensor_requests(), WeightFiles(str(tmp_path)), "X", model.spec.ignored_tensors)
+    with pytest.raises(WeightError, match=r"unexpected \(2\)"):      # without the architecture's say-so: reported
+        check_tensors(model.tensor_requests(), WeightFiles(str(tmp_path)), "X")
+    t["model.layers.0.mlp.gate_up_proj.weight"] = torch.zeros(4)
+    write_safetensors(str(tmp_path / "model.safetensors"), t)
+    with pytest.raises(WeightError, match=r"unexpected \(1\)") as ei:
+        check_tensors(model.tensor_requests(), WeightFiles(str(tmp_path)), "X", model.spec.ignored_tensors)
+    assert "gate_up_proj" in str(ei.value) and "lm_head" not in str(ei.value)
+    # an untied model asks for its head: nothing is passed over there but the frequencies
+    assert _model(pm.tiny_config_b()).spec.ignored_tensors == ("*.rotary_emb.inv_freq",)
 
 
 def test_device_types():
