@@ -71,13 +71,23 @@ __device__ __forceinline__ float xor_sum16_32(float v) {
 }
 
 // What a wavefront keeps per head while it walks keys: per lane, query column r.
+//
+// The exponentials are taken against a reference maximum `m` that follows the true running maximum lazily: it
+// moves only when a score exceeds it by more than kLazyLog2 in the exponent (then every term so far is rescaled);
+// until then a probability may be as large as 2^kLazyLog2 instead of at most 1, which costs 32-bit sums and bfloat16
+// probabilities nothing (the quotient O / l is the same), and spares the rescaling of the whole output in most steps.
+// The sum `l` is formed by the matrix cores too, as one more row of V^T that holds ones: it adds up the same
+// rounded probabilities the output is made of, all 32 keys of a step at once, and every lane of a column has it.
+constexpr float kLazyLog2 = 8.0f;
+
 template <int HD>
 struct HeadState {
   static constexpr int OT = HD / 16;
-  float m = -INFINITY;  // running maximum of the raw scores, equal in the four lanes of a column
-  float l = 0.f;        // this lane's share of the running sum
+  float m = -INFINITY;  // reference maximum of the raw scores, equal in the four lanes of a column
+  f32x4 l;              // running sum of the column's probabilities (every element the same)
   f32x4 o[OT];          // O^T tiles: head_dim rows 16 t + 4g + i, column r
   __device__ HeadState() {
+    l = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < OT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -162,13 +172,21 @@ __device__ __forceinline__ bf16x8 load_v(const VChunks& v, int d, int page_shift
   return u.v8;
 }
 
+__device__ __forceinline__ bf16x8 ones8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (bf16)1.f;
+  return z;
+}
+
 // Scores of 32 keys against one head's 16 queries, then the online softmax: returns the probabilities packed
-// as the B operand of O^T = V^T P^T and the factor the head's output so far must be scaled by.
+// as the B operand of O^T = V^T P^T.  `moved` says whether this lane's reference maximum moved; `m_before` is
+// what it was (the caller rescales the head's sums by 2^((m_before - m) c) then).
 // `masked` false: every key of the step is visible to every query (no comparisons).
 // `vis(key)` says whether this lane's query may see the key (and the key exists).
 template <int HD, typename Visible>
 __device__ __forceinline__ bf16x8 scores32(int key0, int g, const KFrag<HD>& kf, const bf16x8* qf, float c,
-                                           bool masked, HeadState<HD>& st, float& alpha, Visible vis) {
+                                           bool masked, HeadState<HD>& st, bool& moved, float& m_before, Visible vis) {
   float s[8];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -189,20 +207,16 @@ __device__ __forceinline__ bf16x8 scores32(int key0, int g, const KFrag<HD>& kf,
 #pragma unroll
   for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
   mx = xor_max16_32(mx);
-  const float m_new = fmaxf(st.m, mx);
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a column that has seen no key yet
-  alpha = __builtin_amdgcn_exp2f((st.m - m_safe) * c);
+  m_before = st.m;
+  // from -inf any finite score moves it (the difference is +inf); -inf against -inf gives NaN, which compares false
+  moved = (mx - st.m) * c > kLazyLog2;
+  if (moved) st.m = mx;
+  const float m_safe = st.m == -INFINITY ? 0.f : st.m;  // a column that has seen no key yet
   const float shift = -m_safe * c;
   bf16x8 pb;
-  float psum = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float p = __builtin_amdgcn_exp2f(fmaf(s[i], c, shift));  // 2^((s - m) c), c = scale * log2(e)
-    psum += p;
-    pb[i] = (bf16)p;
-  }
-  st.l = st.l * alpha + psum;
-  st.m = m_new;
+  for (int i = 0; i < 8; ++i)
+    pb[i] = (bf16)__builtin_amdgcn_exp2f(fmaf(s[i], c, shift));  // 2^((s - m) c), c = scale * log2(e)
   return pb;
 }
 
@@ -220,30 +234,35 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool valid, int g, bf16
 }
 
 // The arithmetic of one step over 32 keys for GT heads that share the keys: the scores and softmax of every
-// head first, then each V^T tile is used by all heads.  An output is rescaled only when some maximum moved.
+// head first, then each V^T tile is used by all heads.  A head's sums are rescaled only in steps in which the
+// reference maximum of one of its columns moved.
 template <int HD, int GT, typename Visible>
 __device__ __forceinline__ void attend32_core(int key0, int g, const KFrag<HD>& kf, const bf16x8* va,
                                               const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked,
                                               HeadState<HD>* st, Visible vis) {
   constexpr int OT = HeadState<HD>::OT;
   bf16x8 pb[GT];
-  float alpha[GT];
-  bool rescale[GT];
+  bool moved[GT];
+  float m_before[GT];
+#pragma unroll
+  for (int j = 0; j < GT; ++j) pb[j] = scores32<HD>(key0, g, kf, qf[j], c, masked, st[j], moved[j], m_before[j], vis);
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
-    pb[j] = scores32<HD>(key0, g, kf, qf[j], c, masked, st[j], alpha[j], vis);
-    rescale[j] = __any(alpha[j] != 1.0f);
-  }
-#pragma unroll
-  for (int j = 0; j < GT; ++j) {
-    if (rescale[j]) {
+    if (__any(moved[j])) {
       asm volatile("" ::: "memory");  // keep this a branch: as selects it would cost a multiply per output every step
+      // 2^(-inf) = 0 for a column's first keys: its sums are zero anyway
+      const float alpha = moved[j] ? __builtin_amdgcn_exp2f((m_before[j] - st[j].m) * c) : 1.0f;
 #pragma unroll
       for (int t = 0; t < OT; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) st[j].o[t][i] *= alpha[j];
+        for (int i = 0; i < 4; ++i) st[j].o[t][i] *= alpha;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st[j].l[i] *= alpha;
     }
   }
+  const bf16x8 ones = ones8();
+#pragma unroll
+  for (int j = 0; j < GT; ++j) st[j].l = mfma16(ones, pb[j], st[j].l);
 #pragma unroll
   for (int t = 0; t < OT; ++t)
 #pragma unroll
@@ -449,7 +468,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
     attend32<HD, 1>(w, key0, g, r, kf, qf, c, masked, st, [&](int key) { return key >= k_begin && key < k_end; });
   }
   // merge the four wavefronts through LDS; maxima leave in the log2 domain (raw maximum times c)
-  const float l_wave = xor_sum16_32(st[0].l);
+  const float l_wave = st[0].l[0];
   if (g == 0) {
     lds_ml[wave][r][0] = st[0].m * c;
     lds_ml[wave][r][1] = l_wave;
@@ -613,7 +632,7 @@ __device__ __forceinline__ void prefill_tile(const bf16* __restrict__ q, bf16* _
   if (!qvalid) return;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
-    const float inv = 1.0f / xor_sum16_32(st[j].l);
+    const float inv = 1.0f / st[j].l[0];
     bf16* orow = out + ((size_t)(row0 + t0 + r) * nh + head0 + j) * HD;
 #pragma unroll
     for (int t = 0; t < OT; ++t) {
@@ -836,7 +855,7 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
   if (!qvalid) return;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
-    const float inv = 1.0f / xor_sum16_32(st[j].l);
+    const float inv = 1.0f / st[j].l[0];
     bf16* orow = out + ((size_t)(row0 + t0 + r) * nh + head0 + j) * HD;
 #pragma unroll
     for (int t = 0; t < OT; ++t) {
