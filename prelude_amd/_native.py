@@ -50,6 +50,11 @@ _KERNEL_API = {
     "pa_gemm_library": (I, [P, P, P, P, I, I, I, c_long, c_long, P, c_long]),
     "pa_gemm_skinny": (I, [P, I, I, P, P, P, P, I, I, I, c_long, c_long, I]),
     "pa_pack_tiles": (I, [P, P, P, I, I]),
+    "pa_gemm_mid_slices": (I, [I, I]),
+    "pa_gemm_mid_parts": (c_long, [I, I, I]),
+    "pa_gemm_mid": (I, [P, I, I, P, P, P, P, P, I, I, I, c_long, c_long, I]),
+    "pa_sum_slices": (I, [P, I, P, P, I, c_long]),
+    "pa_rmsnorm_slices": (I, [P, I, P, I, c_long, P, P, P, P, I, I, F]),
     "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
     "pa_attn_mfma_supports": (I, [I, I]),
     "pa_attn_decode_workspace": (c_long, [I, I, I, I]),

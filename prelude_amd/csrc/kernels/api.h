@@ -25,6 +25,10 @@ int pa_zero_fresh_rows(void* stream, void* data, long row_bytes, const int* slot
 // with `rows`, output row r comes from input row rows[r] and the residual is left alone.
 int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out, const int* rows,
                int nrows, int hidden, float eps);
+// The same with x given as `slices` 32-bit partial sums [slices, rows, hidden], slice_stride elements apart (what
+// pa_gemm_mid leaves of a product cut along its inner size): they are added in order as they are loaded.
+int pa_rmsnorm_slices(void* stream, int dtype, const float* parts, int slices, long slice_stride, void* residual,
+                      const float* w, void* out, const int* rows, int nrows, int hidden, float eps);
 // out[t, c] = silu(gate_up[t, 2c]) * gate_up[t, 2c + 1]   (columns alternate gate_j, up_j)
 int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter);
 int pa_gather_rows(void* stream, int dtype, const void* x, const int* rows, void* out, int nrows, int width);
@@ -52,6 +56,17 @@ int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, cons
 // tiled 1: w is the weight as pa_pack_tiles lays it out.
 int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
                    int m, int n, int k, long ldx, long ldc, int tiled);
+// C[m, n] = X[m, k] W[n, k]^T for m <= 128 from the weight in tiles, X staged through LDS and W streamed by four
+// wavefronts a workgroup (64 rows of W).  slices 1: as pa_gemm_skinny (epilogue 0 (+ bias) / 1 SiLU * up).
+// slices > 1 (epilogue 0): the inner size is cut into that many slices, each left as 32-bit sums in
+// parts [slices, m, n] (pa_gemm_mid_parts floats; the bias in the first) for the reader to add in order, and c is
+// not written.  pa_gemm_mid_slices: the number of slices that suits an [n, k] weight.
+int pa_gemm_mid_slices(int n, int k);
+long pa_gemm_mid_parts(int m, int n, int slices);
+int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
+                float* parts, int m, int n, int k, long ldx, long ldc, int slices);
+// out[i] = parts[0, i] + parts[1, i] + ..; out_dtype 0 = float32, 1 = bfloat16; total = rows * columns.
+int pa_sum_slices(void* stream, int out_dtype, const float* parts, void* out, int slices, long total);
 // out[tile][step][half][g][r][8] = w[16 tile + r][64 step + 16 g + 8 half ..], zero-padded: ceil(n/16) * ceil(k/64) * 1024 elements.
 int pa_pack_tiles(void* stream, const void* w, void* out, int n, int k);
 

@@ -64,25 +64,35 @@ __global__ void zero_fresh_rows_kernel(uint32_t* __restrict__ data, long row_wor
 //   out = round(s * rsqrt(mean(s^2) + eps) * w)   from the unrounded s
 // With `rows`, output row r is computed from input row rows[r] and nothing
 // is written back to the residual: the final norm of only the wanted rows.
+// x may come as `slices` 32-bit partial sums instead ([slices, rows, hidden], `slice_stride` elements apart, as a
+// product cut along its inner size leaves them): they are added in order, in place of the load of x.
 template <typename T>
-__global__ void rmsnorm_kernel(const T* __restrict__ x, T* residual, const float* __restrict__ w,
-                               T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+__global__ void rmsnorm_kernel(const T* __restrict__ x, const float* __restrict__ parts, int slices, size_t slice_stride,
+                               T* residual, const float* __restrict__ w, T* __restrict__ out,
+                               const int* __restrict__ rows, int hidden, float eps) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
-  const T* xr = x + src * hidden;
+  const T* xr = x ? x + src * hidden : nullptr;
+  const float* pr = parts ? parts + src * hidden : nullptr;
   T* rr = residual ? residual + src * hidden : nullptr;
   T* orow = out + (size_t)r * hidden;
+  auto value = [&](int i) {
+    if (!pr) return to_f32(xr[i]);
+    float v = pr[i];
+    for (int p = 1; p < slices; ++p) v += pr[(size_t)p * slice_stride + i];
+    return v;
+  };
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float s = to_f32(xr[i]);
+    float s = value(i);
     if (rr) s += to_f32(rr[i]);
     ss += s * s;
   }
   ss = block_sum(ss, scratch);
   const float inv = rsqrtf(ss / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float s = to_f32(xr[i]);
+    float s = value(i);
     if (rr) s += to_f32(rr[i]);
     if (rr && !rows) rr[i] = from_f32<T>(s);
     orow[i] = from_f32<T>(s * inv * w[i]);
@@ -93,7 +103,8 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, T* residual, const float
 // two passes: one read of x and the residual, one write of each output.
 // NV vectors per thread; the block has ceil(hidden / VEC / NV) threads rounded up to a wavefront.
 template <typename T, int NV>
-__global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const float* __restrict__ w,
+__global__ void rmsnorm_vec_kernel(const T* __restrict__ x, const float* __restrict__ parts, int slices,
+                                   size_t slice_stride, T* residual, const float* __restrict__ w,
                                    T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
   constexpr int VEC = 16 / sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
@@ -101,6 +112,7 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const f
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
   const vec_t* xr = reinterpret_cast<const vec_t*>(x + src * hidden);
+  const float* pr = parts ? parts + src * hidden : nullptr;
   vec_t* rr = residual ? reinterpret_cast<vec_t*>(residual + src * hidden) : nullptr;
   vec_t* orow = reinterpret_cast<vec_t*>(out + (size_t)r * hidden);
   const int nvec = hidden / VEC;
@@ -111,7 +123,21 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const f
   for (int j = 0; j < NV; ++j) {
     const int v = threadIdx.x + j * blockDim.x;
     if (v < nvec) {
-      const vec_t xv = xr[v];
+      if (pr) {   // the slices of a product, added in their order
+#pragma unroll
+        for (int e = 0; e < VEC; e += 4) {
+          float4 a = *reinterpret_cast<const float4*>(pr + (size_t)v * VEC + e);
+          for (int p = 1; p < slices; ++p) {
+            const float4 b = *reinterpret_cast<const float4*>(pr + (size_t)p * slice_stride + (size_t)v * VEC + e);
+            a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+          }
+          s[j][e] = a.x, s[j][e + 1] = a.y, s[j][e + 2] = a.z, s[j][e + 3] = a.w;
+        }
+      } else {
+        const vec_t xv = xr[v];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s[j][e] = to_f32(xv[e]);
+      }
 #pragma unroll
       for (int e = 0; e < VEC; e += 4) {
         const float4 w4 = *reinterpret_cast<const float4*>(w + (size_t)v * VEC + e);
@@ -120,10 +146,7 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, T* residual, const f
       if (rr) {
         const vec_t rv = rr[v];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) s[j][e] = to_f32(xv[e]) + to_f32(rv[e]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) s[j][e] = to_f32(xv[e]);
+        for (int e = 0; e < VEC; ++e) s[j][e] += to_f32(rv[e]);
       }
 #pragma unroll
       for (int e = 0; e < VEC; ++e) ss += s[j][e] * s[j][e];
@@ -248,10 +271,8 @@ extern "C" int pa_zero_fresh_rows(void* stream, void* data, long row_bytes, cons
   return check_launch("zero_fresh_rows");
 }
 
-extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out,
-                          const int* rows, int nrows, int hidden, float eps) {
-  if (nrows == 0) return 0;
-  PA_REQUIRE(nrows > 0 && hidden > 0, "rmsnorm: bad sizes rows=%d hidden=%d", nrows, hidden);
+static int rmsnorm_launch(void* stream, int dtype, const void* x, const float* parts, int slices, long slice_stride,
+                          void* residual, const float* w, void* out, const int* rows, int nrows, int hidden, float eps) {
   const int vec = dtype == kF32 ? 4 : 8;
   if (hidden % vec == 0 && hidden / vec <= 4 * 1024) {
     const int nvec = hidden / vec;
@@ -260,7 +281,8 @@ extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual
     const int threads = (((nvec + per - 1) / per) + 63) / 64 * 64;
 #define PA_RMS(NV)                                                                                                   \
   PA_DISPATCH(dtype, hipLaunchKernelGGL((rmsnorm_vec_kernel<T, NV>), dim3(nrows), dim3(threads), 0, (hipStream_t)stream, \
-                                        (const T*)x, (T*)residual, w, (T*)out, rows, hidden, eps))
+                                        (const T*)x, parts, slices, (size_t)slice_stride, (T*)residual, w, (T*)out, rows, \
+                                        hidden, eps))
     if (per == 1) {
       PA_RMS(1);
     } else if (per == 2) {
@@ -273,8 +295,26 @@ extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual
   }
   const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
   PA_DISPATCH(dtype, hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(nrows), dim3(threads), 0, (hipStream_t)stream,
-                                        (const T*)x, (T*)residual, w, (T*)out, rows, hidden, eps));
+                                        (const T*)x, parts, slices, (size_t)slice_stride, (T*)residual, w, (T*)out, rows,
+                                        hidden, eps));
   return check_launch("rmsnorm");
+}
+
+extern "C" int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const float* w, void* out,
+                          const int* rows, int nrows, int hidden, float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && hidden > 0, "rmsnorm: bad sizes rows=%d hidden=%d", nrows, hidden);
+  return rmsnorm_launch(stream, dtype, x, nullptr, 0, 0, residual, w, out, rows, nrows, hidden, eps);
+}
+
+extern "C" int pa_rmsnorm_slices(void* stream, int dtype, const float* parts, int slices, long slice_stride,
+                                 void* residual, const float* w, void* out, const int* rows, int nrows, int hidden,
+                                 float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && hidden > 0, "rmsnorm: bad sizes rows=%d hidden=%d", nrows, hidden);
+  PA_REQUIRE(parts && slices >= 1 && slice_stride >= 0 && hidden % 4 == 0,
+             "rmsnorm: %d slices %ld apart of rows of %d (a multiple of 4)", slices, slice_stride, hidden);
+  return rmsnorm_launch(stream, dtype, nullptr, parts, slices, slice_stride, residual, w, out, rows, nrows, hidden, eps);
 }
 
 extern "C" int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter) {

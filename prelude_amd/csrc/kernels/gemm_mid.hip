@@ -1,0 +1,318 @@
+// C[M,N] = X[M,K] * W[N,K]^T for up to 128 rows in bfloat16 with 32-bit accumulation, from the weight in tiles
+// (pa_pack_tiles): the product of decode steps of many requests, and of narrow weights at any number of rows.
+//
+// With more than a few rows the weight-streaming kernel of gemm_skinny.hip reads X as often as it has
+// workgroups: every workgroup owns 16 rows of W and all of K, so a [2560, 9728] weight at 64 rows moves four
+// times as many bytes of X through the caches as it streams of W, and a wavefront that holds the sums of 64
+// rows has few loads in flight.  Here a workgroup owns 64 rows of W (four wavefronts, a tile of 16 rows each)
+// and a slice of K.  X goes through LDS: the slice's columns are staged once per workgroup, a chunk of KC
+// columns ahead of the products, and every wavefront takes its MFMA operands from there; W goes from memory
+// straight into registers, each wavefront streaming its own tile's 2 KB steps with a ring of KC / 64 of them in
+// flight.  X is then read once per 64 rows of W whatever the number of slices, and a narrow weight still gives
+// every compute unit a workgroup: [2560, 4096] is 40 blocks of rows times 8 slices of K.
+//
+// A product cut into slices leaves one 32-bit partial sum per slice, [slices, M, N], and no workgroup waits for
+// another: whoever reads the result adds the slices in order (the residual add + RMSNorm kernel does, as it
+// loads; pa_sum_slices for any other reader).  The order of every sum is fixed by the weight's shape and the
+// number of slices alone.
+//
+// Epilogues of an uncut product as in gemm_skinny.hip: bfloat16 or float32 out, optional bias, or SiLU(gate) * up
+// over rows that alternate gate_j, up_j.
+//
+// Reference counterpart: the GEMM dispatch of crates/prelude-cuda/src/ops/gemm.rs:35-137 (library kernels there).
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+constexpr int kMidWaves = 4;           // wavefronts a workgroup: 64 rows of W
+constexpr int kMidMaxM = 128;
+
+struct MidFrag {
+  bf16x8 lo, hi;
+};
+
+// A step of a tile as pa_pack_tiles lays it out: the wavefront's 64 lanes read 1 KB side by side, twice.
+__device__ __forceinline__ MidFrag mid_load_w(const bf16* tile, int step, int lane) {
+  MidFrag f;
+  const bf16* p = tile + (size_t)step * 1024 + lane * 8;
+  f.lo = *reinterpret_cast<const bf16x8*>(p);
+  f.hi = *reinterpret_cast<const bf16x8*>(p + 512);
+  return f;
+}
+
+enum MidEpilogue : int { kMidPlain = 0, kMidSiluMul = 1, kMidSlices = 2 };
+
+// MT tiles of 16 rows of X; KC columns of X a chunk (a multiple of 64): KC / 64 steps between two barriers.
+template <int MT, int KC, int DEPTH, typename TC, int EPI>
+__global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf16* __restrict__ x,
+                                                                       const bf16* __restrict__ w,
+                                                                       const float* __restrict__ bias,
+                                                                       TC* __restrict__ c, float* __restrict__ parts,
+                                                                       int m, int n, int k, long ldx, long ldc,
+                                                                       int steps_per_slice) {
+  constexpr int SPC = KC / 64;                  // steps a chunk
+  constexpr int CPR = DEPTH / SPC;              // chunks the ring of W steps spans
+  static_assert(DEPTH % SPC == 0 && CPR >= 1, "the ring holds whole chunks");
+  constexpr int ROW = KC + 8;                   // an LDS row: 16 bytes past KC columns, so that the sixteen rows a
+                                                // quarter of a wavefront reads together lie in different banks
+  constexpr int ROWS = 16 * MT;
+  constexpr int PPR = KC / 8;                   // 16-byte pieces a row of a chunk
+  constexpr int PIECES = ROWS * PPR / (kMidWaves * kWave);   // pieces a thread stages
+  static_assert(ROWS * PPR % (kMidWaves * kWave) == 0, "a chunk is a whole number of pieces per thread");
+  extern __shared__ __align__(16) unsigned char mid_lds[];
+  bf16 (*xs)[ROWS][ROW] = reinterpret_cast<bf16 (*)[ROWS][ROW]>(mid_lds);   // two buffers
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
+  const int tile = blockIdx.x * kMidWaves + wave;
+  const bool n_ok = tile < tiles;
+  const bf16* wtile = w + (size_t)(n_ok ? tile : 0) * steps * 1024;
+  const int s_begin = blockIdx.y * steps_per_slice;
+  const int s_end = s_begin + steps_per_slice < steps ? s_begin + steps_per_slice : steps;
+  const int nchunks = (s_end - s_begin + SPC - 1) / SPC;
+
+  // What a thread stages of a chunk: piece p = tid + j * threads is columns 8 (p % PPR) .. + 7 of row p / PPR.
+  // A row past m reads row 0 and columns past k the row's first ones: memory that is there and finite (the
+  // columns meet zeros in the tile, the rows are never stored).
+  const bf16* src[PIECES];
+  int col[PIECES];
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int p = threadIdx.x + j * kMidWaves * kWave;
+    const int row = p / PPR;
+    col[j] = 8 * (p % PPR);
+    src[j] = x + (size_t)(row < m ? row : 0) * ldx;
+  }
+  bf16x8 staged[PIECES];
+  auto stage_load = [&](int chunk) {
+    const int k0 = (s_begin + chunk * SPC) * 64;
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int at = k0 + col[j];
+      staged[j] = *reinterpret_cast<const bf16x8*>(src[j] + (at + 8 <= k ? at : 0));
+    }
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int p = threadIdx.x + j * kMidWaves * kWave;
+      *reinterpret_cast<bf16x8*>(&xs[buf][p / PPR][col[j]]) = staged[j];
+    }
+  };
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // No load stands under a condition (a chunk or a step past the slice's end reads the last one again and is not
+  // used): the compiler then knows how many loads are in flight at every use and waits for no more than it must;
+  // behind a load that may or may not have been issued it would wait for all of them, the newest included.
+  MidFrag wbuf[DEPTH];
+  const int last = s_end - 1;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) wbuf[d] = mid_load_w(wtile, s_begin + d < s_end ? s_begin + d : last, lane);
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+  // X fragments of a step, all asked for from LDS before the step's first product
+  auto load_x = [&](int buf, int ss, bf16x8 (*xf)[2]) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const bf16* xr = &xs[buf][16 * t + r][64 * ss + 16 * g];
+      xf[t][0] = *reinterpret_cast<const bf16x8*>(xr);
+      xf[t][1] = *reinterpret_cast<const bf16x8*>(xr + 8);
+    }
+  };
+  for (int ch0 = 0; ch0 < nchunks; ch0 += CPR) {
+#pragma unroll
+    for (int u = 0; u < CPR; ++u) {
+      const int ch = ch0 + u;   // past the last chunk (the ring spans several): everything again, nothing counted
+      const int buf = ch & 1;
+      stage_load(ch + 1 < nchunks ? ch + 1 : nchunks - 1);
+      bf16x8 xf[2][MT][2];
+      load_x(buf, 0, xf[0]);
+#pragma unroll
+      for (int ss = 0; ss < SPC; ++ss) {
+        const int s = s_begin + ch * SPC + ss;
+        MidFrag wc = wbuf[u * SPC + ss];
+        // the step that takes this slot of the ring next; past the slice's end the last step again, never used
+        wbuf[u * SPC + ss] = mid_load_w(wtile, s + DEPTH < s_end ? s + DEPTH : last, lane);
+        if (ss + 1 < SPC) load_x(buf, ss + 1, xf[(ss + 1) & 1]);   // the next step's, under this step's products
+        if (s >= s_end) {   // a step past the slice's end counts nothing: zeros for W, and no branch around the products
+#pragma unroll
+          for (int i = 0; i < 8; ++i) wc.lo[i] = (bf16)0.f, wc.hi[i] = (bf16)0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.lo, xf[ss & 1][t][0], acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.hi, xf[ss & 1][t][1], acc[t], 0, 0, 0);
+        }
+      }
+      stage_store(buf ^ 1);
+      __syncthreads();
+    }
+  }
+  if (!n_ok) return;
+  // lane (g, r) holds four consecutive n of token 16 t + r
+  const int nb = 16 * tile + 4 * g;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int mi = 16 * t + r;
+    if (mi >= m) continue;
+    if (EPI == kMidSlices) {
+      float* dst = parts + ((size_t)blockIdx.y * m + mi) * n + nb;
+      if (nb + 3 < n && n % 4 == 0) {
+        float4 v{acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        if (bias && blockIdx.y == 0) v.x += bias[nb], v.y += bias[nb + 1], v.z += bias[nb + 2], v.w += bias[nb + 3];
+        *reinterpret_cast<float4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nb + i < n) dst[i] = acc[t][i] + (bias && blockIdx.y == 0 ? bias[nb + i] : 0.f);
+      }
+    } else if (EPI == kMidSiluMul) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int nn = nb + 2 * j;
+        if (nn + 1 < n) {
+          const float gate = acc[t][2 * j], up = acc[t][2 * j + 1];
+          c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate / (1.0f + expf(-gate)) * up);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (nb + i < n) {
+          float v = acc[t][i];
+          if (bias) v += bias[nb + i];
+          c[(size_t)mi * ldc + nb + i] = from_f32<TC>(v);
+        }
+      }
+    }
+  }
+}
+
+// out[row, col] = sum over the slices, in their order, of parts[slice, row, col]
+template <typename T>
+__global__ void sum_slices_kernel(const float* __restrict__ parts, T* __restrict__ out, int slices, size_t total) {
+  const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= total) return;
+  if (i + 3 < total) {
+    float4 s = *reinterpret_cast<const float4*>(parts + i);
+    for (int p = 1; p < slices; ++p) {
+      const float4 v = *reinterpret_cast<const float4*>(parts + (size_t)p * total + i);
+      s.x += v.x, s.y += v.y, s.z += v.z, s.w += v.w;
+    }
+    out[i] = from_f32<T>(s.x), out[i + 1] = from_f32<T>(s.y), out[i + 2] = from_f32<T>(s.z), out[i + 3] = from_f32<T>(s.w);
+  } else {
+    for (size_t e = i; e < total; ++e) {
+      float s = parts[e];
+      for (int p = 1; p < slices; ++p) s += parts[(size_t)p * total + e];
+      out[e] = from_f32<T>(s);
+    }
+  }
+}
+
+template <int MT, int KC, int DEPTH, typename TC, int EPI>
+int launch_mid(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n, int k,
+               long ldx, long ldc, int slices) {
+  const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
+  const int sps = (steps + slices - 1) / slices;
+  constexpr size_t lds = 2 * (size_t)(16 * MT) * (KC + 8) * sizeof(bf16);
+  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mid_kernel<MT, KC, DEPTH, TC, EPI>),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (allowed != hipSuccess) return pa::fail("gemm_mid: %zu bytes of LDS refused: %s", lds, hipGetErrorString(allowed));
+  dim3 grid((tiles + kMidWaves - 1) / kMidWaves, (steps + sps - 1) / sps);
+  hipLaunchKernelGGL((gemm_mid_kernel<MT, KC, DEPTH, TC, EPI>), grid, dim3(kMidWaves * kWave), lds, st, (const bf16*)x,
+                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps);
+  return check_launch("gemm_mid");
+}
+
+template <typename TC, int EPI>
+int launch_mid_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n,
+                  int k, long ldx, long ldc, int slices) {
+#define PA_MID(MT, KC, D) return launch_mid<MT, KC, D, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices)
+  // chunks of 256 columns and a ring of four steps up to 64 rows; 128 columns beyond (LDS holds two chunks);
+  // measured over chunk sizes and ring depths at the shapes of a 4B model: within a microsecond of one another
+  switch ((m + 15) / 16) {
+    case 1: PA_MID(1, 256, 4);
+    case 2: PA_MID(2, 256, 4);
+    case 3: PA_MID(3, 256, 4);   // 48 rows x 32 pieces = 1536 = 6 a thread
+    case 4: PA_MID(4, 256, 4);
+    case 5:
+    case 6: PA_MID(6, 128, 4);   // 96 rows x 16 pieces = 1536
+    default: PA_MID(8, 128, 4);
+  }
+#undef PA_MID
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+// How many slices of K pa_gemm_mid cuts a product into when its reader takes slices: as many as give every
+// compute unit a workgroup or two, each slice at least eight steps of 64 columns, eight at most.  Follows the
+// weight's shape alone.
+extern "C" int pa_gemm_mid_slices(int n, int k) {
+  if (n <= 0 || k <= 0) return 1;
+  const int blocks = ((n + 15) / 16 + kMidWaves - 1) / kMidWaves, steps = (k + 63) / 64;
+  int s = 1;
+  while (s < 8 && blocks * s < 256 && steps / (2 * s) >= 8) s *= 2;
+  return s;
+}
+
+// Floats of `parts` a product of m rows cut into `slices` needs.
+extern "C" long pa_gemm_mid_parts(int m, int n, int slices) { return slices <= 1 ? 0 : (long)slices * m * n; }
+
+// C[m, n] = X[m, k] W^T for m <= 128 from the weight in tiles.  slices 1: epilogue 0 writes C (+ bias) as
+// out_dtype (0 float32, 1 bfloat16), epilogue 1 C[m, n/2] = silu(gate) * up.  slices > 1 (epilogue 0 only):
+// nothing is written to C; parts [slices, m, n] receives each slice's 32-bit sums (the bias in the first).
+extern "C" int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias,
+                           void* c, float* parts, int m, int n, int k, long ldx, long ldc, int slices) {
+  if (m == 0 || n == 0) return 0;
+  PA_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_mid: bad sizes m=%d n=%d k=%d", m, n, k);
+  PA_REQUIRE(m <= kMidMaxM, "gemm_mid: %d rows exceed %d", m, kMidMaxM);
+  PA_REQUIRE(k % 8 == 0 && ldx % 8 == 0 && ldx >= k, "gemm_mid: k=%d and the row stride %ld must be multiples of 8, the stride at least k",
+             k, ldx);
+  const int steps = (k + 63) / 64;
+  PA_REQUIRE(slices >= 1 && slices <= steps && slices <= 64, "gemm_mid: %d slices of %d steps", slices, steps);
+  {
+    const int sps = (steps + slices - 1) / slices;   // every slice must get a step, or its part would stay unwritten
+    PA_REQUIRE((steps + sps - 1) / sps == slices, "gemm_mid: %d steps do not cut into %d slices of %d", steps, slices, sps);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (slices > 1) {
+    PA_REQUIRE(epilogue == kMidPlain && parts, "gemm_mid: a product in slices has no epilogue and needs `parts`");
+    return launch_mid_mt<float, kMidSlices>(st, x, w, bias, nullptr, parts, m, n, k, ldx, ldc, slices);
+  }
+  PA_REQUIRE(c, "gemm_mid: no output");
+  PA_REQUIRE(epilogue == kMidPlain || (epilogue == kMidSiluMul && n % 2 == 0 && !bias),
+             "gemm_mid: the SiLU*up epilogue needs an even n and no bias");
+  PA_REQUIRE(ldc >= (epilogue == kMidSiluMul ? n / 2 : n), "gemm_mid: output row stride %ld is too small", ldc);
+  if (epilogue == kMidPlain && out_dtype == kBF16)
+    return launch_mid_mt<bf16, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1);
+  if (epilogue == kMidPlain && out_dtype == kF32)
+    return launch_mid_mt<float, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1);
+  if (epilogue == kMidSiluMul && out_dtype == kBF16)
+    return launch_mid_mt<bf16, kMidSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1);
+  return pa::fail("gemm_mid: unsupported output type %d with epilogue %d", out_dtype, epilogue);
+}
+
+// out[i] = sum of parts[p, i] over p in order; out_dtype 0 float32, 1 bfloat16; total = rows * columns.
+extern "C" int pa_sum_slices(void* stream, int out_dtype, const float* parts, void* out, int slices, long total) {
+  if (total == 0) return 0;
+  PA_REQUIRE(slices >= 1 && total > 0 && parts && out, "sum_slices: bad operands");
+  const unsigned blocks = (unsigned)((total / 4 + 1 + 255) / 256);
+  if (out_dtype == kBF16) {
+    hipLaunchKernelGGL(sum_slices_kernel<bf16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, parts, (bf16*)out, slices,
+                       (size_t)total);
+  } else if (out_dtype == kF32) {
+    hipLaunchKernelGGL(sum_slices_kernel<float>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, parts, (float*)out,
+                       slices, (size_t)total);
+  } else {
+    return pa::fail("sum_slices: unknown element type code %d", out_dtype);
+  }
+  return check_launch("sum_slices");
+}

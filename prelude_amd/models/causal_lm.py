@@ -136,5 +136,8 @@ class CausalLM:
                                                             write_cache=r.reads_cache_of is None)
         if step.want_rows.shape[0] == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=hidden.device)
+        if not self.final_norm.TAKES_SLICE_SUMS:
+            from ..ops import kernels as K
+            hidden = K.as_tensor(hidden)
         normed = self.final_norm.forward_rows(hidden, residual, step.want_rows)
         return self.head.forward(normed)

@@ -106,6 +106,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optiona
     residual tensor receives the sum.  With ``rows`` (int32 [R]) only those
     rows are normed, into a compact [R, H] output, and the residual is read only.
     """
+    if isinstance(x, SliceSums):
+        return _rmsnorm_slices(x, weight, eps, residual, rows)
     _dev(x, weight, residual, rows)
     _f32(weight, "norm weight")
     if x.dim() != 2 or weight.shape != (x.shape[1],):
@@ -119,6 +121,27 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optiona
     out = torch.empty((n, x.shape[1]), dtype=x.dtype, device=x.device)
     check(kernels().pa_rmsnorm(_stream(), _code(x), _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), n,
                                x.shape[1], float(eps)))
+    return out
+
+
+def _rmsnorm_slices(x, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor],
+                    rows: Optional[torch.Tensor]) -> torch.Tensor:
+    """``rmsnorm`` of a product that comes as partial sums: the slices are added in order as they are loaded."""
+    parts = x.parts
+    _dev(parts, weight, residual, rows)
+    _f32(weight, "norm weight")
+    s, m, h = parts.shape
+    if weight.shape != (h,) or h % 4:
+        raise NativeError(f"rmsnorm: slices {tuple(parts.shape)} / weight {tuple(weight.shape)}")
+    if residual is not None and (tuple(residual.shape) != (m, h) or residual.dtype != x.dtype):
+        raise NativeError(f"rmsnorm: residual {tuple(residual.shape)} {residual.dtype} does not match the product")
+    n = m
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.shape[0]
+    out = torch.empty((n, h), dtype=x.dtype, device=parts.device)
+    check(kernels().pa_rmsnorm_slices(_stream(), _CODES[x.dtype], _ptr(parts), s, m * h, _ptr(residual), _ptr(weight),
+                                      _ptr(out), _ptr(rows), n, h, float(eps)))
     return out
 
 
@@ -326,6 +349,71 @@ def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     return out
 
 
+class SliceSums:
+    """A product left as 32-bit partial sums of slices of its inner size, [slices, M, N]: what ``gemm_mid`` gives
+    when its reader can add the slices itself (``rmsnorm`` does, as it loads them).  ``materialize()`` adds them
+    for any other reader."""
+
+    def __init__(self, parts: torch.Tensor, dtype: torch.dtype):
+        self.parts = parts
+        self.shape = tuple(parts.shape[1:])
+        self.dtype, self.device = dtype, parts.device
+
+    def materialize(self) -> torch.Tensor:
+        s, m, n = self.parts.shape
+        out = torch.empty((m, n), dtype=self.dtype, device=self.device)
+        check(kernels().pa_sum_slices(_stream(), _CODES[self.dtype], _ptr(self.parts), _ptr(out), s, m * n))
+        return out
+
+
+GEMM_MID_MAX_ROWS = 128
+# Where ``linear`` takes the product with X staged in LDS (measured at the shapes of a 4B model, 17 to 128 rows):
+# cut into slices, for a reader that adds them, where the weight is narrow enough to be cut into 8 -- [2560, 4096]
+# at 64 rows 10.9 against the library's 14.4 us, [2560, 9728] 18 against 27; and uncut for very wide weights with
+# 32-bit output (the head: 175 us at 64 rows where the library takes 176 and a conversion pass of 20)
+MID_MIN_SLICES = 8
+MID_WIDE_ROWS = 65536
+MID_WIDE_MAX_M = 64
+MID_PRODUCTS = True    # ``set_mid_products``: off sends these products where they went without this kernel (measurements)
+
+
+def set_mid_products(on: bool) -> None:
+    global MID_PRODUCTS
+    MID_PRODUCTS = bool(on)
+
+
+def gemm_mid_slices(n: int, k: int) -> int:
+    """Into how many slices of its inner size ``gemm_mid`` cuts an [n, k] weight for a reader that adds slices."""
+    return int(kernels().pa_gemm_mid_slices(int(n), int(k)))
+
+
+def gemm_mid(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = None,
+             out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False, slices: int = 1):
+    """x [M <= 128, K] @ w[N, K]^T from the weight in tiles, X staged through LDS; with ``slices`` > 1 the result
+    is a ``SliceSums`` (one 32-bit partial sum per slice of K) instead of a tensor."""
+    if not isinstance(w, TiledWeight):
+        raise NativeError("gemm_mid takes the weight in tiles (pack_tiles)")
+    _dev(x, w.data, bias)
+    _f32(bias, "bias")
+    if x.dim() != 2 or x.shape[1] != w.k or x.dtype != torch.bfloat16:
+        raise NativeError(f"gemm_mid: x {tuple(x.shape)} {x.dtype} / w {w.shape}")
+    m, k = x.shape
+    n = w.n
+    out_dtype = out_dtype or torch.bfloat16
+    if bias is not None and bias.shape != (n,):
+        raise NativeError(f"gemm_mid: bias {tuple(bias.shape)} is not [{n}]")
+    if slices > 1:
+        parts = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+        check(kernels().pa_gemm_mid(_stream(), _CODES[out_dtype], 0, _ptr(x), _ptr(w.data), _ptr(bias), None, _ptr(parts),
+                                    m, n, k, k, n, slices))
+        return SliceSums(parts, out_dtype)
+    cols = n // 2 if silu_mul_epilogue else n
+    out = torch.empty((m, cols), dtype=out_dtype, device=x.device)
+    check(kernels().pa_gemm_mid(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w.data),
+                                _ptr(bias), _ptr(out), None, m, n, k, k, cols, 1))
+    return out
+
+
 LIBRARY_WORKSPACE_BYTES = 76 << 20   # what the library's stream-K kernels may use for partial sums
 _library_workspaces: dict = {}
 
@@ -352,10 +440,14 @@ def gemm_library(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
-           out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+           out_dtype: Optional[torch.dtype] = None, slices_ok: bool = False):
     """y = x W^T (+ b), W [out, in] as a tensor or a ``LinearWeight``.  float32: our own true 32-bit product.
     bfloat16: few rows our weight-streaming kernel (from the tiled copy if the weight has one), above that the
-    library product; 32-bit accumulation in both."""
+    library product or, for the shapes it suits, the product with X staged in LDS; 32-bit accumulation in all.
+
+    ``slices_ok``: the caller's reader adds slices itself (``rmsnorm`` does): a narrow weight at 17 to 128 rows
+    then comes back as ``SliceSums`` (the product cut along its inner size, a 32-bit partial sum per slice)
+    instead of a tensor."""
     tiles = None
     if isinstance(w, LinearWeight):
         w, tiles = w.rows, w.tiles
@@ -367,6 +459,14 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     m, k = x.shape
     if m <= SKINNY_MAX_ROWS and k % 8 == 0:
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
+    if MID_PRODUCTS and tiles is not None and k % 8 == 0 and m <= GEMM_MID_MAX_ROWS:
+        n = w.shape[0]
+        if slices_ok and n % 4 == 0 and out_dtype in (None, torch.bfloat16):
+            s = gemm_mid_slices(n, k)
+            if s >= MID_MIN_SLICES:
+                return gemm_mid(x, tiles, bias, slices=s)
+        if n >= MID_WIDE_ROWS and m <= MID_WIDE_MAX_M:
+            return gemm_mid(x, tiles, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
     if k % 8:
@@ -379,6 +479,11 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     if out_dtype is not None and out_dtype != y.dtype:
         y = to_f32(y)
     return y
+
+
+def as_tensor(x):
+    """A product that may have come back as ``SliceSums``, as a tensor."""
+    return x.materialize() if isinstance(x, SliceSums) else x
 
 
 def set_skinny_max_rows(n: int) -> None:

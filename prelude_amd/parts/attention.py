@@ -93,7 +93,7 @@ class GQAAttention(Mixer):
             o = K.attention_decode_fused(qkv, self.q_norm, self.k_norm, cos, sin, g.slots, self.norm_eps,
                                          cache.k, cache.v, g.block_table, step.decode_seqs, step.cu_q, step.context_lens,
                                          nh, step.max_decode_context, self.window, self.scale, every_seq=True)
-            return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o)
+            return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)
         if write_cache:
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
             q = K.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, cos, sin, step.positions, g.slots, cache.k, cache.v,
@@ -104,4 +104,4 @@ class GQAAttention(Mixer):
             q = K.qknorm_rope_kv(qx, self.q_norm, None, cos, sin, step.positions, None, None, None, nh, 0, hd,
                                  self.rotary_dim, self.norm_eps)
         o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale)
-        return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o)
+        return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)

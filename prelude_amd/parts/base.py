@@ -9,6 +9,8 @@ Categories and the interface each must have:
 
 ``norm``      ``forward(x)``, ``forward_residual(x, residual) -> (residual, normed)``,
               ``forward_rows(x, residual, rows)``
+``mixer``/``ffn`` may return their last product as ``ops.kernels.SliceSums`` (``linear(..., slices_ok=True)``):
+              only a norm reads it, and one that says ``TAKES_SLICE_SUMS`` adds the slices itself
 ``position``  ``prepare(device)``; what it offers (tables) is between it and the mixers that name it
 ``mixer``     ``cache_spec()`` -> ``KVCacheSpec`` | ``StateSpec`` | ``None``;
               ``forward(x, step, cache, write_cache=True)``
@@ -94,6 +96,11 @@ class FeedForward(Part):
 
 
 class Norm(Part):
+    # True for a norm whose three methods also take a product that was left as partial sums of slices of its
+    # inner size (``ops.kernels.SliceSums``) in place of ``x``, adding the slices as it loads them; a block
+    # hands other norms the finished tensor.
+    TAKES_SLICE_SUMS = False
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

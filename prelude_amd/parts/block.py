@@ -7,6 +7,7 @@ crates/prelude-core/src/models/commons/linear.rs:471-488).
 """
 from __future__ import annotations
 
+from ..ops import kernels as K
 from .base import Block, register_part
 
 
@@ -18,8 +19,14 @@ class PreNormBlock(Block):
         self.input_norm, self.mixer, self.post_mixer_norm, self.ffn = input_norm, mixer, post_mixer_norm, ffn
 
     def forward(self, hidden, residual, step, cache, write_cache=True):
+        # a mixer's or feed-forward's last product may come as partial sums of slices (``K.SliceSums``): a norm
+        # that can adds them as it loads them, any other gets the finished tensor
+        if not self.input_norm.TAKES_SLICE_SUMS:
+            hidden = K.as_tensor(hidden)
         residual, h = self.input_norm.forward_residual(hidden, residual)
         h = self.mixer.forward(h, step, cache, write_cache)
+        if not self.post_mixer_norm.TAKES_SLICE_SUMS:
+            h = K.as_tensor(h)
         residual, h = self.post_mixer_norm.forward_residual(h, residual)
         h = self.ffn.forward(h)
         return h, residual

@@ -35,4 +35,4 @@ class GatedMLP(FeedForward):
         self.down = K.prepare_weight(tensors["down_proj.weight"])
 
     def forward(self, x):
-        return K.linear(K.linear_silu_mul(x, self.gate_up), self.down)
+        return K.linear(K.linear_silu_mul(x, self.gate_up), self.down, slices_ok=True)

@@ -17,6 +17,8 @@ from .base import NORM, Norm, TensorReq, register_part
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
+    TAKES_SLICE_SUMS = True
+
     def __init__(self, size: int, eps: float):
         self.size = int(size)
         self.eps = float(eps)
@@ -35,6 +37,7 @@ class RMSNorm(Norm):
         """First use in a model: residual None -> (x, norm(x)).  Afterwards the
         residual is updated in place with residual + x."""
         if residual is None:
+            x = K.as_tensor(x)
             return x, K.rmsnorm(x, self.weight, self.eps)
         out = K.rmsnorm(x, self.weight, self.eps, residual=residual)
         return residual, out

@@ -169,6 +169,68 @@ def test_gemm_skinny(gpu, m, n, k):
                   torch.bfloat16, bf16=1.25e-2)
 
 
+@pytest.mark.parametrize("m,n,k,slices", [(64, 2560, 4096, 8), (33, 331, 1000, 1), (128, 200, 4096, 4), (7, 2560, 9728, 8),
+                                          (17, 6144, 2560, 2), (100, 48, 520, 1), (48, 256, 1024, 2), (1, 64, 64, 1),
+                                          (80, 36, 72, 1), (96, 132, 1288, 2), (20, 2560, 4096, 8)])
+def test_gemm_mid(gpu, m, n, k, slices):
+    """The product with X staged in LDS (up to 128 rows, weight in tiles): whole, and cut into slices of the inner
+    size whose 32-bit partial sums the reader adds -- the residual add + RMSNorm as it loads them, or sum_slices."""
+    x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
+    ref = x.double() @ w.double().T
+    xd, bd = x.to(gpu), b.to(gpu)
+    tiles = K().pack_tiles(w.to(gpu))
+    full = K().gemm_mid(xd, tiles, out_dtype=torch.float32)
+    close(full, ref, torch.float32, f32=2e-5)
+    close(K().gemm_mid(xd, tiles), ref, torch.bfloat16)
+    close(K().gemm_mid(xd, tiles, bd, out_dtype=torch.float32), ref + b.double(), torch.float32, f32=2e-5)
+    # a row's result does not depend on how many rows there are
+    assert torch.equal(K().gemm_mid(xd[m - 1:].contiguous(), tiles, out_dtype=torch.float32)[0], full[m - 1])
+    if n % 2 == 0:
+        close(K().gemm_mid(xd, tiles, silu_mul_epilogue=True), pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
+    if slices > 1:
+        ss = K().gemm_mid(xd, tiles, bd, slices=slices)
+        assert isinstance(ss, K().SliceSums) and tuple(ss.parts.shape) == (slices, m, n) and ss.dtype == torch.bfloat16
+        whole = ss.parts.double().sum(0).cpu()
+        close(whole, ref + b.double(), torch.float32, f32=2e-5)
+        close(ss.materialize(), ref + b.double(), torch.bfloat16)
+        # the norm adds the slices itself: residual + product in 32-bit, the residual rounded once, the norm of the unrounded sum
+        weight, res = 1 + 0.1 * rnd(n, seed=3), rnd(m, n, dtype=torch.bfloat16, seed=4)
+        resd = res.to(gpu)
+        normed = K().rmsnorm(ss, weight.to(gpu), 1e-5, residual=resd)
+        total = whole + res.double()
+        close(resd, total, torch.bfloat16)
+        close(normed, pm.rms_norm(total, weight.double(), 1e-5), torch.bfloat16)
+        rows = torch.tensor([m - 1, 0], dtype=torch.int32)
+        picked = K().rmsnorm(ss, weight.to(gpu), 1e-5, residual=res.to(gpu), rows=rows.to(gpu))
+        close(picked, pm.rms_norm(total[rows.long()], weight.double(), 1e-5), torch.bfloat16)
+    # what lies behind X is not the product's to read: NaN there must not show
+    behind = torch.full((m + 8, k), float("nan"), dtype=torch.bfloat16, device=gpu)
+    behind[:m] = xd
+    got = K().gemm_mid(behind[:m], tiles, out_dtype=torch.float32)
+    assert bool(torch.isfinite(got).all()) and torch.equal(got, full)
+
+
+def test_gemm_mid_refuses_and_is_dispatched(gpu):
+    from prelude_amd._native import NativeError
+    w = rnd(2560, 4096, dtype=torch.bfloat16, seed=1, scale=0.05).to(gpu)
+    tiles = K().pack_tiles(w)
+    with pytest.raises(NativeError, match="exceed 128"):
+        K().gemm_mid(torch.zeros(129, 4096, dtype=torch.bfloat16, device=gpu), tiles)
+    with pytest.raises(NativeError, match="do not cut into"):
+        K().gemm_mid(torch.zeros(8, 4096, dtype=torch.bfloat16, device=gpu), tiles, slices=60)
+    with pytest.raises(NativeError, match="in tiles"):
+        K().gemm_mid(torch.zeros(8, 4096, dtype=torch.bfloat16, device=gpu), w)
+    # linear() hands a narrow weight at 17 to 128 rows to it in slices only when the caller's reader adds slices
+    lw = K().LinearWeight(w, tiles)
+    x = rnd(40, 4096, dtype=torch.bfloat16).to(gpu)
+    assert isinstance(K().linear(x, lw), torch.Tensor)
+    got = K().linear(x, lw, slices_ok=True)
+    assert isinstance(got, K().SliceSums) and got.parts.shape[0] == K().gemm_mid_slices(2560, 4096) == 8
+    close(K().as_tensor(got), x.double().cpu() @ w.double().cpu().T, torch.bfloat16)
+    assert isinstance(K().linear(x[:8].contiguous(), lw, slices_ok=True), torch.Tensor)      # few rows: the streaming kernel
+    assert isinstance(K().linear(x.float(), w.float(), slices_ok=True), torch.Tensor)      # 32-bit: the plain product
+
+
 @pytest.mark.parametrize("m,n,k", [(30, 24, 16), (4, 76, 24), (16, 48, 40), (1, 32, 8), (39, 2304, 24), (64, 40, 72)])
 def test_gemm_skinny_stays_inside_its_rows(gpu, m, n, k):
     """Rows shorter than a step of 64 columns, or ending inside one: what lies behind a row of X is not the
