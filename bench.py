@@ -13,7 +13,8 @@ the host prepares a step while the one before it runs, as the engine's
 generation loop does).
 One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is
 a 2,048-token prompt portion; ``roofline`` prices the decode step against HBM
-bandwidth; ``points`` holds batch 1 and 64.
+bandwidth; ``points`` holds batch 1 and 64 at the same context, batch 8 at a context of 32,768 tokens and the
+prefill of 8,192 tokens in one step (tokens a second each).
 """
 from __future__ import annotations
 
@@ -123,11 +124,11 @@ def time_decode(engine, batch, steps, warmup, vocab):
     return (time.perf_counter() - t0) / steps
 
 
-def decode_point(raw, dtype, batch, context, steps, warmup, layers_note):
+def decode_point(raw, dtype, batch, context, steps, warmup, layers_note, chunk=2048):
     import torch
     total = steps + warmup
-    eng = build_engine(raw, dtype, cache_tokens=batch * (context + 64))
-    prefill_requests(eng, batch, context - total, 2048, raw["vocab_size"], seed=batch)
+    eng = build_engine(raw, dtype, cache_tokens=batch * (context + 64), max_num_batched_tokens=max(8192, chunk))
+    prefill_requests(eng, batch, context - total, chunk, raw["vocab_size"], seed=batch)
     sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"])
     del eng
     release_memory()
@@ -138,7 +139,7 @@ def time_prefill(raw, dtype, tokens, reps):
     import numpy as np
     import torch
     from prelude_amd.engine import StepEntry
-    eng = build_engine(raw, dtype, cache_tokens=(reps + 2) * (tokens + 64))
+    eng = build_engine(raw, dtype, cache_tokens=(reps + 2) * (tokens + 64), max_num_batched_tokens=max(8192, tokens))
     rng = np.random.default_rng(7)
     best = None
     for r in range(reps + 1):
@@ -318,6 +319,12 @@ def main() -> int:
         for b in (1, 64):
             s = decode_point(raw, args.dtype, b, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), None)
             pts[f"decode_b{b}"] = round(b / s, 2)
+        if args.context == 4096 and args.batch == 8:
+            # further from the default point: a long context (the cache is 3.6 times the weights there) and a long portion
+            s = decode_point(raw, args.dtype, 8, 32768, max(8, args.steps // 4), max(2, args.warmup // 4), None, chunk=8192)
+            pts["decode_b8_ctx32768"] = round(8 / s, 2)
+            if not args.no_prefill:
+                pts["prefill_8192"] = round(8192 / time_prefill(raw, args.dtype, 8192, reps=2), 1)
         out["points"] = pts
     print(json.dumps(out), flush=True)
     return 0

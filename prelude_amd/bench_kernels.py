@@ -1,6 +1,6 @@
 """Times single kernels against their rooflines on one MI355X.
 
-    python -m prelude_amd.bench_kernels [gemm] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
+    python -m prelude_amd.bench_kernels [stream] [gemm] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
 
 Each line gives the kernel's time (device events around repeated launches,
 operands rotated over copies larger than the caches where the kernel streams
@@ -49,6 +49,18 @@ def line(name: str, us: float, nbytes: float = 0.0, flops: float = 0.0) -> None:
         rate = flops / us * 1e6
         parts.append(f"{rate / 1e12:8.1f} TFLOP/s  {rate / MFMA_PEAK:5.2f} of MFMA peak")
     print("  ".join(parts), flush=True)
+
+
+def bench_stream(dev, shape) -> None:
+    """The rate a kernel that does nothing but read reaches over 8 GB: what the published 8 TB/s comes to here."""
+    from ._native import check, kernels
+    nbytes = 8 << 30
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    buf.zero_()
+    for blocks in (1024, 2048, 4096, 8192, 16384):
+        out = torch.zeros(blocks, dtype=torch.int32, device=dev)
+        us = timeit(lambda i: check(kernels().pa_stream_read(K._stream(), buf.data_ptr(), nbytes, out.data_ptr(), blocks)), 1, iters=10)
+        line(f"read 8 GB, {blocks} workgroups of 256 threads", us, nbytes=nbytes)
 
 
 def bench_gemm(dev, shape) -> None:
@@ -145,7 +157,7 @@ def bench_sampling(dev, shape) -> None:
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
-    ap.add_argument("what", nargs="*", help="gemm, decode, prefill, elementwise, sampling (default: all)")
+    ap.add_argument("what", nargs="*", help="stream, gemm, decode, prefill, elementwise, sampling (default: all)")
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -153,11 +165,11 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     shape = SHAPES[args.shape]
-    todo = args.what or ["gemm", "decode", "prefill", "elementwise", "sampling"]
+    todo = args.what or ["stream", "gemm", "decode", "prefill", "elementwise", "sampling"]
     print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
           f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
     for name in todo:
-        {"gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
+        {"stream": bench_stream, "gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
          "sampling": bench_sampling}[name](dev, shape)
     return 0
 

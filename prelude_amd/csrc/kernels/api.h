@@ -11,6 +11,9 @@ const char* pa_last_error();
 int pa_device_arch(char* out, int cap);
 int pa_num_compute_units();
 
+// A kernel that only reads: `bytes` (a multiple of 16) from src by `blocks` workgroups; out holds a word per
+// workgroup.  For measuring the rate at which this device streams memory.
+int pa_stream_read(void* stream, const void* src, long bytes, void* out, int blocks);
 // out[t, :] = table[ids[t], :]
 int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, void* out, int tokens, int hidden,
                     int vocab);

@@ -58,6 +58,28 @@ __global__ void zero_fresh_rows_kernel(uint32_t* __restrict__ data, long row_wor
   for (long w = (long)blockIdx.y * blockDim.x + threadIdx.x; w < row_words; w += (long)gridDim.y * blockDim.x) row[w] = 0u;
 }
 
+// ---- how fast memory can be read at all ------------------------------------
+// Every thread reads 16-byte pieces a whole grid apart, eight in flight, and folds them into one word; a block
+// writes one word.  Nothing else happens: the rate this reaches is what a kernel that streams memory can be held to.
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ src, size_t pieces,
+                                                         unsigned* __restrict__ out) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned acc = 0;
+  for (; i + 7 * stride < pieces; i += 8 * stride) {
+    uint4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = src[i + j * stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+  }
+  for (; i < pieces; i += stride) {
+    const uint4 v = src[i];
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x9e3779b9u) out[blockIdx.x] = acc;   // (almost) never: keeps the loads from being dropped
+}
+
 // ---- RMSNorm, optionally fused with the residual add --------------------
 //   s = x (+ residual)                         in 32-bit
 //   residual <- round(s)                       (only when `residual` is given and `rows` is not)
@@ -256,6 +278,14 @@ extern "C" int pa_carry_tokens(void* stream, const int* sampled, const int* src,
   hipLaunchKernelGGL(carry_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, sampled, src, dst,
                      ids, n, sampled_rows, tokens);
   return check_launch("carry_tokens");
+}
+
+// Reads `bytes` (a multiple of 16) from src with `blocks` workgroups of 256 threads; out: one word a workgroup.
+extern "C" int pa_stream_read(void* stream, const void* src, long bytes, void* out, int blocks) {
+  PA_REQUIRE(src && out && bytes > 0 && bytes % 16 == 0 && blocks > 0, "stream_read: bad operands");
+  hipLaunchKernelGGL(stream_read_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
+                     (size_t)(bytes / 16), (unsigned*)out);
+  return check_launch("stream_read");
 }
 
 extern "C" int pa_zero_fresh_rows(void* stream, void* data, long row_bytes, const int* slots, const int* fresh, int nseq,
