@@ -53,7 +53,7 @@ _KERNEL_API = {
     "pa_pack_tiles": (I, [P, P, P, I, I]),
     "pa_gemm_mid_slices": (I, [I, I]),
     "pa_gemm_mid_parts": (c_long, [I, I, I]),
-    "pa_gemm_mid": (I, [P, I, I, P, P, P, P, P, I, I, I, c_long, c_long, I]),
+    "pa_gemm_mid": (I, [P, I, I, P, P, P, P, P, I, I, I, c_long, c_long, I, I]),
     "pa_sum_slices": (I, [P, I, P, P, I, c_long]),
     "pa_rmsnorm_slices": (I, [P, I, P, I, c_long, P, P, P, P, I, I, F]),
     "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),

@@ -59,15 +59,16 @@ int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, cons
 // tiled 1: w is the weight as pa_pack_tiles lays it out.
 int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
                    int m, int n, int k, long ldx, long ldc, int tiled);
-// C[m, n] = X[m, k] W[n, k]^T for m <= 128 from the weight in tiles, X staged through LDS and W streamed by four
-// wavefronts a workgroup (64 rows of W).  slices 1: as pa_gemm_skinny (epilogue 0 (+ bias) / 1 SiLU * up).
+// C[m, n] = X[m, k] W[n, k]^T for m <= 128 from the weight in tiles, X staged through LDS and W streamed by
+// `waves` wavefronts a workgroup, 16 rows of W each (3, 4, 5, 6 or 8; 0: chosen from the weight's shape; the same
+// bits at every number).  slices 1: as pa_gemm_skinny (epilogue 0 (+ bias) / 1 SiLU * up).
 // slices > 1 (epilogue 0): the inner size is cut into that many slices, each left as 32-bit sums in
 // parts [slices, m, n] (pa_gemm_mid_parts floats; the bias in the first) for the reader to add in order, and c is
 // not written.  pa_gemm_mid_slices: the number of slices that suits an [n, k] weight.
 int pa_gemm_mid_slices(int n, int k);
 long pa_gemm_mid_parts(int m, int n, int slices);
 int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
-                float* parts, int m, int n, int k, long ldx, long ldc, int slices);
+                float* parts, int m, int n, int k, long ldx, long ldc, int slices, int waves);
 // out[i] = parts[0, i] + parts[1, i] + ..; out_dtype 0 = float32, 1 = bfloat16; total = rows * columns.
 int pa_sum_slices(void* stream, int out_dtype, const float* parts, void* out, int slices, long total);
 // out[tile][step][half][g][r][8] = w[16 tile + r][64 step + 16 g + 8 half ..], zero-padded: ceil(n/16) * ceil(k/64) * 1024 elements.

@@ -4,12 +4,13 @@
 // With more than a few rows the weight-streaming kernel of gemm_skinny.hip reads X as often as it has
 // workgroups: every workgroup owns 16 rows of W and all of K, so a [2560, 9728] weight at 64 rows moves four
 // times as many bytes of X through the caches as it streams of W, and a wavefront that holds the sums of 64
-// rows has few loads in flight.  Here a workgroup owns 64 rows of W (four wavefronts, a tile of 16 rows each)
-// and a slice of K.  X goes through LDS: the slice's columns are staged once per workgroup, a chunk of KC
-// columns ahead of the products, and every wavefront takes its MFMA operands from there; W goes from memory
-// straight into registers, each wavefront streaming its own tile's 2 KB steps with a ring of KC / 64 of them in
-// flight.  X is then read once per 64 rows of W whatever the number of slices, and a narrow weight still gives
-// every compute unit a workgroup: [2560, 4096] is 40 blocks of rows times 8 slices of K.
+// rows has few loads in flight.  Here a workgroup owns 48 to 128 rows of W (three to eight wavefronts, a tile of
+// 16 rows each; the number that leaves the fewest compute units idle for the weight's shape) and a slice of K.
+// X goes through LDS: the slice's columns are staged once per workgroup, in chunks of KC columns two chunks
+// ahead of the products, and every wavefront takes its MFMA operands from there; W goes from memory straight
+// into registers, each wavefront streaming its own tile's 2 KB steps with a ring of four of them in flight.
+// X is then read once per workgroup whatever the number of slices, and a narrow weight still gives every
+// compute unit a workgroup: [2560, 4096] is 32 blocks of rows times 8 slices of K.
 //
 // A product cut into slices leaves one 32-bit partial sum per slice, [slices, M, N], and no workgroup waits for
 // another: whoever reads the result adds the slices in order (the residual add + RMSNorm kernel does, as it
@@ -25,8 +26,8 @@
 
 namespace pa {
 
-constexpr int kMidWaves = 4;           // wavefronts a workgroup: 64 rows of W
 constexpr int kMidMaxM = 128;
+constexpr int kMidMaxWaves = 8;
 
 struct MidFrag {
   bf16x8 lo, hi;
@@ -43,9 +44,10 @@ __device__ __forceinline__ MidFrag mid_load_w(const bf16* tile, int step, int la
 
 enum MidEpilogue : int { kMidPlain = 0, kMidSiluMul = 1, kMidSlices = 2 };
 
-// MT tiles of 16 rows of X; KC columns of X a chunk (a multiple of 64): KC / 64 steps between two barriers.
-template <int MT, int KC, int DEPTH, typename TC, int EPI>
-__global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf16* __restrict__ x,
+// MT tiles of 16 rows of X; KC columns of X a chunk (a multiple of 64): KC / 64 steps between two barriers; WN
+// wavefronts a workgroup, a tile of 16 rows of W each.
+template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI>
+__global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __restrict__ x,
                                                                        const bf16* __restrict__ w,
                                                                        const float* __restrict__ bias,
                                                                        TC* __restrict__ c, float* __restrict__ parts,
@@ -58,15 +60,16 @@ __global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf1
                                                 // quarter of a wavefront reads together lie in different banks
   constexpr int ROWS = 16 * MT;
   constexpr int PPR = KC / 8;                   // 16-byte pieces a row of a chunk
-  constexpr int PIECES = ROWS * PPR / (kMidWaves * kWave);   // pieces a thread stages
-  static_assert(ROWS * PPR % (kMidWaves * kWave) == 0, "a chunk is a whole number of pieces per thread");
+  constexpr int THREADS = WN * kWave;
+  constexpr int PIECES = (ROWS * PPR + THREADS - 1) / THREADS;   // pieces a thread stages
+  constexpr bool EVEN = ROWS * PPR % THREADS == 0;               // else the last piece of the later threads is none
   extern __shared__ __align__(16) unsigned char mid_lds[];
   bf16 (*xs)[ROWS][ROW] = reinterpret_cast<bf16 (*)[ROWS][ROW]>(mid_lds);   // two buffers
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
-  const int tile = blockIdx.x * kMidWaves + wave;
+  const int tile = blockIdx.x * WN + wave;
   const bool n_ok = tile < tiles;
   const bf16* wtile = w + (size_t)(n_ok ? tile : 0) * steps * 1024;
   const int s_begin = blockIdx.y * steps_per_slice;
@@ -80,25 +83,32 @@ __global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf1
   int col[PIECES];
 #pragma unroll
   for (int j = 0; j < PIECES; ++j) {
-    const int p = threadIdx.x + j * kMidWaves * kWave;
+    const int p = threadIdx.x + j * THREADS;
     const int row = p / PPR;
     col[j] = 8 * (p % PPR);
-    src[j] = x + (size_t)(row < m ? row : 0) * ldx;
+    src[j] = x + (size_t)(row < m ? row : 0) * ldx;   // a piece past the chunk reads row 0 and is not stored
   }
+  // The pieces are dealt out over a chunk's SPC steps (group q: pieces [q * PIECES / SPC, (q + 1) * PIECES / SPC)):
+  // at step q of chunk c a thread stores group q, which it loaded a chunk ago and which belongs to chunk c + 1, and
+  // loads group q of chunk c + 2 in its place.  A wait for staged pieces then never asks for more of the weight's
+  // loads than the step at hand needs anyway (loads come back in the order they were asked for: one wait for a
+  // whole chunk's pieces at the chunk's end would drain the ring of weight steps each time).
   bf16x8 staged[PIECES];
-  auto stage_load = [&](int chunk) {
+  auto stage_load = [&](int chunk, int q0, int q1) {
     const int k0 = (s_begin + chunk * SPC) * 64;
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
+      if (j < q0 * PIECES / SPC || j >= q1 * PIECES / SPC) continue;
       const int at = k0 + col[j];
       staged[j] = *reinterpret_cast<const bf16x8*>(src[j] + (at + 8 <= k ? at : 0));
     }
   };
-  auto stage_store = [&](int buf) {
+  auto stage_store = [&](int buf, int q0, int q1) {
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
-      const int p = threadIdx.x + j * kMidWaves * kWave;
-      *reinterpret_cast<bf16x8*>(&xs[buf][p / PPR][col[j]]) = staged[j];
+      if (j < q0 * PIECES / SPC || j >= q1 * PIECES / SPC) continue;
+      const int p = threadIdx.x + j * THREADS;
+      if (EVEN || j + 1 < PIECES || p < ROWS * PPR) *reinterpret_cast<bf16x8*>(&xs[buf][p / PPR][col[j]]) = staged[j];
     }
   };
 
@@ -113,8 +123,9 @@ __global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf1
   const int last = s_end - 1;
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) wbuf[d] = mid_load_w(wtile, s_begin + d < s_end ? s_begin + d : last, lane);
-  stage_load(0);
-  stage_store(0);
+  stage_load(0, 0, SPC);
+  stage_store(0, 0, SPC);
+  stage_load(nchunks > 1 ? 1 : 0, 0, SPC);
   __syncthreads();
   // X fragments of a step, all asked for from LDS before the step's first product
   auto load_x = [&](int buf, int ss, bf16x8 (*xf)[2]) {
@@ -130,7 +141,7 @@ __global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf1
     for (int u = 0; u < CPR; ++u) {
       const int ch = ch0 + u;   // past the last chunk (the ring spans several): everything again, nothing counted
       const int buf = ch & 1;
-      stage_load(ch + 1 < nchunks ? ch + 1 : nchunks - 1);
+      const int ahead = ch + 2 < nchunks ? ch + 2 : nchunks - 1;
       bf16x8 xf[2][MT][2];
       load_x(buf, 0, xf[0]);
 #pragma unroll
@@ -139,6 +150,8 @@ __global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf1
         MidFrag wc = wbuf[u * SPC + ss];
         // the step that takes this slot of the ring next; past the slice's end the last step again, never used
         wbuf[u * SPC + ss] = mid_load_w(wtile, s + DEPTH < s_end ? s + DEPTH : last, lane);
+        stage_store(buf ^ 1, ss, ss + 1);
+        stage_load(ahead, ss, ss + 1);
         if (ss + 1 < SPC) load_x(buf, ss + 1, xf[(ss + 1) & 1]);   // the next step's, under this step's products
         if (s >= s_end) {   // a step past the slice's end counts nothing: zeros for W, and no branch around the products
 #pragma unroll
@@ -150,7 +163,6 @@ __global__ __launch_bounds__(kMidWaves* kWave, 2) void gemm_mid_kernel(const bf1
           acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc.hi, xf[ss & 1][t][1], acc[t], 0, 0, 0);
         }
       }
-      stage_store(buf ^ 1);
       __syncthreads();
     }
   }
@@ -215,37 +227,67 @@ __global__ void sum_slices_kernel(const float* __restrict__ parts, T* __restrict
   }
 }
 
-template <int MT, int KC, int DEPTH, typename TC, int EPI>
+template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI>
 int launch_mid(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n, int k,
                long ldx, long ldc, int slices) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
   const int sps = (steps + slices - 1) / slices;
   constexpr size_t lds = 2 * (size_t)(16 * MT) * (KC + 8) * sizeof(bf16);
-  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mid_kernel<MT, KC, DEPTH, TC, EPI>),
+  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI>),
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (allowed != hipSuccess) return pa::fail("gemm_mid: %zu bytes of LDS refused: %s", lds, hipGetErrorString(allowed));
-  dim3 grid((tiles + kMidWaves - 1) / kMidWaves, (steps + sps - 1) / sps);
-  hipLaunchKernelGGL((gemm_mid_kernel<MT, KC, DEPTH, TC, EPI>), grid, dim3(kMidWaves * kWave), lds, st, (const bf16*)x,
+  dim3 grid((tiles + WN - 1) / WN, (steps + sps - 1) / sps);
+  hipLaunchKernelGGL((gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI>), grid, dim3(WN * kWave), lds, st, (const bf16*)x,
                      (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps);
   return check_launch("gemm_mid");
 }
 
-template <typename TC, int EPI>
+// How many wavefronts (tiles of 16 rows of W) a workgroup takes: the number from 3 to 8 that leaves the compute
+// units the least idle when every unit works through its workgroups one after the other -- 1,216 tiles are 304
+// workgroups of four (a quarter of the units get two, the others wait: 59 % busy) or 244 of five (95 %).
+// Equal numbers go to four, then to the larger.
+inline int mid_waves(int n, int slices) {
+  const int tiles = (n + 15) / 16;
+  const int order[] = {4, 5, 6, 8, 3};
+  int best = 4;
+  double best_busy = 0.0;
+  for (int wn : order) {
+    const long groups = (long)((tiles + wn - 1) / wn) * slices;
+    const long rounds = (groups + 255) / 256;
+    const double busy = (double)tiles * slices / (double)(rounds * 256 * wn);
+    if (busy > best_busy + 0.02) best = wn, best_busy = busy;
+  }
+  return best;
+}
+
+template <int WN, typename TC, int EPI>
 int launch_mid_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n,
                   int k, long ldx, long ldc, int slices) {
-#define PA_MID(MT, KC, D) return launch_mid<MT, KC, D, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices)
+#define PA_MID(MT, KC, D) return launch_mid<MT, KC, D, WN, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices)
   // chunks of 256 columns and a ring of four steps up to 64 rows; 128 columns beyond (LDS holds two chunks);
   // measured over chunk sizes and ring depths at the shapes of a 4B model: within a microsecond of one another
   switch ((m + 15) / 16) {
     case 1: PA_MID(1, 256, 4);
     case 2: PA_MID(2, 256, 4);
-    case 3: PA_MID(3, 256, 4);   // 48 rows x 32 pieces = 1536 = 6 a thread
+    case 3: PA_MID(3, 256, 4);
     case 4: PA_MID(4, 256, 4);
     case 5:
-    case 6: PA_MID(6, 128, 4);   // 96 rows x 16 pieces = 1536
+    case 6: PA_MID(6, 128, 4);
     default: PA_MID(8, 128, 4);
   }
 #undef PA_MID
+}
+
+template <typename TC, int EPI>
+int launch_mid_wn(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n,
+                  int k, long ldx, long ldc, int slices, int waves) {
+  switch (waves ? waves : mid_waves(n, slices)) {
+    case 3: return launch_mid_mt<3, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
+    case 5: return launch_mid_mt<5, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
+    case 6: return launch_mid_mt<6, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
+    case 8: return launch_mid_mt<8, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
+    default: return launch_mid_mt<4, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
+  }
 }
 
 }  // namespace pa
@@ -257,7 +299,7 @@ using namespace pa;
 // weight's shape alone.
 extern "C" int pa_gemm_mid_slices(int n, int k) {
   if (n <= 0 || k <= 0) return 1;
-  const int blocks = ((n + 15) / 16 + kMidWaves - 1) / kMidWaves, steps = (k + 63) / 64;
+  const int blocks = ((n + 15) / 16 + 4) / 5, steps = (k + 63) / 64;
   int s = 1;
   while (s < 8 && blocks * s < 256 && steps / (2 * s) >= 8) s *= 2;
   return s;
@@ -269,8 +311,10 @@ extern "C" long pa_gemm_mid_parts(int m, int n, int slices) { return slices <= 1
 // C[m, n] = X[m, k] W^T for m <= 128 from the weight in tiles.  slices 1: epilogue 0 writes C (+ bias) as
 // out_dtype (0 float32, 1 bfloat16), epilogue 1 C[m, n/2] = silu(gate) * up.  slices > 1 (epilogue 0 only):
 // nothing is written to C; parts [slices, m, n] receives each slice's 32-bit sums (the bias in the first).
+// waves: wavefronts (tiles of 16 rows of W) a workgroup, 3, 4, 5, 6 or 8, or 0 for the launcher's choice; the sums
+// are the same bits at every number.
 extern "C" int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias,
-                           void* c, float* parts, int m, int n, int k, long ldx, long ldc, int slices) {
+                           void* c, float* parts, int m, int n, int k, long ldx, long ldc, int slices, int waves) {
   if (m == 0 || n == 0) return 0;
   PA_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_mid: bad sizes m=%d n=%d k=%d", m, n, k);
   PA_REQUIRE(m <= kMidMaxM, "gemm_mid: %d rows exceed %d", m, kMidMaxM);
@@ -278,6 +322,8 @@ extern "C" int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void
              k, ldx);
   const int steps = (k + 63) / 64;
   PA_REQUIRE(slices >= 1 && slices <= steps && slices <= 64, "gemm_mid: %d slices of %d steps", slices, steps);
+  PA_REQUIRE(waves == 0 || waves == 3 || waves == 4 || waves == 5 || waves == 6 || waves == 8,
+             "gemm_mid: %d wavefronts a workgroup (3, 4, 5, 6, 8, or 0 to let the launcher choose)", waves);
   {
     const int sps = (steps + slices - 1) / slices;   // every slice must get a step, or its part would stay unwritten
     PA_REQUIRE((steps + sps - 1) / sps == slices, "gemm_mid: %d steps do not cut into %d slices of %d", steps, slices, sps);
@@ -285,18 +331,18 @@ extern "C" int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void
   hipStream_t st = (hipStream_t)stream;
   if (slices > 1) {
     PA_REQUIRE(epilogue == kMidPlain && parts, "gemm_mid: a product in slices has no epilogue and needs `parts`");
-    return launch_mid_mt<float, kMidSlices>(st, x, w, bias, nullptr, parts, m, n, k, ldx, ldc, slices);
+    return launch_mid_wn<float, kMidSlices>(st, x, w, bias, nullptr, parts, m, n, k, ldx, ldc, slices, waves);
   }
   PA_REQUIRE(c, "gemm_mid: no output");
   PA_REQUIRE(epilogue == kMidPlain || (epilogue == kMidSiluMul && n % 2 == 0 && !bias),
              "gemm_mid: the SiLU*up epilogue needs an even n and no bias");
   PA_REQUIRE(ldc >= (epilogue == kMidSiluMul ? n / 2 : n), "gemm_mid: output row stride %ld is too small", ldc);
   if (epilogue == kMidPlain && out_dtype == kBF16)
-    return launch_mid_mt<bf16, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1);
+    return launch_mid_wn<bf16, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves);
   if (epilogue == kMidPlain && out_dtype == kF32)
-    return launch_mid_mt<float, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1);
+    return launch_mid_wn<float, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves);
   if (epilogue == kMidSiluMul && out_dtype == kBF16)
-    return launch_mid_mt<bf16, kMidSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1);
+    return launch_mid_wn<bf16, kMidSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves);
   return pa::fail("gemm_mid: unsupported output type %d with epilogue %d", out_dtype, epilogue);
 }
 

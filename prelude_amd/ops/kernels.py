@@ -367,13 +367,17 @@ class SliceSums:
 
 
 GEMM_MID_MAX_ROWS = 128
-# Where ``linear`` takes the product with X staged in LDS (measured at the shapes of a 4B model, 17 to 128 rows):
-# cut into slices, for a reader that adds them, where the weight is narrow enough to be cut into 8 -- [2560, 4096]
-# at 64 rows 10.9 against the library's 14.4 us, [2560, 9728] 18 against 27; and uncut for very wide weights with
-# 32-bit output (the head: 175 us at 64 rows where the library takes 176 and a conversion pass of 20)
-MID_MIN_SLICES = 8
+# Where ``linear`` takes the product with X staged in LDS (measured at the shapes of 4B, 8B and 32B models, 17 to
+# 128 rows).  Cut into slices, for a reader that adds them, wherever the weight's shape gives two slices or more:
+# [2560, 4096] at 64 rows 9.2 against the library's 14.7 us, [2560, 9728] 14.4 against 28, [4096, 12288] 28 against
+# 37, [5120, 25600] 50 against 155 (and 73 against 179 at 128 rows).  Uncut for very wide weights with 32-bit output
+# (the head: at 64 rows and 2,560 columns 196 us where the library takes 176 and a conversion pass of 20; with longer
+# rows the library is ahead from 48 rows on).  The gated product with its activation in the epilogue: see
+# ``linear_silu_mul``.
+MID_MIN_SLICES = 2
 MID_WIDE_ROWS = 65536
-MID_WIDE_MAX_M = 64
+MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns, half of it beyond
+MID_WIDE_SHORT_K = 4096
 MID_PRODUCTS = True    # ``set_mid_products``: off sends these products where they went without this kernel (measurements)
 
 
@@ -388,9 +392,10 @@ def gemm_mid_slices(n: int, k: int) -> int:
 
 
 def gemm_mid(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = None,
-             out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False, slices: int = 1):
+             out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False, slices: int = 1, waves: int = 0):
     """x [M <= 128, K] @ w[N, K]^T from the weight in tiles, X staged through LDS; with ``slices`` > 1 the result
-    is a ``SliceSums`` (one 32-bit partial sum per slice of K) instead of a tensor."""
+    is a ``SliceSums`` (one 32-bit partial sum per slice of K) instead of a tensor.  ``waves``: wavefronts a
+    workgroup (3, 4, 5, 6, 8; 0 lets the launcher choose by the weight's shape; the same bits at every number)."""
     if not isinstance(w, TiledWeight):
         raise NativeError("gemm_mid takes the weight in tiles (pack_tiles)")
     _dev(x, w.data, bias)
@@ -405,12 +410,12 @@ def gemm_mid(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = N
     if slices > 1:
         parts = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
         check(kernels().pa_gemm_mid(_stream(), _CODES[out_dtype], 0, _ptr(x), _ptr(w.data), _ptr(bias), None, _ptr(parts),
-                                    m, n, k, k, n, slices))
+                                    m, n, k, k, n, slices, waves))
         return SliceSums(parts, out_dtype)
     cols = n // 2 if silu_mul_epilogue else n
     out = torch.empty((m, cols), dtype=out_dtype, device=x.device)
     check(kernels().pa_gemm_mid(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w.data),
-                                _ptr(bias), _ptr(out), None, m, n, k, k, cols, 1))
+                                _ptr(bias), _ptr(out), None, m, n, k, k, cols, 1, waves))
     return out
 
 
@@ -465,7 +470,7 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
             s = gemm_mid_slices(n, k)
             if s >= MID_MIN_SLICES:
                 return gemm_mid(x, tiles, bias, slices=s)
-        if n >= MID_WIDE_ROWS and m <= MID_WIDE_MAX_M:
+        if n >= MID_WIDE_ROWS and m <= (MID_WIDE_MAX_M if k <= MID_WIDE_SHORT_K else MID_WIDE_MAX_M // 2):
             return gemm_mid(x, tiles, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
@@ -496,6 +501,11 @@ def set_skinny_max_rows(n: int) -> None:
 # SiLU*up kernel: measured in the decode step, that is the faster way up to 24 rows for [19456, 2560] (5.76 against
 # 5.79 ms a step at 24 rows, 6.76 against 6.71 at 32) and up to 32 rows for [24576, 4096] (6.94 against 7.26 ms at
 # 24 rows, 7.98 against 8.18 at 32); for [51200, 5120] the library with the separate kernel is ahead from 12 rows on
+# Beyond 16 rows the product with X staged in LDS takes it, activation in its epilogue too: [19456, 2560] 20.3 us at
+# 32 rows, 22.9 at 64 and 33.0 at 128 against the library's 27.3, 31.0 and 35.3 with the separate kernel (the
+# streaming kernel: 30 and 47 at 32 and 64); [24576, 4096] 37.6 at 64 rows against 47.7; [51200, 5120] stays with the
+# library (110 against 105 at 64 rows, 163 against 119 at 128).  The bounds below are for weights without tiles
+# for that kernel to read, and for measurements with it switched off.
 GATED_TILED_ROWS = 24          # ... and 32 for rows of GATED_TILED_LONG_K columns or more
 GATED_TILED_LONG_K = 4096
 GATED_TILED_ELEMENTS = 1 << 27
@@ -514,6 +524,8 @@ def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
             if isinstance(w, LinearWeight):
                 w = tiles if tiles is not None and m <= 16 else w.rows
             return gemm_skinny(x, w, silu_mul_epilogue=True)
+        if MID_PRODUCTS and tiles is not None and m <= GEMM_MID_MAX_ROWS and tiles.n * k <= GATED_TILED_ELEMENTS:
+            return gemm_mid(x, tiles, silu_mul_epilogue=True)
         if tiles is not None and _gated_tiled(m, tiles.n, k):
             return gemm_skinny(x, tiles, silu_mul_epilogue=True)
     return silu_mul(linear(x, w))

@@ -208,6 +208,11 @@ def test_gemm_mid(gpu, m, n, k, slices):
     behind[:m] = xd
     got = K().gemm_mid(behind[:m], tiles, out_dtype=torch.float32)
     assert bool(torch.isfinite(got).all()) and torch.equal(got, full)
+    # how many wavefronts share a workgroup (which the launcher picks by the weight's shape) changes no bit
+    for waves in (3, 4, 5, 6, 8):
+        assert torch.equal(K().gemm_mid(xd, tiles, out_dtype=torch.float32, waves=waves), full), f"{waves} wavefronts"
+        if slices > 1:
+            assert torch.equal(K().gemm_mid(xd, tiles, bd, slices=slices, waves=waves).parts, ss.parts), f"{waves} wavefronts, slices"
 
 
 def test_gemm_mid_refuses_and_is_dispatched(gpu):
@@ -220,6 +225,8 @@ def test_gemm_mid_refuses_and_is_dispatched(gpu):
         K().gemm_mid(torch.zeros(8, 4096, dtype=torch.bfloat16, device=gpu), tiles, slices=60)
     with pytest.raises(NativeError, match="in tiles"):
         K().gemm_mid(torch.zeros(8, 4096, dtype=torch.bfloat16, device=gpu), w)
+    with pytest.raises(NativeError, match="7 wavefronts"):
+        K().gemm_mid(torch.zeros(8, 4096, dtype=torch.bfloat16, device=gpu), tiles, waves=7)
     # linear() hands a narrow weight at 17 to 128 rows to it in slices only when the caller's reader adds slices
     lw = K().LinearWeight(w, tiles)
     x = rnd(40, 4096, dtype=torch.bfloat16).to(gpu)
@@ -229,6 +236,19 @@ def test_gemm_mid_refuses_and_is_dispatched(gpu):
     close(K().as_tensor(got), x.double().cpu() @ w.double().cpu().T, torch.bfloat16)
     assert isinstance(K().linear(x[:8].contiguous(), lw, slices_ok=True), torch.Tensor)      # few rows: the streaming kernel
     assert isinstance(K().linear(x.float(), w.float(), slices_ok=True), torch.Tensor)      # 32-bit: the plain product
+    # the gated product beyond 16 rows: activation in this kernel's epilogue (the same bits as asked for directly)
+    wg = rnd(1216, 520, dtype=torch.bfloat16, seed=5, scale=0.05).to(gpu)
+    lg = K().LinearWeight(wg, K().pack_tiles(wg))
+    xg = rnd(40, 520, dtype=torch.bfloat16, seed=6).to(gpu)
+    assert torch.equal(K().linear_silu_mul(xg, lg), K().gemm_mid(xg, lg.tiles, silu_mul_epilogue=True))
+    K().set_mid_products(False)
+    try:
+        other = K().linear_silu_mul(xg, lg)
+    finally:
+        K().set_mid_products(True)
+    ref = xg.double().cpu() @ wg.double().cpu().T
+    close(other, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16, bf16=1.25e-2)
+    close(K().linear_silu_mul(xg, lg), pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16, bf16=1.25e-2)
 
 
 @pytest.mark.parametrize("m,n,k", [(30, 24, 16), (4, 76, 24), (16, 48, 40), (1, 32, 8), (39, 2304, 24), (64, 40, 72)])
