@@ -245,9 +245,12 @@ int launch_mid(hipStream_t st, const void* x, const void* w, const float* bias, 
 // How many wavefronts (tiles of 16 rows of W) a workgroup takes: the number from 3 to 8 that leaves the compute
 // units the least idle when every unit works through its workgroups one after the other -- 1,216 tiles are 304
 // workgroups of four (a quarter of the units get two, the others wait: 59 % busy) or 244 of five (95 %).
-// Equal numbers go to four, then to the larger.
+// Equal numbers go to four, then to the larger.  (The model is one of few rounds; see below for many.)
 inline int mid_waves(int n, int slices) {
   const int tiles = (n + 15) / 16;
+  // a grid of many rounds whatever the number: the most wavefronts, which stage X the fewest times (the head of
+  // 151,936 rows at 64 rows of X: 166 us with eight, 179 with four, 185 with three)
+  if ((long)((tiles + 7) / 8) * slices >= 4 * 256) return 8;
   const int order[] = {4, 5, 6, 8, 3};
   int best = 4;
   double best_busy = 0.0;
