@@ -674,15 +674,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   const int g = lane / 16, r = lane % 16;
   const int group = nh / nkv;
   const int hgroups = group / GT;
-  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int kvh = blockIdx.x / hgroups, hg = blockIdx.x % hgroups;   // head groups fastest over the grid
   const int seq = seq_ids[blockIdx.z];
   const int row0 = cu_q[seq];
   const int q_len = cu_q[seq + 1] - row0;
   const int ctx = context_lens[seq];
   const int tiles = (q_len + 63) / 64;
   // unpaired: one tile per workgroup, late (long) tiles first
-  const int first = paired ? (int)blockIdx.x : tiles - 1 - (int)blockIdx.x;
-  const int second = paired ? tiles - 1 - (int)blockIdx.x : first;
+  const int first = paired ? (int)blockIdx.y : tiles - 1 - (int)blockIdx.y;
+  const int second = paired ? tiles - 1 - (int)blockIdx.y : first;
   if (first > second || first < 0) return;
   const int* table = block_table + (size_t)seq * table_stride;
   const int head0 = kvh * group + hg * GT;
@@ -897,14 +897,14 @@ __global__ __launch_bounds__(256 * HW, 2) void attn_prefill_lds_kernel(
   const int g = lane / 16, r = lane % 16;
   const int group = nh / nkv;
   const int hgroups = group / (GT * HW);
-  const int kvh = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+  const int kvh = blockIdx.x / hgroups, hg = blockIdx.x % hgroups;   // head groups fastest over the grid
   const int seq = seq_ids[blockIdx.z];
   const int row0 = cu_q[seq];
   const int q_len = cu_q[seq + 1] - row0;
   const int ctx = context_lens[seq];
   const int tiles = (q_len + 63) / 64;
-  const int first = paired ? (int)blockIdx.x : tiles - 1 - (int)blockIdx.x;
-  const int second = paired ? tiles - 1 - (int)blockIdx.x : first;
+  const int first = paired ? (int)blockIdx.y : tiles - 1 - (int)blockIdx.y;
+  const int second = paired ? tiles - 1 - (int)blockIdx.y : first;
   if (first > second || first < 0) return;   // the same for the whole workgroup
   const int* table = block_table + (size_t)seq * table_stride;
   const int head0 = kvh * group + hg * GT * HW;
@@ -952,7 +952,7 @@ int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const v
                           int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale,
                           int paired) {
   const int tiles = (max_q_len + 63) / 64;
-  dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / (GT * HW)), nseq);
+  dim3 grid(nkv * (nh / nkv / (GT * HW)), paired ? (tiles + 1) / 2 : tiles, nseq);
   // the two buffers are more than the 64 KB a kernel may declare: asked for at launch, allowed once per kernel
   static const hipError_t allowed =
       hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_lds_kernel<HD, GT, HW>),
@@ -971,7 +971,7 @@ int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void*
                       int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, int paired,
                       int hw, bool staged) {
   const int tiles = (max_q_len + 63) / 64;
-  dim3 grid(paired ? (tiles + 1) / 2 : tiles, nkv * (nh / nkv / GT), nseq);
+  dim3 grid(nkv * (nh / nkv / GT), paired ? (tiles + 1) / 2 : tiles, nseq);
   if (staged) {
     if (hw == 2)
       return launch_prefill_staged<HD, GT, 2>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
