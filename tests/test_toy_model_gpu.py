@@ -69,6 +69,20 @@ def register_toy():
             s_all.index_copy_(0, slots, s)
             return K.linear(s.to(x.dtype), self.w)
 
+    @register_part("mixer", "toy_decay_whole")
+    class ToyDecayWhole(ToyDecay):
+        """The same mixer, declared unable to take a prompt in portions: it refuses any portion of several tokens
+        that does not start its request, and the scheduler is to feed it prompts whole."""
+        ATOMIC_PREFILL = True
+        portions = []          # (tokens, fresh) of every portion it was given, for the test to look at
+
+        def forward(self, x, step, cache, write_cache=True):
+            for n, fresh in zip(step.q_lens, step.fresh_host):
+                ToyDecayWhole.portions.append((n, bool(fresh)))
+                if n > 1 and not fresh:
+                    raise RuntimeError(f"a prompt came in portions: {n} tokens behind an earlier portion")
+            return super().forward(x, step, cache, write_cache)
+
     @dataclasses.dataclass
     class ToyConfig:
         vocab_size: int
@@ -106,6 +120,9 @@ def register_toy():
     register_architecture(Architecture("toy", ("Toy",), ("toy",), parse, spec))
     register_architecture(Architecture("toydevice", ("ToyDevice",), ("toydevice",), parse,
                                        lambda c: spec(c, "toy_decay_device")))
+    register_architecture(Architecture("toywhole", ("ToyWhole",), ("toywhole",), parse,
+                                       lambda c: spec(c, "toy_decay_whole")))
+    return ToyDecayWhole
 
 
 RAW = dict(architectures=["ToyForCausalLM"], vocab_size=97, hidden_size=48, inter=80, heads=3, head_dim=16, decay=0.7,
@@ -256,6 +273,42 @@ def test_toy_model_with_state_decodes_from_graphs(gpu, tmp_path):
     from helpers import check
     for r, lo, hi in ((0, 20, 40), (1, 9, 21), (2, 0, 8)):
         check(replayed[r], refs[r][lo:hi], "bfloat16", f"request {r}")
+
+
+def test_toy_mixer_that_takes_prompts_whole(gpu, tmp_path):
+    """A mixer that sets ATOMIC_PREFILL: under a token budget that would cut prompts, the scheduler feeds each
+    prompt in one step (later, if it does not fit beside the others), the tokens are the plain model's, and a
+    request that could never be fed whole is refused when it is added."""
+    whole = register_toy()
+    from prelude_amd import LLM
+    from prelude_amd.engine.scheduler import SchedulerError
+    from prelude_amd.weights import WeightFiles, write_random_model
+    raw = dict(RAW, architectures=["ToyWholeForCausalLM"])
+    folder = write_random_model(raw, str(tmp_path / "toywhole"), seed=7, std=0.2, norm_std=0.1, dtype=torch.float32)
+    files = WeightFiles(folder)
+    w = {n: files.tensor(n).clone() for n in files.names()}
+    llm = LLM(folder, dtype="float32", page_size=8, max_cache_tokens=256, max_state_slots=3, max_num_batched_tokens=16)
+    assert llm.engine.model.atomic_prefill and not llm.engine.model.graph_safe
+    whole.portions.clear()
+    prompts = [[5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15], [11, 12, 13, 14, 15, 16, 17, 18, 19], [20] * 12, [3, 4]]
+    outs = llm.generate(prompts, max_tokens=4, temperature=0.0)
+    for p, o in zip(prompts, outs):
+        seq = list(p)
+        assert o.finish_reason in ("length", "eos") and o.error is None
+        for tok in o.token_ids:
+            assert tok == int(torch.argmax(plain_toy(w, seq)[-1]))
+            seq.append(tok)
+    # every prompt arrived whole (11 + 9 would fit a step of 16 only in part: the second waited), none in pieces
+    firsts = sorted(n for n, fresh in whole.portions if fresh)
+    assert firsts == sorted([len(p) for p in prompts] * 2)        # the mixer runs twice a step (its layer is named twice)
+    assert all(n == 1 for n, fresh in whole.portions if not fresh)
+    # 14 prompt tokens and up to 4 new ones cannot be fed in one step of 16 after an eviction: refused at once
+    session = llm.session()
+    with pytest.raises(SchedulerError, match="must be fed whole"):
+        session.add(list(range(14)), max_tokens=4)
+    assert session.add(list(range(13)), max_tokens=4) == 0
+    session.abandon()
+    assert llm.engine.tables.audit() == "" and llm.engine.tables.free_state_slots() == 3
 
 
 def rows_of(d):
