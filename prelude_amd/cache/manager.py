@@ -185,7 +185,7 @@ class PageTables:
 class KVLayerCache:
     """What an attention-like mixer gets: its pages and the group whose tables index them."""
     k: torch.Tensor   # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor   # [pages, kv_heads, head_dim, page_size]
+    v: torch.Tensor   # [pages, kv_heads, value width (head_dim unless the spec says otherwise), page_size]
     group: int
 
 
@@ -229,7 +229,7 @@ def plan_groups(cache_specs: Sequence[object]) -> Tuple[List[KVCacheSpec], List[
 
 def bytes_per_token(cache_specs: Sequence[object], dtype: torch.dtype) -> int:
     el = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * cs.num_kv_heads * cs.head_dim * el for cs in cache_specs if isinstance(cs, KVCacheSpec))
+    return sum(cs.num_kv_heads * (cs.head_dim + cs.v_dim) * el for cs in cache_specs if isinstance(cs, KVCacheSpec))
 
 
 def state_bytes_per_slot(cache_specs: Sequence[object]) -> int:
@@ -277,7 +277,7 @@ def allocate_storage(cache_specs: Sequence[object], of_slot: Sequence[Optional[i
         if isinstance(cs, KVCacheSpec):
             n = pages_per_group[g]
             out.append(KVLayerCache(torch.zeros((n, cs.num_kv_heads, page_size, cs.head_dim), dtype=dtype, device=device),
-                                    torch.zeros((n, cs.num_kv_heads, cs.head_dim, page_size), dtype=dtype, device=device), g))
+                                    torch.zeros((n, cs.num_kv_heads, cs.v_dim, page_size), dtype=dtype, device=device), g))
         elif isinstance(cs, StateSpec):
             out.append(StateLayerCache({name: torch.zeros((state_slots, *shape), dtype=dt, device=device)
                                         for name, shape, dt in cs.tensors}))

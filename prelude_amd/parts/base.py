@@ -44,10 +44,17 @@ class TensorReq:
 
 @dataclasses.dataclass(frozen=True)
 class KVCacheSpec:
-    """Keys and values per token, in pages.  ``window`` = keys looked back over, own included; 0 = all."""
+    """Keys and values per token, in pages.  ``window`` = keys looked back over, own included; 0 = all.
+    ``value_dim``: the width of a value where it is not the key's (None: ``head_dim``); mixers with the same
+    heads, widths and window share a group of pages."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: Optional[int] = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclasses.dataclass(frozen=True)

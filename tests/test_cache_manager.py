@@ -214,3 +214,16 @@ def test_pool_sizes_per_group():
     # never more than the tokens asked for, never less than a page
     assert pages_per_group(40, groups, 8, max_requests=4, max_request_tokens=2048, chunk=16) == [5, 5, 5]
     assert pages_per_group(1, groups, 8, max_requests=1, max_request_tokens=8, chunk=1) == [1, 1, 1]
+
+
+def test_a_value_width_of_its_own_counts_in_the_bytes():
+    """A mixer whose values are narrower (or wider) than its keys: a group of its own, and the bytes a token takes
+    follow both widths."""
+    import torch
+    from prelude_amd.cache.manager import bytes_per_token, plan_groups
+    from prelude_amd.parts import KVCacheSpec
+    same, narrow = KVCacheSpec(2, 64, 0), KVCacheSpec(2, 64, 0, value_dim=16)
+    assert same.v_dim == 64 and narrow.v_dim == 16
+    groups, of_slot = plan_groups([same, narrow, same])
+    assert groups == [same, narrow] and of_slot == [0, 1, 0]
+    assert bytes_per_token([same, narrow], torch.bfloat16) == 2 * (64 + 64) * 2 + 2 * (64 + 16) * 2

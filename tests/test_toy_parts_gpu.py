@@ -192,3 +192,118 @@ def test_routed_ffn_and_another_position_encoding(gpu, tmp_path):
     for tok in f32.token_ids:
         assert tok == int(torch.argmax(plain(w, seq)[0][-1]))
         seq.append(tok)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# a mixer whose values are narrower than its keys: the pages of its group are shaped by the mixer's own spec
+KD, VD = 16, 8
+
+
+def register_narrow_values():
+    from prelude_amd.config.registry import Architecture, register_architecture
+    from prelude_amd.models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
+    from prelude_amd.ops import kernels as K
+    from prelude_amd.parts import MATRIX, KVCacheSpec, Mixer, TensorReq, register_part
+
+    @register_part("mixer", "toy_narrow_values")
+    class ToyNarrowValues(Mixer):
+        """One head, no rotation: keys of KD elements, values of VD, both kept in the framework's pages and found
+        through the step's block table and slot numbers (plain tensor indexing; it walks the step's host lists)."""
+        GRAPH_SAFE = False
+
+        def __init__(self, hidden_size):
+            self.hidden_size = hidden_size
+
+        def cache_spec(self):
+            return KVCacheSpec(1, KD, 0, value_dim=VD)
+
+        def tensors(self):
+            h = self.hidden_size
+            return {"q.weight": TensorReq((KD, h), MATRIX), "k.weight": TensorReq((KD, h), MATRIX),
+                    "v.weight": TensorReq((VD, h), MATRIX), "o.weight": TensorReq((h, VD), MATRIX)}
+
+        def load(self, tensors, dtype, device):
+            self.w = dict(tensors)
+
+        def forward(self, x, step, cache, write_cache=True):
+            q, k, v = (K.linear(x, self.w[n + ".weight"]) for n in "qkv")
+            grp = step.kv[cache.group]
+            page = step.page_size
+            assert cache.k.shape[1:] == (1, page, KD) and cache.v.shape[1:] == (1, VD, page)
+            slots = grp.slots.to(torch.int64)
+            cache.k[slots // page, 0, slots % page] = k
+            cache.v[slots // page, 0, :, slots % page] = v
+            out = torch.empty((x.shape[0], VD), dtype=x.dtype, device=x.device)
+            t = 0
+            for i, n in enumerate(step.q_lens):
+                ctx = step.starts[i] + n
+                pages = grp.block_table[i, :-(-ctx // page)].to(torch.int64)
+                keys = cache.k[pages, 0].reshape(-1, KD)[:ctx].float()
+                vals = cache.v[pages, 0].permute(0, 2, 1).reshape(-1, VD)[:ctx].float()
+                s = q[t:t + n].float() @ keys.T / 4.0
+                pos = torch.arange(step.starts[i], ctx, device=x.device).reshape(-1, 1)
+                s = s.masked_fill(torch.arange(ctx, device=x.device).reshape(1, -1) > pos, float("-inf"))
+                out[t:t + n] = (torch.softmax(s, dim=-1) @ vals).to(x.dtype)
+                t += n
+            return K.linear(out, self.w["o.weight"])
+
+    @dataclasses.dataclass
+    class Cfg:
+        vocab_size: int
+        hidden_size: int
+        inter: int
+        eps: float
+        max_positions: int
+
+    def spec(c):
+        norm = lambda name: PartSpec("rms_norm", dict(size=c.hidden_size, eps=c.eps), {"weight": name})
+        layer = LayerSpec("prenorm", {
+            "input_norm": norm("n1"), "post_mixer_norm": norm("n2"),
+            "mixer": PartSpec("toy_narrow_values", dict(hidden_size=c.hidden_size), {f"{x}.weight": f"mix.{x}" for x in "qkvo"}),
+            "ffn": PartSpec("gated_mlp", dict(hidden_size=c.hidden_size, intermediate_size=c.inter),
+                            {f"{x}_proj.weight": f"ffn.{x}" for x in ("gate", "up", "down")})})
+        return ModelSpec("ToyNarrowForCausalLM", c.vocab_size, c.hidden_size, c.max_positions, (0,),
+                         PartSpec("token_embedding", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "emb"}),
+                         [layer], [RunSpec(0)], norm("final"),
+                         PartSpec("linear_head", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "emb"}), {})
+
+    register_architecture(Architecture("toy_narrow", ("ToyNarrow",), ("toy_narrow",),
+                                       lambda raw: Cfg(**{f.name: raw[f.name] for f in dataclasses.fields(Cfg)}), spec))
+
+
+def test_a_mixer_with_values_narrower_than_its_keys(gpu, tmp_path):
+    register_narrow_values()
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    from prelude_amd.weights import WeightFiles, write_random_model
+    raw = dict(architectures=["ToyNarrowForCausalLM"], vocab_size=53, hidden_size=24, inter=40, eps=1e-5, max_positions=64)
+    folder = write_random_model(raw, str(tmp_path / "narrow"), seed=3, std=0.3, norm_std=0.1, dtype=torch.float32)
+    files = WeightFiles(folder)
+    w = {n: files.tensor(n).double() for n in files.names()}
+    toks = torch.randint(0, 53, (45,), generator=torch.Generator().manual_seed(2)).tolist()
+    n = len(toks)
+    x = w["emb"][toks]
+    h = pm.rms_norm(x, w["n1"], 1e-5)
+    q, k, v = (h @ w["mix." + c].T for c in "qkv")
+    o = pm.attention(q.reshape(n, 1, KD), k.reshape(n, 1, KD), torch.cat([v, torch.zeros(n, KD - VD, dtype=v.dtype)], -1).reshape(n, 1, KD),
+                     0.25).reshape(n, KD)[:, :VD]
+    x = x + o @ w["mix.o"].T
+    x = x + pm.swiglu(pm.rms_norm(x, w["n2"], 1e-5), w["ffn.gate"], w["ffn.up"], w["ffn.down"])
+    ref = pm.rms_norm(x, w["final"], 1e-5) @ w["emb"].T
+
+    eng = Engine.from_model_dir(folder, EngineConfig(dtype="float32", page_size=8, max_cache_tokens=128))
+    assert eng.caches[0].k.shape[-1] == KD and eng.caches[0].v.shape[-2] == VD
+    assert eng.group_specs[0].v_dim == VD
+
+    def close(got, want):
+        assert float((got.double().cpu() - want).abs().max()) < 2e-5 * max(1.0, float(want.abs().max()))
+
+    close(eng.step([StepEntry(0, toks, list(range(n)))]), ref)
+    eng.release(0)
+    at, got = 0, []
+    for size in (7, 2, 13, 1, 1, 9, 12):                  # portions and single tokens, across pages of 8
+        got.append(eng.step([StepEntry(1, toks[at:at + size], list(range(size)))]))
+        at += size
+    close(torch.cat(got), ref)
+    eng.release(1)
+    assert eng.tables.audit() == ""
