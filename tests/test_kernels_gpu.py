@@ -300,6 +300,27 @@ def test_drawn_products(gpu, seed):
         assert tuple(got.shape) == tuple(want.shape), f"{what}, {name}: shape {tuple(got.shape)}"
         err = float((got.double().cpu() - want).abs().max())
         assert err <= tol(dt, want, f32=2e-5), f"{what}, {name}: max error {err:.3e} > {tol(dt, want, f32=2e-5):.3e}"
+    # the product with X staged in LDS, at a drawn number of rows up to 128, of wavefronts and of slices
+    m3 = int(rng.choice([17, 64, 65, 128, int(rng.integers(1, 129))]))
+    x3 = rnd(m3, k, dtype=torch.bfloat16, seed=seed + 5)
+    x3d = x3.to(gpu)
+    ref3 = x3.double() @ w.double().T
+    waves = int(rng.choice([0, 3, 4, 5, 6, 8]))
+    steps = (k + 63) // 64
+    cuts = [c for c in (2, 3, 4, 8) if c <= steps and -(-steps // -(-steps // c)) == c]
+    for name, got, want, dt in (
+            ("mid", K().gemm_mid(x3d, tiles, out_dtype=torch.float32, waves=waves), ref3, torch.float32),
+            ("mid, bias", K().gemm_mid(x3d, tiles, bd, waves=waves), ref3 + b.double(), torch.bfloat16),
+            ("mid, SiLU*up", K().gemm_mid(x3d, tiles, silu_mul_epilogue=True, waves=waves), pm.silu(ref3[:, 0::2]) * ref3[:, 1::2],
+             torch.bfloat16),
+            ("linear for a reader of slices", K().as_tensor(K().linear(x3d, lw, bd, slices_ok=True)), ref3 + b.double(), torch.bfloat16)):
+        err = float((got.double().cpu() - want).abs().max())
+        assert err <= tol(dt, want, f32=2e-5), f"{what}, rows {m3}, {waves} wavefronts, {name}: max error {err:.3e}"
+    if cuts:
+        c = int(rng.choice(cuts))
+        parts = K().gemm_mid(x3d, tiles, bd, slices=c, waves=waves).parts
+        err = float((parts.double().sum(0).cpu() - ref3 - b.double()).abs().max())
+        assert err <= tol(torch.float32, ref3, f32=2e-5), f"{what}, rows {m3}, {waves} wavefronts, {c} slices: max error {err:.3e}"
     # many rows through the dispatcher (the library product beyond the streaming kernel's rows)
     m2 = int(rng.integers(65, 400))
     x2 = rnd(m2, k, dtype=torch.bfloat16, seed=seed + 3)
