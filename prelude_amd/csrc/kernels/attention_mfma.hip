@@ -76,6 +76,9 @@ __device__ __forceinline__ float xor_sum16_32(float v) {
 // moves only when a score exceeds it by more than kLazyLog2 in the exponent (then every term so far is rescaled);
 // until then a probability may be as large as 2^kLazyLog2 instead of at most 1, which costs 32-bit sums and bfloat16
 // probabilities nothing (the quotient O / l is the same), and spares the rescaling of the whole output in most steps.
+// Whether it must move is asked of every lane's own eight scores against `lim` = m + kLazyLog2 / c, one compare;
+// only when some lane of the wavefront says yes is the column's maximum formed across its four lanes (the same
+// compare on it then decides per column, so a column's sums do not depend on what its neighbours hold).
 // The sum `l` is formed by the matrix cores too, as one more row of V^T that holds ones: it adds up the same
 // rounded probabilities the output is made of, all 32 keys of a step at once, and every lane of a column has it.
 constexpr float kLazyLog2 = 8.0f;
@@ -84,6 +87,8 @@ template <int HD>
 struct HeadState {
   static constexpr int OT = HD / 16;
   float m = -INFINITY;  // reference maximum of the raw scores, equal in the four lanes of a column
+  float lim = -INFINITY;  // a score above this moves m: m + kLazyLog2 / c
+  float shift = 0.f;      // -m c (0 while the column has seen no key): the exponent is s c + shift
   f32x4 l;              // running sum of the column's probabilities (every element the same)
   f32x4 o[OT];          // O^T tiles: head_dim rows 16 t + 4g + i, column r
   __device__ HeadState() {
@@ -179,15 +184,13 @@ __device__ __forceinline__ bf16x8 ones8() {
   return z;
 }
 
-// Scores of 32 keys against one head's 16 queries, then the online softmax: returns the probabilities packed
-// as the B operand of O^T = V^T P^T.  `moved` says whether this lane's reference maximum moved; `m_before` is
-// what it was (the caller rescales the head's sums by 2^((m_before - m) c) then).
+// Scores of 32 keys against one head's 16 queries, s[8] per lane (keys key0 + 8g + 0..7 of query r), and the
+// largest of the lane's eight.
 // `masked` false: every key of the step is visible to every query (no comparisons).
 // `vis(key)` says whether this lane's query may see the key (and the key exists).
 template <int HD, typename Visible>
-__device__ __forceinline__ bf16x8 scores32(int key0, int g, const KFrag<HD>& kf, const bf16x8* qf, float c,
-                                           bool masked, HeadState<HD>& st, bool& moved, float& m_before, Visible vis) {
-  float s[8];
+__device__ __forceinline__ float scores32(int key0, int g, const KFrag<HD>& kf, const bf16x8* qf, bool masked,
+                                          float* s, Visible vis) {
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     f32x4 acc{0.f, 0.f, 0.f, 0.f};
@@ -206,17 +209,37 @@ __device__ __forceinline__ bf16x8 scores32(int key0, int g, const KFrag<HD>& kf,
   float mx = s[0];
 #pragma unroll
   for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-  mx = xor_max16_32(mx);
-  m_before = st.m;
-  // from -inf any finite score moves it (the difference is +inf); -inf against -inf gives NaN, which compares false
-  moved = (mx - st.m) * c > kLazyLog2;
-  if (moved) st.m = mx;
-  const float m_safe = st.m == -INFINITY ? 0.f : st.m;  // a column that has seen no key yet
-  const float shift = -m_safe * c;
+  return mx;
+}
+
+// The reference maximum of a head's columns moves where the step's largest score (`mx_lane`: the lane's own) lies
+// above the column's limit; the sums so far are rescaled by 2^((m_before - m) c) there.  Called only when some
+// lane of the wavefront is above its limit.
+template <int HD>
+__device__ __forceinline__ void move_reference(HeadState<HD>& st, float mx_lane, float c, float over) {
+  constexpr int OT = HeadState<HD>::OT;
+  const float mx = xor_max16_32(mx_lane);
+  const bool moved = mx > st.lim;   // from -inf any finite score; -inf against -inf is false
+  // 2^(-inf) = 0 for a column's first keys: its sums are zero anyway
+  const float alpha = moved ? __builtin_amdgcn_exp2f((st.m - mx) * c) : 1.0f;
+  if (moved) {
+    st.m = mx;
+    st.lim = mx + over;
+    st.shift = -mx * c;
+  }
+#pragma unroll
+  for (int t = 0; t < OT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st.o[t][i] *= alpha;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) st.l[i] *= alpha;
+}
+
+// The probabilities 2^((s - m) c), c = scale * log2(e), packed as the B operand of O^T = V^T P^T.
+__device__ __forceinline__ bf16x8 probabilities(const float* s, float c, float shift) {
   bf16x8 pb;
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
-    pb[i] = (bf16)__builtin_amdgcn_exp2f(fmaf(s[i], c, shift));  // 2^((s - m) c), c = scale * log2(e)
+  for (int i = 0; i < 8; ++i) pb[i] = (bf16)__builtin_amdgcn_exp2f(fmaf(s[i], c, shift));
   return pb;
 }
 
@@ -242,23 +265,16 @@ __device__ __forceinline__ void attend32_core(int key0, int g, const KFrag<HD>& 
                                               HeadState<HD>* st, Visible vis) {
   constexpr int OT = HeadState<HD>::OT;
   bf16x8 pb[GT];
-  bool moved[GT];
-  float m_before[GT];
-#pragma unroll
-  for (int j = 0; j < GT; ++j) pb[j] = scores32<HD>(key0, g, kf, qf[j], c, masked, st[j], moved[j], m_before[j], vis);
+  const float over = kLazyLog2 / c;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
-    if (__any(moved[j])) {
+    float s[8];
+    const float mx = scores32<HD>(key0, g, kf, qf[j], masked, s, vis);
+    if (__any(mx > st[j].lim)) {
       asm volatile("" ::: "memory");  // keep this a branch: as selects it would cost a multiply per output every step
-      // 2^(-inf) = 0 for a column's first keys: its sums are zero anyway
-      const float alpha = moved[j] ? __builtin_amdgcn_exp2f((m_before[j] - st[j].m) * c) : 1.0f;
-#pragma unroll
-      for (int t = 0; t < OT; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) st[j].o[t][i] *= alpha;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) st[j].l[i] *= alpha;
+      move_reference<HD>(st[j], mx, c, over);
     }
+    pb[j] = probabilities(s, c, st[j].shift);
   }
   const bf16x8 ones = ones8();
 #pragma unroll
