@@ -378,6 +378,8 @@ MID_MIN_SLICES = 2
 MID_WIDE_ROWS = 65536
 MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns, half of it beyond
 MID_WIDE_SHORT_K = 4096
+MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
+MID_SLICED_LONG_K = 8192
 MID_PRODUCTS = True    # ``set_mid_products``: off sends these products where they went without this kernel (measurements)
 
 
@@ -462,14 +464,21 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise NativeError(f"linear: x {x.dtype} / w {w.dtype}")
     m, k = x.shape
+    n = w.shape[0]
+    # what a reader of slices gets from the product with X in LDS: from MID_SLICED_MIN_ROWS rows on where the rows are
+    # long (the streaming kernel sums such a row in one workgroup: [2560, 9728] with the norm behind it 20.2 us
+    # at 16 rows against 17.7 in four or eight slices, [5120, 25600] 60.4 against 50.6; at 8 rows and fewer it is
+    # the other way round), from 17 rows on everywhere
+    sliced = (MID_PRODUCTS and slices_ok and tiles is not None and k % 8 == 0 and n % 4 == 0 and m <= GEMM_MID_MAX_ROWS
+              and out_dtype in (None, torch.bfloat16)
+              and (m > SKINNY_MAX_ROWS or (m >= MID_SLICED_MIN_ROWS and k >= MID_SLICED_LONG_K)))
+    if sliced:
+        s = gemm_mid_slices(n, k)
+        if s >= MID_MIN_SLICES:
+            return gemm_mid(x, tiles, bias, slices=s)
     if m <= SKINNY_MAX_ROWS and k % 8 == 0:
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
     if MID_PRODUCTS and tiles is not None and k % 8 == 0 and m <= GEMM_MID_MAX_ROWS:
-        n = w.shape[0]
-        if slices_ok and n % 4 == 0 and out_dtype in (None, torch.bfloat16):
-            s = gemm_mid_slices(n, k)
-            if s >= MID_MIN_SLICES:
-                return gemm_mid(x, tiles, bias, slices=s)
         if n >= MID_WIDE_ROWS and m <= (MID_WIDE_MAX_M if k <= MID_WIDE_SHORT_K else MID_WIDE_MAX_M // 2):
             return gemm_mid(x, tiles, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
