@@ -77,12 +77,29 @@ def bench_gemm(dev, shape) -> None:
             x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
             us = timeit(lambda i: K.gemm_skinny(x, tiles[i], out_dtype=f32, silu_mul_epilogue=silu), copies)
             line(f"gemm {name} [{n}x{k}] M={m} tiled", us, nbytes=n * k * 2)
-        for m in (64, 2048):
+        # what the engine's dispatcher sends 32 to 128 rows to (the product with X staged in LDS where it measured
+        # faster: cut into slices of K for o and down, whose reader adds them; SiLU*up in its epilogue), and the
+        # library beside it
+        weights_of = [K.LinearWeight(r, t) for r, t in zip(rows, tiles)]
+        for m in (32, 64, 128):
             x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
-            us = timeit(lambda i: K.gemm_library(x, rows[i]), copies, iters=20)
-            line(f"gemm {name} [{n}x{k}] M={m} library", us, nbytes=n * k * 2 if m == 64 else 0.0,
-                 flops=2.0 * m * n * k if m > 64 else 0.0)
-        del rows, tiles
+            if silu:
+                us = timeit(lambda i: K.linear_silu_mul(x, weights_of[i]), copies, iters=20)
+            else:
+                us = timeit(lambda i: K.linear(x, weights_of[i], out_dtype=f32, slices_ok=name in ("o", "down")), copies, iters=20)
+            line(f"gemm {name} [{n}x{k}] M={m} as dispatched", us, nbytes=n * k * 2)
+            if silu:
+                us = timeit(lambda i: K.silu_mul(K.gemm_library(x, rows[i])), copies, iters=20)
+            elif f32 is not None:
+                us = timeit(lambda i: K.to_f32(K.gemm_library(x, rows[i])), copies, iters=20)
+            else:
+                us = timeit(lambda i: K.gemm_library(x, rows[i]), copies, iters=20)
+            line(f"gemm {name} [{n}x{k}] M={m} library" + (" + SiLU*up" if silu else " + widening" if f32 is not None else ""),
+                 us, nbytes=n * k * 2)
+        x = torch.randn(2048, k, device=dev, dtype=torch.bfloat16)
+        us = timeit(lambda i: K.gemm_library(x, rows[i]), copies, iters=20)
+        line(f"gemm {name} [{n}x{k}] M=2048 library", us, flops=2.0 * 2048 * n * k)
+        del rows, tiles, weights_of
 
 
 def bench_decode(dev, shape, page: int = 16) -> None:
