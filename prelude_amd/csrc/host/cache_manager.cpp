@@ -4,28 +4,118 @@
 
 namespace pa {
 
-PagePool::PagePool(int num_pages) : held_(num_pages > 0 ? num_pages : 0, 0) {
-  for (int i = 0; i < capacity(); ++i) free_.push_back(i);
+PagePool::PagePool(int num_pages, int run) : run_(run > 1 ? run : 1), held_(num_pages > 0 ? num_pages : 0, 0) {
+  const int n = capacity(), runs = (n + run_ - 1) / run_;
+  claim_.assign(n, kNobody);
+  stamp_.assign(n, 0);
+  unclaimed_free_.assign(runs, 0);
+  run_stamp_.assign(runs, 0);
+  free_count_ = n;
+  for (int i = 0; i < n; ++i) free_.push_back({i, 0});
+  for (int r = 0; r < runs; ++r) {
+    unclaimed_free_[r] = run_len(r);
+    runs_.push_back({r, 0});
+  }
 }
 
-int PagePool::take() {
-  if (free_.empty()) return -1;
-  int p = free_.front();
-  free_.pop_front();
-  held_[p] = 1;
-  return p;
+// A free page becomes a held one.
+void PagePool::grab(int page) {
+  if (claim_[page] == kNobody) --unclaimed_free_[page / run_];
+  claim_[page] = kNobody;
+  held_[page] = 1;
+  ++stamp_[page];   // its entry in free_ is void from now on
+  --free_count_;
+}
+
+// A page that is free has lost its claim, or has just become free: its run may be whole again.
+void PagePool::page_is_unclaimed_and_free(int page) {
+  const int r = page / run_;
+  if (++unclaimed_free_[r] == run_len(r) && run_ > 1) runs_.push_back({r, ++run_stamp_[r]});
+}
+
+int PagePool::take(int64_t owner, int after) {
+  if (free_count_ == 0) return -1;
+  if (run_ > 1) {
+    const int next = after + 1;
+    if (after >= 0 && next < capacity() && !held_[next] && (claim_[next] == kNobody || claim_[next] == owner)) {
+      grab(next);
+      return next;
+    }
+    while (!runs_.empty()) {
+      const Entry e = runs_.front();
+      runs_.pop_front();
+      if (e.stamp != run_stamp_[e.index] || unclaimed_free_[e.index] != run_len(e.index)) continue;
+      const int first = e.index * run_;
+      grab(first);
+      if (owner != kNobody) {
+        auto& mine = claims_of_[owner];
+        for (int p = first + 1; p < first + run_len(e.index); ++p) {
+          claim_[p] = owner;
+          --unclaimed_free_[e.index];
+          mine.push_back(p);
+        }
+      }
+      return first;
+    }
+  }
+  while (!free_.empty()) {
+    const Entry e = free_.front();
+    free_.pop_front();
+    if (e.stamp != stamp_[e.index] || held_[e.index]) continue;
+    grab(e.index);
+    return e.index;
+  }
+  return -1;   // not reached while free_count_ is right
 }
 
 bool PagePool::give(int page) {
   if (!held(page)) return false;
   held_[page] = 0;
-  free_.push_back(page);
+  ++free_count_;
+  free_.push_back({page, ++stamp_[page]});
+  page_is_unclaimed_and_free(page);
   return true;
+}
+
+void PagePool::release_claims(int64_t owner) {
+  auto it = claims_of_.find(owner);
+  if (it == claims_of_.end()) return;
+  for (int p : it->second) {
+    if (held_[p] || claim_[p] != owner) continue;   // taken since (by its owner or by someone in need)
+    claim_[p] = kNobody;
+    page_is_unclaimed_and_free(p);
+  }
+  claims_of_.erase(it);
+}
+
+std::string PagePool::check() const {
+  int free_pages = 0;
+  std::vector<int> count(unclaimed_free_.size(), 0);
+  for (int p = 0; p < capacity(); ++p) {
+    if (held_[p]) {
+      if (claim_[p] != kNobody) return "page " + std::to_string(p) + " is held and claimed";
+      continue;
+    }
+    ++free_pages;
+    if (claim_[p] == kNobody) ++count[p / run_];
+  }
+  if (free_pages != free_count_) return "the count of free pages is off";
+  for (size_t r = 0; r < count.size(); ++r)
+    if (count[r] != unclaimed_free_[r]) return "run " + std::to_string(r) + ": the count of unclaimed free pages is off";
+  // every free page can still be reached through the queue
+  std::vector<uint8_t> queued(capacity(), 0);
+  for (const Entry& e : free_)
+    if (e.stamp == stamp_[e.index] && !held_[e.index]) queued[e.index] = 1;
+  for (int p = 0; p < capacity(); ++p)
+    if (!held_[p] && !queued[p]) return "free page " + std::to_string(p) + " is in no queue";
+  return "";
 }
 
 CacheManager::CacheManager(int page_size, const std::vector<GroupSpec>& groups, int num_state_slots)
     : page_size_(page_size), groups_(groups), num_state_slots_(num_state_slots > 0 ? num_state_slots : 0) {
-  for (const auto& g : groups_) pools_.emplace_back(g.num_pages);
+  // runs of 128 tokens: what a request is given side by side where that is free (see PagePool)
+  const int run = page_size_ > 0 && page_size_ < 128 ? 128 / page_size_ : 1;
+  for (const auto& g : groups_) pools_.emplace_back(g.num_pages, run);
   slot_held_.assign(num_state_slots_, 0);
   for (int i = 0; i < num_state_slots_; ++i) free_slots_.push_back(i);
 }
@@ -142,7 +232,7 @@ int CacheManager::reserve(int64_t id, int new_len) {
   // inside what the portion writes: none of them can be skipped for a window.
   for (int g = 0; g < G; ++g) {
     auto& table = rc.tables[g];
-    while ((int)table.size() < want) table.push_back(pools_[g].take());
+    while ((int)table.size() < want) table.push_back(pools_[g].take(id, table.empty() ? -1 : table.back()));
   }
   rc.reserved_len = new_len;
   return 0;
@@ -192,9 +282,11 @@ bool CacheManager::close(int64_t id) {
     return false;
   }
   RequestCache& rc = it->second;
-  for (int g = 0; g < num_groups(); ++g)
+  for (int g = 0; g < num_groups(); ++g) {
     for (int p : rc.tables[g])
       if (p >= 0) pools_[g].give(p);
+    pools_[g].release_claims(id);
+  }
   if (rc.state_slot >= 0) {
     slot_held_[rc.state_slot] = 0;
     free_slots_.push_back(rc.state_slot);
@@ -277,6 +369,13 @@ std::string CacheManager::audit() const {
     }
     if (held + pools_[g].free_count() != pools_[g].capacity())
       return "group " + std::to_string(g) + ": free and held pages do not add up";
+    const std::string inside = pools_[g].check();
+    if (!inside.empty()) return "group " + std::to_string(g) + ": " + inside;
+    for (int p = 0; p < pools_[g].capacity(); ++p) {
+      const int64_t c = pools_[g].claimed_by(p);
+      if (c != PagePool::kNobody && !requests_.count(c))
+        return "group " + std::to_string(g) + ": page " + std::to_string(p) + " is kept for a request that is gone";
+    }
   }
   std::vector<int> slot_owner(num_state_slots_, 0);
   for (const auto& kv : requests_) {

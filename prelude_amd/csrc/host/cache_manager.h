@@ -3,12 +3,16 @@
 // passed, and a pool of slots for per-request state of fixed size.
 //
 // What the reference does and where: FIFO free list and slot arithmetic,
-// crates/prelude-core/src/scheduler/components/cache/block_manager.rs:12-109;
+// crates/prelude-core/src/scheduler/components/cache/block_manager.rs:12-109
+// (ours hands a growing request pages that lie side by side where it can,
+// and falls back to first-in first-out: see PagePool);
 // slots of fixed-size state, zeroed on allocation and freed with the pages,
 // crates/prelude-core/src/scheduler/components/cache/deltanet_pool.rs:54-173.
 // Ours: several groups with pages of their own, windows, all-or-nothing
 // reservation across groups, and the step's index arrays built here.
 #pragma once
+#include <algorithm>
+#include <climits>
 #include <cstdint>
 #include <deque>
 #include <string>
@@ -22,19 +26,53 @@ struct GroupSpec {
   int window = 0;  // keys a layer of this group looks back over, the query's own included; 0 = all
 };
 
-// A fixed set of pages handed out first-in first-out.
+// A fixed set of pages.  A page goes to whoever asks, first-in first-out, but a request's pages are kept in runs
+// where that costs nothing: the attention kernels read a request's pages in order, and pages that lie side by
+// side in memory stream faster than pages scattered over the pool (measured on an MI355X, 64 requests of 4,096
+// keys in pages of 16: 5.7 TB/s in order, 5.6 in runs of eight pages, 5.2 scattered; a decode step of 64 requests
+// whose contexts grew a page at a time in turn: 9.9 ms with runs, 10.6 without).  So a request that grows is
+// given, in this order:
+//   1. the page behind its last one, if that is free and no other request has a claim on it;
+//   2. the first page of a whole run of `run` pages (aligned, all free, none claimed), first-in first-out among
+//      such runs; the rest of the run is then claimed for it;
+//   3. the page that has been free the longest, whoever claims it.
+// A claim only orders the hand-out: a claimed page is free, counts as free, and is taken by anyone in step 3 when
+// nothing else is left, so the pool's capacity is what it would be without claims.  Claims end when their page is
+// taken or their request closes.
 class PagePool {
  public:
-  explicit PagePool(int num_pages);
+  static constexpr int64_t kNobody = INT64_MIN;
+  explicit PagePool(int num_pages, int run = 1);
   int capacity() const { return (int)held_.size(); }
-  int free_count() const { return (int)free_.size(); }
-  int take();             // -1 when empty
+  int free_count() const { return free_count_; }
+  int run() const { return run_; }
+  // A page for `owner`, whose last page is `after` (-1: none yet); -1 when the pool is empty.
+  int take(int64_t owner = kNobody, int after = -1);
   bool give(int page);    // false when the page is not held (never double-freed silently)
+  void release_claims(int64_t owner);
   bool held(int page) const { return page >= 0 && page < capacity() && held_[page]; }
+  int64_t claimed_by(int page) const { return page >= 0 && page < capacity() ? claim_[page] : kNobody; }
+  std::string check() const;   // "" or what is inconsistent
 
  private:
-  std::deque<int> free_;
+  struct Entry {
+    int index;        // a page (in free_) or a run (in runs_)
+    uint32_t stamp;   // valid while it equals the index's current stamp
+  };
+  int run_len(int r) const { return std::min(run_, capacity() - r * run_); }
+  void grab(int page);
+  void page_is_unclaimed_and_free(int page);
+
+  int run_;
+  int free_count_ = 0;
   std::vector<uint8_t> held_;
+  std::vector<int64_t> claim_;        // free page -> the request it is kept for, or kNobody
+  std::vector<uint32_t> stamp_;       // per page: bumped when it is queued and when it is taken
+  std::deque<Entry> free_;            // free pages in the order they became free (void entries are skipped)
+  std::vector<int> unclaimed_free_;   // per run: pages that are free and not claimed
+  std::vector<uint32_t> run_stamp_;   // per run: bumped when it is queued
+  std::deque<Entry> runs_;            // runs that were whole when queued (void entries are skipped)
+  std::unordered_map<int64_t, std::vector<int>> claims_of_;
 };
 
 struct RequestCache {

@@ -149,11 +149,68 @@ def test_step_arrays():
         _fill(t, [10], [8], [32])
 
 
-@pytest.mark.parametrize("seed", range(6))
+def runs_of(table):
+    """Lengths of the stretches of a table whose pages lie side by side in the pool."""
+    out, n = [], 0
+    for i, p in enumerate(table):
+        if i and p == table[i - 1] + 1:
+            n += 1
+        else:
+            if n:
+                out.append(n)
+            n = 1
+    return out + ([n] if n else [])
+
+
+def test_requests_that_grow_in_turn_get_their_pages_in_runs():
+    """Pages of 16 tokens are handed out in runs of 8 (128 tokens) where whole runs are free: four requests that
+    grow a page at a time, in turn, each end up with their pages side by side, not interleaved."""
+    t = PageTables(16, [(64, 0)])
+    for r in range(4):
+        t.open(r)
+    for n in range(1, 16):
+        for r in range(4):
+            t.reserve(r, 16 * n); t.commit(r, 16 * n)
+        assert t.audit() == ""
+    for r in range(4):
+        table = t.table(r, 0)
+        assert len(table) == 15 and runs_of(table) == [8, 7], table
+    assert t.free_pages(0) == 4                      # what the four keep in reserve is free all the same
+    # a fifth request finds no whole run: it is given the pages that have been free the longest, one by one,
+    # though each of them is kept for someone else -- and then the pool is empty, as it would be without runs
+    t.open(9); t.reserve(9, 64); t.commit(9, 64)
+    assert t.free_pages(0) == 0 and t.audit() == ""
+    with pytest.raises(OutOfPages):
+        t.reserve(0, 16 * 16)
+    t.close(9)
+    t.reserve(0, 16 * 16); t.commit(0, 16 * 16)      # the page behind its last one is free again: a run of 8 + 8
+    assert runs_of(t.table(0, 0)) == [8, 8]
+    for r in range(4):
+        t.close(r)
+    assert t.free_pages(0) == 64 and t.audit() == ""
+    # everything is free and unclaimed again: a new request gets whole runs from the start
+    t.open(5); t.reserve(5, 16 * 20); t.commit(5, 16 * 20)
+    assert max(runs_of(t.table(5, 0))) >= 8 and t.audit() == ""
+
+
+def test_a_request_that_ends_gives_up_what_was_kept_for_it():
+    t = PageTables(16, [(16, 0)])
+    t.open(1); t.reserve(1, 16); t.commit(1, 16)     # takes page 0, pages 1..7 are kept for it
+    t.open(2); t.reserve(2, 16); t.commit(2, 16)     # takes page 8, pages 9..15 are kept for it
+    assert t.table(1, 0) == [0] and t.table(2, 0) == [8]
+    t.close(1)                                       # run 0 is whole again
+    t.open(3); t.reserve(3, 48); t.commit(3, 48)
+    assert t.table(3, 0) == [0, 1, 2] and t.audit() == ""
+    t.reserve(2, 32); t.commit(2, 32)
+    assert t.table(2, 0) == [8, 9]
+
+
+@pytest.mark.parametrize("seed", range(10))
 def test_random_orders_lose_nothing(seed):
     rng = random.Random(seed)
     page = rng.choice([1, 4, 8, 16])
-    groups = [(rng.randint(6, 40), 0), (rng.randint(6, 40), rng.choice([3, 9, 20]))]
+    big = seed >= 6                                  # pools of several runs of 128 tokens
+    groups = [(rng.randint(6, 40) * (6 if big else 1), 0), (rng.randint(6, 40) * (6 if big else 1), rng.choice([3, 9, 20]))]
     t = PageTables(page, groups, state_slots=3)
     live = {}
     nxt = 0
@@ -166,7 +223,7 @@ def test_random_orders_lose_nothing(seed):
             nxt += 1
         elif op < 0.8 and live:
             rid = rng.choice(list(live))
-            n = rng.choice([1, 1, 1, 2, 5, 13, 30])
+            n = rng.choice([1, 1, 1, 2, 5, 13, 30] + ([70, 200] if big else []))
             before = [t.free_pages(g) for g in range(2)]
             try:
                 t.reserve(rid, live[rid] + n)
