@@ -515,6 +515,9 @@ def set_skinny_max_rows(n: int) -> None:
 # streaming kernel: 30 and 47 at 32 and 64); [24576, 4096] 37.6 at 64 rows against 47.7; [51200, 5120] stays with the
 # library (110 against 105 at 64 rows, 163 against 119 at 128).  The bounds below are for weights without tiles
 # for that kernel to read, and for measurements with it switched off.
+# Up to 16 rows the two kernels are close: [19456, 2560] takes the product with X in LDS 19.4 us at any number of rows
+# and the streaming kernel 18.7 at one row, 20.0 at 8, 23.2 at 16; [24576, 4096] 35.0 against 35.8 to 36.7
+GATED_MID_MIN_ROWS = 8         # ... for rows shorter than GATED_TILED_LONG_K columns; 1 for longer ones
 GATED_TILED_ROWS = 24          # ... and 32 for rows of GATED_TILED_LONG_K columns or more
 GATED_TILED_LONG_K = 4096
 GATED_TILED_ELEMENTS = 1 << 27
@@ -530,6 +533,9 @@ def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
     if x.dtype == torch.bfloat16 and k % 8 == 0:
         tiles = w.tiles if isinstance(w, LinearWeight) else None
         if m <= SKINNY_MAX_ROWS:
+            if (MID_PRODUCTS and tiles is not None and tiles.n * k <= GATED_TILED_ELEMENTS
+                    and m >= (GATED_MID_MIN_ROWS if k < GATED_TILED_LONG_K else 1)):
+                return gemm_mid(x, tiles, silu_mul_epilogue=True)
             if isinstance(w, LinearWeight):
                 w = tiles if tiles is not None and m <= 16 else w.rows
             return gemm_skinny(x, w, silu_mul_epilogue=True)

@@ -156,7 +156,10 @@ def test_gemm_skinny(gpu, m, n, k):
         if n % 2 == 0:
             tact = K().gemm_skinny(xd, tiles, silu_mul_epilogue=True)
             close(tact, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
-            assert torch.equal(K().linear_silu_mul(xd, lw), tact)
+            # the dispatcher's choice between this kernel and the one with X in LDS follows the shape and the rows
+            got = K().linear_silu_mul(xd, lw)
+            assert torch.equal(got, tact) or torch.equal(got, K().gemm_mid(xd, tiles, silu_mul_epilogue=True))
+            close(got, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
     else:                                # more rows from tiles: the same sums per row as with few rows
         many = K().gemm_skinny(xd, tiles, out_dtype=torch.float32)
         close(many, ref, torch.float32, f32=2e-5)
