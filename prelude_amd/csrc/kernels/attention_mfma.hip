@@ -86,9 +86,11 @@ constexpr float kLazyLog2 = 8.0f;
 template <int HD>
 struct HeadState {
   static constexpr int OT = HD / 16;
-  float m = -INFINITY;  // reference maximum of the raw scores, equal in the four lanes of a column
-  float lim = -INFINITY;  // a score above this moves m: m + kLazyLog2 / c
+  // The reference maximum m of the raw scores, equal in the four lanes of a column, is kept as what is made of it:
+  float lim = -INFINITY;  // a score above this moves m: m + kLazyLog2 / c (-inf while the column has seen no key)
   float shift = 0.f;      // -m c (0 while the column has seen no key): the exponent is s c + shift
+  // m c, the exponent's reference, as the merge of splits wants it
+  __device__ __forceinline__ float reference() const { return lim == -INFINITY ? -INFINITY : -shift; }
   f32x4 l;              // running sum of the column's probabilities (every element the same)
   f32x4 o[OT];          // O^T tiles: head_dim rows 16 t + 4g + i, column r
   __device__ HeadState() {
@@ -220,10 +222,9 @@ __device__ __forceinline__ void move_reference(HeadState<HD>& st, float mx_lane,
   constexpr int OT = HeadState<HD>::OT;
   const float mx = xor_max16_32(mx_lane);
   const bool moved = mx > st.lim;   // from -inf any finite score; -inf against -inf is false
-  // 2^(-inf) = 0 for a column's first keys: its sums are zero anyway
-  const float alpha = moved ? __builtin_amdgcn_exp2f((st.m - mx) * c) : 1.0f;
+  // 2^((m_before - mx) c); for a column's first keys m_before c counts as 0, and its sums are zero anyway
+  const float alpha = moved ? __builtin_amdgcn_exp2f(-st.shift - mx * c) : 1.0f;
   if (moved) {
-    st.m = mx;
     st.lim = mx + over;
     st.shift = -mx * c;
   }
@@ -504,7 +505,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   // merge the four wavefronts through LDS; maxima leave in the log2 domain (raw maximum times c)
   const float l_wave = st[0].l[0];
   if (g == 0) {
-    lds_ml[wave][r][0] = st[0].m * c;
+    lds_ml[wave][r][0] = st[0].reference();
     lds_ml[wave][r][1] = l_wave;
   }
 #pragma unroll
