@@ -13,7 +13,7 @@ the host prepares a step while the one before it runs, as the engine's
 generation loop does).
 One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is
 a 2,048-token prompt portion; ``roofline`` prices the decode step against HBM
-bandwidth; ``points`` holds batch 1 and 64 at the same context, batch 8 at a context of 32,768 tokens and the
+bandwidth; ``points`` holds batch 1, 32 and 64 at the same context, batch 8 at a context of 32,768 tokens and the
 prefill of 8,192 tokens in one step (tokens a second each).
 """
 from __future__ import annotations
@@ -233,7 +233,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 0.6B, 8B or 32B")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip the points at other batches and lengths")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone and print its record (for profiles)")
     ap.add_argument("--mixed", action="store_true",
@@ -316,7 +316,7 @@ def main() -> int:
                           "frac": round(flops / psec / MFMA_PEAK[short], 4)}
     if not args.no_points:
         pts = {}
-        for b in (1, 64):
+        for b in (1, 32, 64):   # 32: the products of 17 to 128 rows, where attention does not yet dominate the step
             s = decode_point(raw, args.dtype, b, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), None)
             pts[f"decode_b{b}"] = round(b / s, 2)
         if args.context == 4096 and args.batch == 8:
