@@ -27,7 +27,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--model-path", help="same as --model (the reference's flag for a local folder)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32", "bfloat16", "float32"])
     ap.add_argument("--device", default="cuda:0")
-    ap.add_argument("--random-weights", action="store_true", help="draw weights from --seed instead of loading them")
+    ap.add_argument("--random-weights", action="store_true", help="draw weights from --weights-seed instead of loading them")
     ap.add_argument("--weights-seed", type=int, default=0)
     ap.add_argument("--write-model", metavar="DIR", help="with --random-weights: write the model folder (config.json, "
                                                          "model.safetensors) there and load it from there")
