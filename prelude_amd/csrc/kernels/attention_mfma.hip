@@ -862,18 +862,30 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
 
   Stage<HD, 4 * HW> stage;
   const int lo_page = wg_lo >> page_shift, hi_page = (wg_hi - 1) >> page_shift;
+  // A block is put into LDS a whole block before it is used: while the wavefronts work on block b out of one
+  // buffer, each first writes its share of block b + 1 (asked for from memory a block ago) into the other and asks
+  // for block b + 2; the barrier at the block's end then says both that block b + 1 is complete and that nobody
+  // reads block b any more.  (Written right before its use, the LDS writes and the barrier stood between every
+  // block's arrival and its first product.)
   int key0 = (wg_lo / kStageKeys) * kStageKeys;
   stage.load_pages(w, key0, wave, lane, lo_page, hi_page);
   stage.load(w, wave, lane);
   if (key0 + kStageKeys < wg_hi) stage.load_pages(w, key0 + kStageKeys, wave, lane, lo_page, hi_page);
+  stage.store(lds, 0, wave, lane);
+  if (key0 + kStageKeys < wg_hi) {
+    stage.load(w, wave, lane);
+    if (key0 + 2 * kStageKeys < wg_hi) stage.load_pages(w, key0 + 2 * kStageKeys, wave, lane, lo_page, hi_page);
+  }
+  __syncthreads();
   int buf = 0;
   for (; key0 < wg_hi; key0 += kStageKeys, buf ^= 1) {
-    stage.store(lds, buf, wave, lane);
-    __syncthreads();
     if (key0 + kStageKeys < wg_hi) {
-      stage.load(w, wave, lane);   // the next block, from the pages looked up a block ago
-      if (key0 + 2 * kStageKeys < wg_hi)
-        stage.load_pages(w, key0 + 2 * kStageKeys, wave, lane, lo_page, hi_page);  // and the pages of the one after
+      stage.store(lds, buf ^ 1, wave, lane);   // the next block, asked for a block ago
+      if (key0 + 2 * kStageKeys < wg_hi) {
+        stage.load(w, wave, lane);             // the one after it, from the pages looked up a block ago
+        if (key0 + 3 * kStageKeys < wg_hi)
+          stage.load_pages(w, key0 + 3 * kStageKeys, wave, lane, lo_page, hi_page);
+      }
     }
     if (wave_on) {
 #pragma unroll
@@ -885,8 +897,9 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
                              [&](int key) { return key >= my_lo && key <= my_pos; });
       }
     }
+    __syncthreads();
   }
-  __syncthreads();  // the buffers are free for the next tile
+  // (the loop's last barrier leaves the buffers free for the next tile)
   if (!qvalid) return;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
