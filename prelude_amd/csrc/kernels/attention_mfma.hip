@@ -301,9 +301,9 @@ __device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int 
 }
 
 // ---------------------------------------------------------------------------
-// decode: grid (nkv * qtiles, splits, sequences), 4 wavefronts, each taking every fourth step of 32 keys
+// decode: grid (nkv * qtiles, splits, sequences), WAVES wavefronts (4, or 2 for small grids), each taking every
+// WAVES-th step of 32 keys
 // ---------------------------------------------------------------------------
-constexpr int kDecodeWaves = 4;
 
 // What the decode kernel needs to take the merged QKV projection as it leaves the product instead of queries
 // that have been through the QK-norm + RoPE kernel: it norms and rotates its own queries, and the workgroup
@@ -426,8 +426,8 @@ __device__ __forceinline__ void fused_load_q(const FusedQkv& f, const bf16* qrow
   }
 }
 
-template <int HD, bool FUSED>
-__global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
+template <int HD, bool FUSED, int WAVES>
+__global__ __launch_bounds__(WAVES* kWave, 12 / WAVES) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* kc, const bf16* vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
@@ -435,8 +435,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
     int split_keys, int max_splits, FusedQkv fq, int contiguous) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
-  __shared__ float lds_o[kDecodeWaves][16][HD + 1];
-  __shared__ float lds_ml[kDecodeWaves][16][2];
+  __shared__ float lds_o[WAVES][16][HD + 1];
+  __shared__ float lds_ml[WAVES][16][2];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int group = nh / nkv;
@@ -493,8 +493,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
   HeadState<HD> st[1];
   const int step0 = (sp * split_keys) / 32;  // splits start at multiples of 32 keys
   const int steps = split_keys / 32;
-  // a wavefront has two steps at most here: many wavefronts per SIMD hide the latency, not a prefetch
-  for (int i = wave; i < steps; i += kDecodeWaves) {
+  // a wavefront has two steps here (four with two wavefronts): many wavefronts per SIMD hide the latency, not a prefetch
+  for (int i = wave; i < steps; i += WAVES) {
     const int key0 = (step0 + i) * 32;
     if (key0 + 32 <= k_begin || key0 >= k_end) continue;
     KFrag<HD> kf;
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
     const bool masked = key0 < k_begin || key0 + 32 > k_end;
     attend32<HD, 1>(w, key0, g, r, kf, qf, c, masked, st, [&](int key) { return key >= k_begin && key < k_end; });
   }
-  // merge the four wavefronts through LDS; maxima leave in the log2 domain (raw maximum times c)
+  // merge the wavefronts through LDS; maxima leave in the log2 domain (raw maximum times c)
   const float l_wave = st[0].l[0];
   if (g == 0) {
     lds_ml[wave][r][0] = st[0].reference();
@@ -518,10 +518,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 3) void attn_decode_kernel(
     const int qi = e / HD, d = e % HD;
     float mm = lds_ml[0][qi][0];
 #pragma unroll
-    for (int v = 1; v < kDecodeWaves; ++v) mm = fmaxf(mm, lds_ml[v][qi][0]);
+    for (int v = 1; v < WAVES; ++v) mm = fmaxf(mm, lds_ml[v][qi][0]);
     float o = 0.f, l = 0.f;
 #pragma unroll
-    for (int v = 0; v < kDecodeWaves; ++v) {
+    for (int v = 0; v < WAVES; ++v) {
       const float f = lds_ml[v][qi][0] == -INFINITY ? 0.f : exp2f(lds_ml[v][qi][0] - mm);
       o += lds_o[v][qi][d] * f;
       l += lds_ml[v][qi][1] * f;
@@ -959,10 +959,23 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   const int contiguous = total <= 1024;
   dim3 grid(nkv * qtiles, max_splits, nseq);
   if (contiguous) grid = dim3((unsigned)total, 1, 1);
-  hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED>), grid, dim3(kDecodeWaves * kWave), 0, st, (const bf16*)q,
-                     (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens,
-                     (bf16*)out, part_o, part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits,
-                     fq, contiguous);
+  // Three workgroups of four wavefronts fit a compute unit, 768 the chip.  A grid just above that (batch 7 and 8 at
+  // 4,096 keys) would run a second, nearly empty round; with two wavefronts a workgroup six fit and the whole grid is on
+  // the chip at once: +1.5 % of the decode step there.  Smaller grids want the four wavefronts for their parallelism
+  // (batch 1: -3.7 % with two), larger ones measured 1 to 3 % slower with two, with or without the mapping above.
+  // With two wavefronts a split's steps are added in another order (wavefront w takes the steps w, w + 2, .. instead
+  // of w, w + 4, ..), so a token's sums can differ in their last bits between steps whose grids fall on either side
+  // of these limits; what else is in the batch changes nothing beyond that.
+  const bool two_wavefronts = total > 768 && total <= 1024;
+  if (two_wavefronts) {
+    hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 2>), grid, dim3(2 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
+                       (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
+                       part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits, fq, contiguous);
+  } else {
+    hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 4>), grid, dim3(4 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
+                       (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
+                       part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits, fq, contiguous);
+  }
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
     // a group for every run of 64 splits the longest context can have, eight at most

@@ -682,6 +682,18 @@ def test_decode_attention_of_single_tokens_only(gpu, nh, nkv, hd, page, window):
     close(out, ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window,seqs", [
+    (32, 8, 128, 16, 0, [(4096, 1), (4095, 1), (3841, 1), (3840, 1), (2000, 1), (300, 1), (1, 1)]),     # 8 x 16 x 7 = 896
+    (16, 4, 64, 32, 700, [(8192, 1), (8000, 1), (7937, 1), (7936, 1), (100, 1), (257, 1), (5000, 1), (31, 1)]),   # 4 x 32 x 8 = 1,024
+    (3, 3, 48, 8, 0, [(16384, 1), (16129, 1), (2, 1), (9000, 1)])])                                      # 3 x 64 x 4 = 768: four wavefronts
+def test_decode_attention_in_grids_that_run_with_two_wavefronts(gpu, nh, nkv, hd, page, window, seqs):
+    """Grids of 769 to 1,024 workgroups run with two wavefronts a workgroup, each taking every second step of a
+    split; the last case lies at the edge and keeps four."""
+    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=6, kernel="mfma")
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.bfloat16)
+
+
 def draw_attention_case(seed: int):
     rng = np.random.default_rng(seed)
     hd = int(rng.choice([16, 32, 48, 64, 96, 128]))
@@ -728,16 +740,18 @@ def test_mfma_attention_batch_and_page_independence(gpu):
     assert torch.equal(one, other)                               # other page size, other pages
 
 
-@pytest.mark.parametrize("nh,nkv,hd,page,window,norm", [(32, 8, 128, 16, 0, True), (8, 8, 64, 8, 0, True), (16, 1, 128, 64, 40, True),
-                                                        (4, 2, 64, 16, 0, False)])
-def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, window, norm):
+@pytest.mark.parametrize("nh,nkv,hd,page,window,norm,ctxs", [
+    (32, 8, 128, 16, 0, True, [1, 17, 256, 257, 700, 33, 512]), (8, 8, 64, 8, 0, True, [1, 17, 256, 257, 700, 33, 512]),
+    (16, 1, 128, 64, 40, True, [1, 17, 256, 257, 700, 33, 512]), (4, 2, 64, 16, 0, False, [1, 17, 256, 257, 700, 33, 512]),
+    # 8 KV heads, 16 splits and 7 listed sequences: 896 workgroups, a grid that runs with two wavefronts a workgroup
+    (32, 8, 128, 16, 0, True, [4096, 3841, 3840, 2000, 300, 33, 1, 4095])])
+def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, window, norm, ctxs):
     """QK-norm, rotation, cache write and split attention in one kernel against the two kernels one after the
     other: the same outputs and the same keys and values in the cache, for contexts that end at a page's first
     and last place and at a split's edge; sequences outside the list are left alone."""
     eps = 1e-6
-    ctxs = [1, 17, 256, 257, 700, 33, 512]             # 33: a sequence that is not in the list
-    listed = [0, 1, 2, 3, 4, 6]
     t = len(ctxs)
+    listed = [i for i in range(t) if i != 5]           # the sixth sequence is not in the list
     g = torch.Generator().manual_seed(3)
     total_pages = sum(-(-c // page) for c in ctxs) + 2
     perm = torch.randperm(total_pages, generator=g).tolist()
@@ -750,15 +764,15 @@ def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, windo
         for p in range(-(-c // page)):
             table[i, p] = perm.pop()
         hist = c - 1                                   # keys before the token's own
-        for pos in range(hist):
-            ph = int(table[i, pos // page])
-            kc[ph, :, pos % page] = torch.randn(nkv, hd, generator=g).to(torch.bfloat16)
-            vc[ph, :, :, pos % page] = torch.randn(nkv, hd, generator=g).to(torch.bfloat16)
+        for p in range(-(-hist // page)):
+            n, ph = min(page, hist - p * page), int(table[i, p])
+            kc[ph, :, :n] = torch.randn(nkv, n, hd, generator=g).to(torch.bfloat16)
+            vc[ph, :, :, :n] = torch.randn(nkv, hd, n, generator=g).to(torch.bfloat16)
         slots.append(int(table[i, (c - 1) // page]) * page + (c - 1) % page)
     qkv = (2.0 * torch.randn(t, (nh + 2 * nkv) * hd, generator=g)).to(torch.bfloat16)
     qw = (1.0 + 0.2 * rnd(hd, seed=1)) if norm else None
     kw = (1.0 + 0.2 * rnd(hd, seed=2)) if norm else None
-    cos, sin = pm.rope_tables(hd, 1024, 10000.0, torch.float32)
+    cos, sin = pm.rope_tables(hd, max(ctxs), 10000.0, torch.float32)
     dev = lambda x: None if x is None else x.to(gpu)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
     pos, sl, seqs, cu, cl = i32([c - 1 for c in ctxs]), i32(slots), i32(listed), i32(list(range(t + 1))), i32(ctxs)
