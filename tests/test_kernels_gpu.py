@@ -732,6 +732,46 @@ def test_drawn_attention(gpu, seed):
     assert err <= tol(torch.float32, ref, f32=3e-6), f"{what}: 32-bit kernel, max error {err:.3e}"
 
 
+def draw_two_wavefront_case(seed: int):
+    """A step of single tokens whose grid (KV heads x splits of the longest context x sequences) has 769 to 1,024
+    workgroups."""
+    rng = np.random.default_rng(1000 + seed)
+    while True:
+        hd = int(rng.choice([16, 32, 48, 64, 96, 128]))
+        nkv = int(rng.choice([1, 2, 3, 4, 8]))
+        group = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        page = int(rng.choice([4, 8, 16, 32, 64, 128]))
+        nseq = int(rng.integers(2, 11))
+        window = int(rng.choice([0, 0, 0, int(rng.integers(300, 4000))]))
+        lo, hi = 768 // (nkv * nseq) + 1, 1024 // (nkv * nseq)     # numbers of splits that land in the range
+        if lo > hi or hi > 64 or lo < 2:
+            continue
+        splits = int(rng.integers(lo, hi + 1))
+        if window:      # a windowed sequence has the splits its window touches, one more than the window's own
+            if splits < 3:
+                continue
+            window = (splits - 3) * 256 + int(rng.integers(1, 257))
+            longest = window + 256 + int(rng.integers(0, 3000))
+        else:
+            longest = (splits - 1) * 256 + int(rng.integers(1, 257))
+        ctxs = [longest] + [int(rng.integers(1, longest + 1)) for _ in range(nseq - 1)]
+        rng.shuffle(ctxs)
+        span = min(longest, window + 256) if window else longest           # as the launcher counts the splits
+        grid = nkv * (-(-span // 256) + (1 if window else 0)) * nseq
+        return nkv * group, nkv, hd, page, window, [(int(c), 1) for c in ctxs], grid
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_ATTENTION", "10")))))   # widen for a hunt
+def test_drawn_attention_in_grids_of_two_wavefronts(gpu, seed):
+    nh, nkv, hd, page, window, seqs, grid = draw_two_wavefront_case(seed)
+    assert 768 < grid <= 1024
+    what = f"seed {seed}: {nh} heads over {nkv}, head_dim {hd}, page {page}, window {window}, (context, new) {seqs}"
+    out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=seed, kernel="mfma")
+    assert not bool(torch.isnan(out).any()), what
+    err = float((out.double().cpu() - ref).abs().max())
+    assert err <= tol(torch.bfloat16, ref), f"{what}: max error {err:.3e}"
+
+
 def test_mfma_attention_batch_and_page_independence(gpu):
     one, _ = paged_case(gpu, torch.bfloat16, 8, 2, 128, 16, [(900, 1)], 0, seed=5, kernel="mfma")
     many, _ = paged_case(gpu, torch.bfloat16, 8, 2, 128, 16, [(900, 1), (40, 1), (300, 30)], 0, seed=5, kernel="mfma")
