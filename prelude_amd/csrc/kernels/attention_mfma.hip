@@ -427,7 +427,7 @@ __device__ __forceinline__ void fused_load_q(const FusedQkv& f, const bf16* qrow
 }
 
 template <int HD, bool FUSED, int WAVES>
-__global__ __launch_bounds__(WAVES* kWave, 12 / WAVES) void attn_decode_kernel(
+__global__ __launch_bounds__(WAVES* kWave, 3) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* kc, const bf16* vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
@@ -952,21 +952,21 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
                   float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_shift, int window, float scale,
                   int split_keys, int max_splits, const FusedQkv& fq) {
   const int qtiles = (nh / nkv + 15) / 16;
-  // Up to 1,024 workgroups (a little more than the chip holds at once) each XCD gets a contiguous stretch of them;
-  // measured in the decode step of a 4B model: batch 8 at 4,096 keys +0.9 %, batch 2 at 16,384 +0.3 %, while larger
-  // grids do better dealt out plainly (batch 64 at 4,096: +3.5 %, batch 8 at 8,192: +0.5 %, batch 16 to 32: equal)
+  // Up to 1,536 workgroups (what the chip holds at once, below) each XCD gets a contiguous stretch of them; measured
+  // in the decode step of a 4B model: batch 8 at 4,096 keys +0.9 %, batch 9 to 12 +0.8 to 1.2 %, batch 2 at 16,384
+  // +0.3 %, while larger grids do better dealt out plainly (batch 64 at 4,096: +3.5 %, batch 16 to 32: equal)
   const long total = (long)nkv * qtiles * max_splits * nseq;
-  const int contiguous = total <= 1024;
+  const int contiguous = total <= 1536;
   dim3 grid(nkv * qtiles, max_splits, nseq);
   if (contiguous) grid = dim3((unsigned)total, 1, 1);
-  // Three workgroups of four wavefronts fit a compute unit, 768 the chip.  A grid just above that (batch 7 and 8 at
-  // 4,096 keys) would run a second, nearly empty round; with two wavefronts a workgroup six fit and the whole grid is on
-  // the chip at once: +1.5 % of the decode step there.  Smaller grids want the four wavefronts for their parallelism
-  // (batch 1: -3.7 % with two), larger ones measured 1 to 3 % slower with two, with or without the mapping above.
-  // With two wavefronts a split's steps are added in another order (wavefront w takes the steps w, w + 2, .. instead
-  // of w, w + 4, ..), so a token's sums can differ in their last bits between steps whose grids fall on either side
-  // of these limits; what else is in the batch changes nothing beyond that.
-  const bool two_wavefronts = total > 768 && total <= 1024;
+  // Twelve wavefronts fit a compute unit (three a SIMD by their registers): three workgroups of four, 768 on the
+  // chip.  A grid just above that would run a second, nearly empty round; with two wavefronts a workgroup six fit,
+  // 1,536 on the chip, and the whole grid is there at once: batch 7 to 12 at 4,096 keys +0.3 to 2.3 % of the decode
+  // step.  Smaller grids want the four wavefronts for their parallelism (batch 1: -3.7 % with two), larger ones
+  // measured 1 to 2 % slower with two.  With two wavefronts a split's steps are added in another order (wavefront w
+  // takes the steps w, w + 2, .. instead of w, w + 4, ..), so a token's sums can differ in their last bits between
+  // steps whose grids fall on either side of these limits; what else is in the batch changes nothing beyond that.
+  const bool two_wavefronts = total > 768 && total <= 1536;
   if (two_wavefronts) {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 2>), grid, dim3(2 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,

@@ -684,10 +684,13 @@ def test_decode_attention_of_single_tokens_only(gpu, nh, nkv, hd, page, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,window,seqs", [
     (32, 8, 128, 16, 0, [(4096, 1), (4095, 1), (3841, 1), (3840, 1), (2000, 1), (300, 1), (1, 1)]),     # 8 x 16 x 7 = 896
-    (16, 4, 64, 32, 700, [(8192, 1), (8000, 1), (7937, 1), (7936, 1), (100, 1), (257, 1), (5000, 1), (31, 1)]),   # 4 x 32 x 8 = 1,024
+    (16, 4, 64, 32, 700, [(8192, 1), (8000, 1), (7937, 1), (7936, 1), (100, 1), (257, 1), (5000, 1), (31, 1)]),   # 4 x 5 x 8 = 160: four
+    (16, 4, 64, 32, 0, [(8192, 1), (8000, 1), (7937, 1), (7936, 1), (100, 1), (257, 1), (5000, 1), (31, 1)]),     # 4 x 32 x 8 = 1,024
+    (8, 2, 128, 16, 0, [(12288, 1), (12033, 1), (12032, 1), (1, 1), (256, 1), (6000, 1), (11000, 1), (9999, 1),
+                        (77, 1), (4096, 1), (12287, 1), (513, 1), (10000, 1), (2222, 1), (8191, 1), (300, 1)]),   # 2 x 48 x 16 = 1,536
     (3, 3, 48, 8, 0, [(16384, 1), (16129, 1), (2, 1), (9000, 1)])])                                      # 3 x 64 x 4 = 768: four wavefronts
 def test_decode_attention_in_grids_that_run_with_two_wavefronts(gpu, nh, nkv, hd, page, window, seqs):
-    """Grids of 769 to 1,024 workgroups run with two wavefronts a workgroup, each taking every second step of a
+    """Grids of 769 to 1,536 workgroups run with two wavefronts a workgroup, each taking every second step of a
     split; the last case lies at the edge and keeps four."""
     out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=6, kernel="mfma")
     assert not bool(torch.isnan(out).any())
@@ -733,7 +736,7 @@ def test_drawn_attention(gpu, seed):
 
 
 def draw_two_wavefront_case(seed: int):
-    """A step of single tokens whose grid (KV heads x splits of the longest context x sequences) has 769 to 1,024
+    """A step of single tokens whose grid (KV heads x splits of the longest context x sequences) has 769 to 1,536
     workgroups."""
     rng = np.random.default_rng(1000 + seed)
     while True:
@@ -743,7 +746,7 @@ def draw_two_wavefront_case(seed: int):
         page = int(rng.choice([4, 8, 16, 32, 64, 128]))
         nseq = int(rng.integers(2, 11))
         window = int(rng.choice([0, 0, 0, int(rng.integers(300, 4000))]))
-        lo, hi = 768 // (nkv * nseq) + 1, 1024 // (nkv * nseq)     # numbers of splits that land in the range
+        lo, hi = 768 // (nkv * nseq) + 1, 1536 // (nkv * nseq)     # numbers of splits that land in the range
         if lo > hi or hi > 64 or lo < 2:
             continue
         splits = int(rng.integers(lo, hi + 1))
@@ -764,7 +767,7 @@ def draw_two_wavefront_case(seed: int):
 @pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_ATTENTION", "10")))))   # widen for a hunt
 def test_drawn_attention_in_grids_of_two_wavefronts(gpu, seed):
     nh, nkv, hd, page, window, seqs, grid = draw_two_wavefront_case(seed)
-    assert 768 < grid <= 1024
+    assert 768 < grid <= 1536
     what = f"seed {seed}: {nh} heads over {nkv}, head_dim {hd}, page {page}, window {window}, (context, new) {seqs}"
     out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=seed, kernel="mfma")
     assert not bool(torch.isnan(out).any()), what
