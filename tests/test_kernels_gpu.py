@@ -792,6 +792,27 @@ def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, windo
     """QK-norm, rotation, cache write and split attention in one kernel against the two kernels one after the
     other: the same outputs and the same keys and values in the cache, for contexts that end at a page's first
     and last place and at a split's edge; sequences outside the list are left alone."""
+    raw_projection_case(gpu, nh, nkv, hd, page, window, norm, ctxs)
+    assert not K().attention_decode_fused_supported(nh, nkv, hd, hd // 2, page)      # partial rotation
+    assert not K().attention_decode_fused_supported(34, 2, 128, 128, 16)             # more than 16 heads per KV head
+    assert not K().attention_decode_fused_supported(4, 2, 96, 96, 16)
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_ATTENTION", "10")) // 2)))
+def test_drawn_raw_projection_in_grids_of_two_wavefronts(gpu, seed):
+    """The one-kernel form in grids of 769 to 1,536 workgroups, drawn: it has a two-wavefront variant of its own."""
+    s = seed
+    while True:
+        nh, nkv, hd, page, window, seqs, grid = draw_two_wavefront_case(10_000 + s)
+        if hd in (64, 128) and nh // nkv <= 16 and page >= 8 and len(seqs) >= 5:
+            break
+        s += 1000
+    ctxs = [c for c, _ in seqs]
+    ctxs.insert(5, 33)       # the case leaves its sixth sequence out of the step: one that does not count in the grid
+    raw_projection_case(gpu, nh, nkv, hd, page, window, bool(seed % 2), ctxs)
+
+
+def raw_projection_case(gpu, nh, nkv, hd, page, window, norm, ctxs):
     eps = 1e-6
     t = len(ctxs)
     listed = [i for i in range(t) if i != 5]           # the sixth sequence is not in the list
@@ -845,9 +866,6 @@ def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, windo
     assert torch.equal(k2.cpu()[mask[:, None, :].expand(total_pages, nkv, page)], kc[mask[:, None, :].expand(total_pages, nkv, page)])
     assert torch.equal(v2.cpu().transpose(2, 3)[mask[:, None, :].expand(total_pages, nkv, page)],
                        vc.transpose(2, 3)[mask[:, None, :].expand(total_pages, nkv, page)])
-    assert not K().attention_decode_fused_supported(nh, nkv, hd, hd // 2, page)      # partial rotation
-    assert not K().attention_decode_fused_supported(34, 2, 128, 128, 16)             # more than 16 heads per KV head
-    assert not K().attention_decode_fused_supported(4, 2, 96, 96, 16)
 
 
 def test_mfma_attention_refuses_what_it_does_not_take(gpu):
