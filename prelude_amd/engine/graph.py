@@ -44,7 +44,6 @@ class _Captured:
 
 
 class DecodeGraphs:
-    STRIDE_STEP_TOKENS = 1024   # table widths are rounded up to this many tokens
 
     def __init__(self, engine, max_batch: int, cache_size: int = 32):
         self.engine = engine
@@ -65,10 +64,11 @@ class DecodeGraphs:
         return any(t is g.logits for g in self._graphs.values())
 
     def _stride_for(self, ends: Sequence[int]) -> int:
+        # the bound the decode kernels round a step's longest context to anyway: a replayed step is then launched
+        # exactly as the same step run directly would be
+        from ..ops import kernels as K
         page = self.engine.page_size
-        step = max(1, self.STRIDE_STEP_TOKENS // page)
-        need = -(-max(ends) // page)
-        return -(-need // step) * step
+        return K.decode_context_bound(max(ends), page) // page
 
     def run(self, entries: Sequence, starts: Sequence[int], carried=None) -> torch.Tensor:
         eng = self.engine

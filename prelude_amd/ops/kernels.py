@@ -585,6 +585,23 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 
 
 DECODE_SPLIT_KEYS = 256   # keys per split of the decode kernel: fixed, so a token's result never depends on its batch
+DECODE_CONTEXT_STEP = 1024   # the longest context of a step counts rounded up to this many tokens (whole pages)
+
+
+def decode_context_bound(max_context: int, page_size: int) -> int:
+    """The longest context of a step of single tokens, rounded up: the number of splits the decode kernels are
+    launched for follows this bound and not the context itself, and so do the choices that follow the grid's size
+    (wavefronts a workgroup, groups of the merge), which change a sum's last bits.  A step replayed from a graph
+    knows only such a bound (the width of its block tables); with the same rounding a step run directly is launched
+    alike and gives the same bits."""
+    step = max(1, DECODE_CONTEXT_STEP // page_size) * page_size
+    return -(-max(int(max_context), 1) // step) * step
+
+
+def _decode_splits(max_context: int, window: int, page_size: int) -> int:
+    bound = decode_context_bound(max_context, page_size)
+    span = min(bound, window + DECODE_SPLIT_KEYS) if window else bound
+    return max(1, -(-span // DECODE_SPLIT_KEYS) + (1 if window else 0))
 
 
 def mfma_attention_supported(head_dim: int, page_size: int) -> bool:
@@ -602,8 +619,7 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_le
     n = seq_ids.shape[0]
     if n == 0:
         return
-    span = min(max_context, window + DECODE_SPLIT_KEYS) if window else max_context
-    max_splits = max(1, -(-span // DECODE_SPLIT_KEYS) + (1 if window else 0))
+    max_splits = _decode_splits(max_context, window, k_cache.shape[2])
     words = kernels().pa_attn_decode_workspace(n, nh, hd, max_splits)
     ws = torch.empty((max(words, 1),), dtype=torch.float32, device=q.device)
     check(kernels().pa_attn_decode(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
@@ -641,8 +657,7 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
     n = seq_ids.shape[0]
     if n == 0:
         return out
-    span = min(max_context, window + DECODE_SPLIT_KEYS) if window else max_context
-    max_splits = max(1, -(-span // DECODE_SPLIT_KEYS) + (1 if window else 0))
+    max_splits = _decode_splits(max_context, window, page)
     words = kernels().pa_attn_decode_workspace(n, nh, hd, max_splits)
     ws = torch.empty((max(words, 1),), dtype=torch.float32, device=qkv.device)
     check(kernels().pa_attn_decode_fused(_stream(), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin),

@@ -737,7 +737,8 @@ def test_drawn_attention(gpu, seed):
 
 def draw_two_wavefront_case(seed: int):
     """A step of single tokens whose grid (KV heads x splits of the longest context x sequences) has 769 to 1,536
-    workgroups."""
+    workgroups.  The splits are counted as the launcher counts them: from the longest context rounded up."""
+    from prelude_amd.ops.kernels import decode_context_bound
     rng = np.random.default_rng(1000 + seed)
     while True:
         hd = int(rng.choice([16, 32, 48, 64, 96, 128]))
@@ -745,22 +746,17 @@ def draw_two_wavefront_case(seed: int):
         group = int(rng.choice([1, 2, 3, 4, 8, 16]))
         page = int(rng.choice([4, 8, 16, 32, 64, 128]))
         nseq = int(rng.integers(2, 11))
-        window = int(rng.choice([0, 0, 0, int(rng.integers(300, 4000))]))
-        lo, hi = 768 // (nkv * nseq) + 1, 1536 // (nkv * nseq)     # numbers of splits that land in the range
-        if lo > hi or hi > 64 or lo < 2:
+        longest = int(rng.integers(300, 16385))
+        window = int(rng.choice([0, 0, 0, int(rng.integers(300, 8000))]))
+        if window >= longest:
+            window = 0
+        bound = decode_context_bound(longest, page)
+        span = min(bound, window + 256) if window else bound
+        grid = nkv * (-(-span // 256) + (1 if window else 0)) * nseq
+        if not 768 < grid <= 1536:
             continue
-        splits = int(rng.integers(lo, hi + 1))
-        if window:      # a windowed sequence has the splits its window touches, one more than the window's own
-            if splits < 3:
-                continue
-            window = (splits - 3) * 256 + int(rng.integers(1, 257))
-            longest = window + 256 + int(rng.integers(0, 3000))
-        else:
-            longest = (splits - 1) * 256 + int(rng.integers(1, 257))
         ctxs = [longest] + [int(rng.integers(1, longest + 1)) for _ in range(nseq - 1)]
         rng.shuffle(ctxs)
-        span = min(longest, window + 256) if window else longest           # as the launcher counts the splits
-        grid = nkv * (-(-span // 256) + (1 if window else 0)) * nseq
         return nkv * group, nkv, hd, page, window, [(int(c), 1) for c in ctxs], grid
 
 

@@ -289,6 +289,40 @@ def test_graph_replays_equal_eager_steps(gpu):
         assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
 
 
+def test_graph_replays_equal_eager_steps_where_the_grid_sets_the_wavefronts(gpu):
+    """The decode attention runs grids of 769 to 1,536 workgroups with two wavefronts a workgroup, which add a
+    split's steps in another order than four.  A replayed step knows its longest context only as a bound (the
+    width of its block tables), so a step run directly counts its splits from the same bound: five requests of 8
+    KV heads at some 4,200 tokens are 8 x 17 x 5 = 680 workgroups by their lengths and 8 x 20 x 5 = 800 by the
+    bound.  Replay and direct run give the same bits there too."""
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    import plain_model as pm
+    cfg = dict(pm.tiny_config_b(), num_attention_heads=8, num_key_value_heads=8, head_dim=64, num_hidden_layers=1,
+               max_position_embeddings=4400, vocab_size=200, eos_token_id=199)
+    rng = np.random.default_rng(9)
+    lens = [4200, 4150, 3000, 4199, 500]
+    seqs = [rng.integers(0, cfg["vocab_size"], size=n + 6).tolist() for n in lens]
+
+    def play(hip_graph):
+        eng = Engine.from_config(cfg, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=5 * 4416,
+                                                   hip_graph=hip_graph), seed=4, std=0.05)
+        outs = []
+        for r, n in enumerate(lens):
+            for lo in range(0, n, 2048):
+                hi = min(n, lo + 2048)
+                eng.step([StepEntry(r, seqs[r][lo:hi], [])])
+        for k in range(6):
+            outs.append(eng.step([StepEntry(r, [seqs[r][n + k]], [0]) for r, n in enumerate(lens)]).cpu())
+        return eng, outs
+
+    eager_eng, eager = play(False)
+    graph_eng, graphed = play(True)
+    assert eager_eng._graphs is None and graph_eng._graphs.replays == 6
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
+
+
 def test_graph_replays_with_library_products_equal_eager_steps(gpu):
     """A decode step of more than 48 requests multiplies through the library product, also inside a captured
     graph (with its workspace): every replay, with eager steps of other shapes between them, gives the eager
