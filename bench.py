@@ -193,14 +193,15 @@ def time_mixed(raw, dtype, chunk, decoding, context, steps, warmup):
     return sum(times[warmup:]) / steps
 
 
-def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency):
+def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency, **cfg_overrides):
     """`requests` prompts of `prompt_len` random tokens, `max_tokens` new tokens each, through an LLM session
     that is kept at `concurrency` requests: whenever one ends the next is added, as a load generator with that
     many clients does (the reference's published workload is this with one new token, over HTTP).
     Returns (seconds in all, sorted list of seconds from a request's arrival to its end)."""
     import numpy as np
     from prelude_amd import LLM, SamplingParams
-    eng = build_engine(raw, dtype, cache_tokens=min(requests, max(concurrency, 16)) * (prompt_len + max_tokens + 64))
+    eng = build_engine(raw, dtype, cache_tokens=min(requests, max(concurrency, 16)) * (prompt_len + max_tokens + 64),
+                       **cfg_overrides)
     llm = LLM.from_engine(eng)
     rng = np.random.default_rng(5)
     prompts = [rng.integers(0, raw["vocab_size"] - 1000, size=prompt_len).tolist() for _ in range(requests)]
@@ -243,6 +244,9 @@ def main() -> int:
                     help="time this many prompts (--prompt-len tokens, --new-tokens new tokens each) through "
                          "LLM.generate, --concurrency at a time, and print the record")
     ap.add_argument("--concurrency", type=int, default=96)
+    ap.add_argument("--graph-portion-tokens", type=int, default=None,
+                    help="--requests: steps with prompt portions of up to this many tokens are replayed from graphs "
+                         "(0: never; default: the engine's own)")
     ap.add_argument("--prompt-len", type=int, default=512, help="prompt length of --requests")
     ap.add_argument("--new-tokens", type=int, default=1, help="new tokens per request of --requests")
     args = ap.parse_args()
@@ -268,8 +272,9 @@ def main() -> int:
               flush=True)
         return 0
     if args.requests:
+        over = {} if args.graph_portion_tokens is None else {"hip_graph_portion_tokens": args.graph_portion_tokens}
         total, calls, firsts = time_requests(raw, args.dtype, args.requests, args.prompt_len, args.new_tokens,
-                                             args.concurrency)
+                                             args.concurrency, **over)
         mean = lambda v: sum(v) / len(v)
         tpot = (mean(calls) - mean(firsts)) / max(args.new_tokens - 1, 1)
         print(json.dumps({"model": name, "workload": f"{args.requests} prompts of {args.prompt_len} tokens, "

@@ -30,6 +30,9 @@ class EngineConfig:
     hip_graph: bool = True
     hip_graph_max_bs: int = 64
     hip_graph_cache_size: int = 32          # captured graphs kept (one per batch size and table width); the least recently used goes
+    # steps that bring prompt portions are replayed from a graph too when they are small (at most this many tokens:
+    # there the host's launches take longer than the kernels) and their shape has been met before; 0: never
+    hip_graph_portion_tokens: int = 1024
     # a second copy of every bfloat16 weight matrix, in the tiles the few-row product streams fastest
     # (decode steps run about a tenth faster for twice the weight memory)
     weight_tiles: bool = True

@@ -94,7 +94,8 @@ class Engine:
         # decode steps as HIP graphs, in the serving type, for models none of whose parts says it cannot be replayed
         if config.hip_graph and model.graph_safe and self.dtype == torch.bfloat16:
             from .graph import DecodeGraphs
-            self._graphs = DecodeGraphs(self, config.hip_graph_max_bs, config.hip_graph_cache_size)
+            self._graphs = DecodeGraphs(self, config.hip_graph_max_bs, config.hip_graph_cache_size,
+                                        self._graph_portion_tokens())
 
     def _chunk_cap(self) -> int:
         """The most tokens of one request a step may bring."""
@@ -151,6 +152,14 @@ class Engine:
         load_random(model, config.torch_dtype(), device, seed, std, norm_std)
         return cls(model, config, dict(raw_config))
 
+    def _graph_portion_tokens(self) -> int:
+        """Up to how many tokens a step with portions is replayed from a graph (0: such steps never are)."""
+        from .graph import portion_tokens_worth_a_graph
+        if not (self.config.hip_graph and self.model.graph_safe_portions and self.dtype == torch.bfloat16):
+            return 0
+        return portion_tokens_worth_a_graph(self.model.matrix_elements(), len(self.model.spec.order), 2,
+                                            int(self.config.hip_graph_portion_tokens))
+
     def _cache_bytes(self, tokens: int, specs) -> int:
         """Bytes the pages take when live requests may hold ``tokens`` tokens (windowed groups are bounded)."""
         el = torch.empty((), dtype=self.dtype).element_size()
@@ -188,6 +197,10 @@ class Engine:
         if self.config.hip_graph and self.model.graph_safe and self.dtype == torch.bfloat16:
             logits = int(self.config.hip_graph_max_bs) * self.vocab_size * 4
             reserve_graphs = int(self.config.hip_graph_cache_size) * logits + (256 << 20)
+            # captured steps with portions keep their activations in the graphs' shared pool: what the measured
+            # step took, in proportion to the tokens such a step may have
+            probed = max(1, min(self._chunk_cap(), self.max_positions))
+            reserve_graphs += peak * min(probed, self._graph_portion_tokens()) // probed
         budget = int(total * self.config.gpu_memory_utilization) - in_use - peak - reserve_state - reserve_library \
             - reserve_graphs
         self.memory_plan = dict(total=total, in_use=in_use, step_peak=peak, state=reserve_state,
@@ -395,6 +408,9 @@ class Engine:
             from ..ops import kernels as K
             self._validate_carried(entries, carried)
             K.carry_tokens(carried, view("carry_src"), view("carry_dst"), view("token_ids"))
+        max_pre = max([counts[i] for i in pre], default=0)
+        min_pre = min([starts[i] for i in pre], default=0)
+        level = bool(pre) and min_pre >= max_pre
         G = len(self.group_specs)
         bt = view("block_tables").view(G, n, stride) if G else None
         sl = view("slots").view(G, total) if G else None
@@ -407,20 +423,24 @@ class Engine:
                          max_q_len=max(counts), max_context_len=stride * self.page_size if fixed else max(ends),
                          page_size=self.page_size,
                          decode_seqs=view("decode_seqs")[:len(dec)], prefill_seqs=view("prefill_seqs")[:len(pre)],
-                         n_decode=len(dec), n_prefill=len(pre), max_prefill_q=max([counts[i] for i in pre], default=0),
-                         min_prefill_prefix=min([starts[i] for i in pre], default=0),
-                         # with fixed buffers the launch shapes must not follow the data: bound by what the tables can hold
-                         max_decode_context=(stride * self.page_size if fixed else max([ends[i] for i in dec], default=0)))
+                         n_decode=len(dec), n_prefill=len(pre), max_prefill_q=max_pre,
+                         # with fixed buffers the launch shapes must not follow the data.  The fewest tokens behind
+                         # a portion only says whether every portion has its own length behind it; the decode
+                         # kernels are bound by what the tables can hold, and without fixed buffers by the step's
+                         # longest sequence of either kind, which rounds to the same bound.
+                         min_prefill_prefix=((max_pre if level else 0) if fixed else min_pre),
+                         max_decode_context=(stride * self.page_size if fixed else (max(ends) if dec else 0)))
 
     def run(self, entries: Sequence[StepEntry], starts: Sequence[int],
             carried: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs a step whose pages are already reserved (the scheduler's path).
 
         A step of single tokens whose logits are all wanted is replayed from a
-        captured HIP graph when graphs are on; the logits tensor it returns is
-        then the graph's own and is overwritten by the next such step.
+        captured HIP graph when graphs are on, and so is a small step with
+        prompt portions whose shape has been met before; the logits tensor it
+        returns is then the graph's own and is overwritten by the next such step.
         """
-        if self._graphs is not None and self._graphs.eligible(entries):
+        if self._graphs is not None and self._graphs.eligible(entries, starts):
             return self._graphs.run(entries, starts, carried)
         batch = self.build_batch(entries, starts, carried=carried)
         return self.forward(batch, any(batch.fresh_host))

@@ -1,4 +1,4 @@
-"""Decode steps replayed from HIP graphs.
+"""Steps replayed from HIP graphs.
 
 A decode step of a 36-layer model is some four hundred small launches; issued
 one by one from the host they take several times longer than the kernels run.
@@ -25,6 +25,16 @@ Nothing inside a captured step may depend on the step's data through the
 host: launch shapes follow the batch size and the table width only (the
 decode attention kernel is launched for as many splits as the table could
 hold; workgroups beyond a sequence's length leave at once).
+
+Small steps that bring portions of prompts are bound by the host's launches
+as well (a 128-token prompt of a 28-layer model is some 280 launches of a few
+microseconds of device work each), so they are replayed too, where every part
+of the model allows it (``Part.GRAPH_SAFE_PORTIONS``): such a step's key is
+its portion lengths, its number of wanted rows, its table width and whether
+every portion has at least its own length of context behind it (which decides
+how the prefill attention cuts its work).  There are many such shapes and most
+come once, so a shape is captured when it is met a second time.  The reference
+captures decode steps only.
 """
 from __future__ import annotations
 
@@ -33,6 +43,27 @@ import dataclasses
 from typing import Sequence, Tuple
 
 import torch
+
+
+# What a step with portions is taken to cost, to tell where its capture pays: the host some ten launches a layer
+# at 8 us each; the device the weights streamed once at 4 TB/s or, beyond a few tokens, two operations per matrix
+# element and token at 0.4 PFLOP/s (what the library's products reach at some hundred rows).
+HOST_SECONDS_PER_LAYER = 10 * 8e-6
+STREAM_BYTES_PER_SECOND = 4e12
+PRODUCT_OPS_PER_SECOND = 0.4e15
+
+
+def portion_tokens_worth_a_graph(matrix_elements: int, layers: int, element_bytes: int, cap: int) -> int:
+    """Up to how many tokens a step with portions is replayed from a graph: as long as the host's launches are
+    estimated to take longer than the device's work, and never beyond ``cap``.  (Measured: a 28-layer model of
+    0.6 G elements takes 2.04 instead of 2.51 ms for a prompt of 128 tokens; a 36-layer model of 4 G elements is
+    bound by the device at 512 tokens, 7.3 ms either way, and gains nothing from the capture.)"""
+    if cap <= 0 or matrix_elements <= 0:
+        return max(cap, 0)
+    host = layers * HOST_SECONDS_PER_LAYER
+    if matrix_elements * element_bytes / STREAM_BYTES_PER_SECOND >= host:
+        return 0
+    return int(min(cap, host * PRODUCT_OPS_PER_SECOND / (2.0 * matrix_elements)))
 
 
 @dataclasses.dataclass
@@ -45,20 +76,50 @@ class _Captured:
 
 class DecodeGraphs:
 
-    def __init__(self, engine, max_batch: int, cache_size: int = 32):
+    SEEN_SHAPES = 512   # shapes of steps with portions remembered as met once
+
+    def __init__(self, engine, max_batch: int, cache_size: int = 32, portion_tokens: int = 0):
         self.engine = engine
         self.max_batch = int(max_batch)
         self.cache_size = max(1, int(cache_size))
-        self._graphs: "collections.OrderedDict[Tuple[int, int], _Captured]" = collections.OrderedDict()
+        self.portion_tokens = int(portion_tokens)
+        self._graphs: "collections.OrderedDict[tuple, _Captured]" = collections.OrderedDict()
+        self._seen: "collections.OrderedDict[tuple, None]" = collections.OrderedDict()
         self._pool = None
         self.replays = 0
         self.captures = 0
         self.evictions = 0
 
-    def eligible(self, entries: Sequence) -> bool:
+    def eligible(self, entries: Sequence, starts: Sequence[int] = ()) -> bool:
+        """Whether the step is to be replayed.  A step of single tokens is, from its first time; a step with
+        portions from the second time its shape is met (the first time only remembers the shape)."""
         if not 1 <= len(entries) <= self.max_batch:
             return False
-        return all(len(e.tokens) == 1 and len(e.want) == 1 and int(e.want[0]) == 0 for e in entries)
+        if all(len(e.tokens) == 1 and len(e.want) == 1 and int(e.want[0]) == 0 for e in entries):
+            return True
+        if self.portion_tokens <= 0 or sum(len(e.tokens) for e in entries) > self.portion_tokens:
+            return False
+        if any(len(e.want) > 1 for e in entries):
+            return False       # rows of logits beyond one a request: the graph's own output tensor would be large
+        key = self._key(entries, starts)
+        if key in self._graphs:
+            return True
+        if key in self._seen:
+            del self._seen[key]
+            return True
+        self._seen[key] = None
+        while len(self._seen) > self.SEEN_SHAPES:
+            self._seen.popitem(last=False)
+        return False
+
+    def _key(self, entries: Sequence, starts: Sequence[int]) -> tuple:
+        counts = tuple(len(e.tokens) for e in entries)
+        stride = self._stride_for([s + c for s, c in zip(starts, counts)])
+        if max(counts) == 1:
+            return (len(entries), stride)
+        portions = [i for i, c in enumerate(counts) if c > 1]
+        level = min(starts[i] for i in portions) >= max(counts)
+        return (counts, sum(len(e.want) for e in entries), level, stride)
 
     def owns(self, t: torch.Tensor) -> bool:
         return any(t is g.logits for g in self._graphs.values())
@@ -72,9 +133,8 @@ class DecodeGraphs:
 
     def run(self, entries: Sequence, starts: Sequence[int], carried=None) -> torch.Tensor:
         eng = self.engine
-        n = len(entries)
-        stride = self._stride_for([s + 1 for s in starts])
-        key = (n, stride)
+        key = self._key(entries, starts)
+        stride = key[-1]
         cap = self._graphs.get(key)
         if cap is None:
             while len(self._graphs) >= self.cache_size:
@@ -94,7 +154,8 @@ class DecodeGraphs:
     def _capture(self, entries: Sequence, starts: Sequence[int], stride: int, carried=None) -> _Captured:
         eng = self.engine
         n = len(entries)
-        size = eng.tables.step_layout(n, n, stride, n)["_total"][1]
+        size = eng.tables.step_layout(n, sum(len(e.tokens) for e in entries), stride,
+                                      sum(len(e.want) for e in entries))["_total"][1]
         buffer = torch.empty(size, dtype=torch.int32, device=eng.device)
         batch = eng.build_batch(entries, starts, stride=stride, device_buffer=buffer, carried=carried)
         # once outside a capture, on a side stream, so that whatever libraries set up lazily exists already;

@@ -106,6 +106,22 @@ class CausalLM:
         for p in self.shared.values():
             p.prepare(device)
 
+    def matrix_elements(self) -> int:
+        """Elements of the weight matrices a step multiplies with (the embedding table is only looked up in)."""
+        from ..parts.base import MATRIX
+        seen, total = set(), 0
+        for part, ps in self._parts:
+            if part is self.embedding:
+                continue
+            for local, req in part.tensors().items():
+                if req.kind == MATRIX and ps.weights[local] not in seen:
+                    seen.add(ps.weights[local])
+                    n = 1
+                    for d in req.shape:
+                        n *= int(d)
+                    total += n
+        return total
+
     # ---- what the cache manager must provide ------------------------------
     @property
     def needs_state(self) -> bool:
@@ -115,6 +131,12 @@ class CausalLM:
     def graph_safe(self) -> bool:
         """Whether a decode step may be captured once and replayed: no part says no."""
         return all(p.GRAPH_SAFE for p, _ in self._parts) and all(b.GRAPH_SAFE for b in self.blocks)
+
+    @property
+    def graph_safe_portions(self) -> bool:
+        """Whether a step that brings prompt portions may be captured and replayed too: every part says yes."""
+        return self.graph_safe and all(p.GRAPH_SAFE_PORTIONS for p, _ in self._parts) and \
+            all(b.GRAPH_SAFE_PORTIONS for b in self.blocks)
 
     @property
     def atomic_prefill(self) -> bool:

@@ -22,6 +22,8 @@ from .base import MATRIX, NORM, VECTOR, KVCacheSpec, Mixer, PartError, TensorReq
 
 @register_part("mixer", "gqa_attention")
 class GQAAttention(Mixer):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, norm_eps: float = 1e-6,
                  qk_norm: bool = True, bias: bool = False, window: int = 0, position: Optional[str] = None,
                  rotary_dim: Optional[int] = None, scale: Optional[float] = None):

@@ -73,6 +73,11 @@ class Part:
     # slots through the device array ``StepBatch.state_slots`` alone; the slots of starting requests are
     # cleared on the device before it runs.
     GRAPH_SAFE = True
+    # The same for steps that bring portions of prompts: True says that ``forward`` launches the same work for
+    # every step with the same portion lengths, numbers of wanted rows and table width, whatever the tokens, the
+    # positions the portions start at, the pages and the state slots are (these it reads on the device).  False
+    # by default: a part has to say so itself.
+    GRAPH_SAFE_PORTIONS = False
 
     def tensors(self) -> Dict[str, TensorReq]:
         """Local tensor name -> what is required of it."""

@@ -13,6 +13,8 @@ from .base import Block, register_part
 
 @register_part("block", "prenorm")
 class PreNormBlock(Block):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     SLOTS = {"input_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm", "ffn": "ffn"}
 
     def __init__(self, input_norm, mixer, post_mixer_norm, ffn):

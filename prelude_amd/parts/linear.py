@@ -14,6 +14,8 @@ from .base import MATRIX, Part, TensorReq, register_part
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight = None
@@ -30,6 +32,8 @@ class TokenEmbedding(Part):
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight = None

@@ -16,6 +16,8 @@ from .base import MATRIX, FeedForward, PartError, TensorReq, register_part
 
 @register_part("ffn", "gated_mlp")
 class GatedMLP(FeedForward):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
             raise PartError(f"gated_mlp: activation {activation!r} is not supported (silu)")

@@ -17,6 +17,8 @@ from .base import NORM, Norm, TensorReq, register_part
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     TAKES_SLICE_SUMS = True
 
     def __init__(self, size: int, eps: float):

@@ -16,6 +16,8 @@ from .base import PartError, PositionEncoding, register_part
 
 @register_part("position", "rope")
 class RotaryEmbedding(PositionEncoding):
+    GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
+
     def __init__(self, rotary_dim: int, max_positions: int, theta: float):
         if rotary_dim <= 0 or rotary_dim % 2:
             raise PartError(f"rope: rotary width {rotary_dim} must be positive and even")

@@ -96,3 +96,25 @@ def test_read_config_json(tmp_path):
         read_config_json(str(tmp_path))
     (tmp_path / "config.json").write_text(json.dumps(pm.tiny_config_a()))
     assert read_config_json(str(tmp_path))["hidden_size"] == 64
+
+
+def test_where_a_step_with_portions_is_worth_a_graph():
+    """Steps with prompt portions are replayed from graphs up to the number of tokens at which the device's work
+    is taken to reach the host's launches: some hundreds for a small model, about 140 for a 36-layer model of 4 G
+    matrix elements, none where streaming the weights alone takes longer than the launches; never beyond the
+    configured number, and the matrix elements are counted from the model's own tensors."""
+    from prelude_amd.engine.graph import portion_tokens_worth_a_graph as worth
+    assert 600 < worth(int(0.6e9), 28, 2, 1024) < 900
+    assert worth(int(0.6e9), 28, 2, 256) == 256
+    assert 100 < worth(int(4.0e9), 36, 2, 1024) < 200
+    assert worth(int(8.2e9), 36, 2, 1024) == 0
+    assert worth(int(0.6e9), 28, 2, 0) == 0
+    from prelude_amd.models.causal_lm import CausalLM
+    from prelude_amd.config import resolve_architecture
+    for cfg in (pm.tiny_config_a(), pm.tiny_config_b(), pm.tiny_config_c()):
+        arch = resolve_architecture(cfg)
+        model = CausalLM(arch.build_spec(arch.parse_config(cfg)))
+        shapes = pm.tensor_shapes(cfg)
+        want = sum(a * b for name, (a, *rest) in shapes.items() for b in rest
+                   if name != "model.embed_tokens.weight" or cfg["tie_word_embeddings"])
+        assert model.matrix_elements() == want and model.graph_safe_portions

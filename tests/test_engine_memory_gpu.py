@@ -24,8 +24,9 @@ def mid_config() -> dict:
 def test_pool_sized_from_a_measured_step(gpu):
     """``max_cache_tokens=None``: the pool is what the device has left after the weights, a measured step of
     ``max_num_batched_tokens`` tokens and the stated reserves.  Then the worst the engine is configured for is run
-    -- a portion of 8,192 tokens, decode steps of 64 requests captured at several table widths -- and the device
-    must still hold no more than the share it was given."""
+    -- a portion of 8,192 tokens, decode steps of 64 requests captured at several table widths, portions of 250
+    and 256 tokens captured when their shape comes a second time -- and the device must still hold no more than
+    the share it was given."""
     from prelude_amd.config import EngineConfig
     from prelude_amd.engine import Engine, StepEntry
     torch.cuda.empty_cache()
@@ -36,7 +37,11 @@ def test_pool_sized_from_a_measured_step(gpu):
     eng = Engine.from_config(mid_config(), cfg, seed=1)
     plan = eng.memory_plan
     assert plan["step_peak"] > 512 * 151936 * 4          # the probe saw the logits of its wanted rows
-    assert plan["graphs"] == 4 * 64 * 151936 * 4 + (256 << 20)
+    # a logits tensor per kept graph, the decode steps' activations, and a share of the measured step for the
+    # captured steps with portions: this model's are worth a graph up to some 380 of the step's 8,192 tokens
+    worth = eng._graphs.portion_tokens
+    assert 256 <= worth < 512
+    assert plan["graphs"] == 4 * 64 * 151936 * 4 + (256 << 20) + plan["step_peak"] * worth // 8192
     assert plan["cache"] > 0 and eng.cache_tokens >= 16 * 16
     per_token = 2 * 2 * 2 * 64 * 2
     assert abs(eng.cache_tokens * per_token - plan["cache"]) <= 32 * per_token      # the budget is what was allocated
@@ -47,14 +52,18 @@ def test_pool_sized_from_a_measured_step(gpu):
     eng.release(0)
     # 64 decoding requests, captured at three table widths (contexts under 1,024, 2,048 and 3,072 tokens)
     for r in range(64):
-        eng.step([StepEntry(100 + r, rng.integers(0, v, 1000).tolist(), [])])
+        for _ in range(4):
+            eng.step([StepEntry(100 + r, rng.integers(0, v, 250).tolist(), [])])
     for width in range(3):
         for _ in range(2):
             eng.step([StepEntry(100 + r, [int(rng.integers(0, v))], [0]) for r in range(64)])
         if width < 2:
             for r in range(64):
-                eng.step([StepEntry(100 + r, rng.integers(0, v, 1024).tolist(), [])])
-    assert eng._graphs.captures == 3
+                for _ in range(4):
+                    eng.step([StepEntry(100 + r, rng.integers(0, v, 256).tolist(), [])])
+    # three shapes of decode steps and four of portions (250 tokens from the start; 250 behind as many or more; 256
+    # behind 1,001 and behind 2,026, with wider tables), four kept at a time
+    assert eng._graphs.captures == 7 and eng._graphs.evictions == 3
     torch.cuda.synchronize()
     free, _ = torch.cuda.mem_get_info(gpu)
     assert total - free <= share * total, f"{(total - free) >> 20} MB in use, the share was {int(share * total) >> 20} MB"

@@ -323,6 +323,57 @@ def test_graph_replays_equal_eager_steps_where_the_grid_sets_the_wavefronts(gpu)
         assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
 
 
+def test_graph_replays_of_steps_with_portions_equal_eager_steps(gpu):
+    """Small steps that bring prompt portions are captured when their shape (portion lengths, wanted rows, table
+    width, whether every portion has its own length behind it) comes a second time, and replayed from then on: whole
+    prompts of one length, portions without wanted rows, portions behind a long context, and steps of portions
+    beside single tokens, with other requests, other pages and other positions at every replay.  Every step gives
+    the eager step's logits bit for bit."""
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    folder, cfg, _ = model_folder("b")
+    rng = np.random.default_rng(12)
+    seqs = [rng.integers(0, cfg["vocab_size"], size=200).tolist() for _ in range(8)]
+
+    def play(hip_graph, portion_tokens=1024):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=8 * 208,
+                                                         hip_graph=hip_graph, hip_graph_portion_tokens=portion_tokens))
+        outs, at = [], [0] * 8
+
+        def feed(parts):
+            entries = []
+            for r, n, wanted in parts:
+                entries.append(StepEntry(r, seqs[r][at[r]:at[r] + n], [n - 1] if wanted else []))
+                at[r] += n
+            outs.append(eng.step(entries).cpu())
+        for r in range(4):
+            feed([(r, 40, True)])                    # a prompt of 40 tokens: met, then captured and replayed
+        for r in range(4):
+            feed([(r, 30, False)])                   # a portion behind 40 tokens, nothing wanted
+        for r in range(4):
+            feed([(r, 24, True)])                    # a portion with more than its own length behind it
+        for r in range(4, 7):
+            feed([(0, 1, True), (r, 33, True), (1, 1, True)])     # a prompt between two decoding requests
+        for r in range(4):
+            feed([(r, 40, True)])                    # 40 tokens again, behind 94 or 95: a shape of its own
+        feed([(7, 37, True)])                        # a shape that comes once
+        for _ in range(3):
+            feed([(r, 1, True) for r in range(8)])   # decode steps: captured at once, as ever
+        return eng, outs
+
+    eager_eng, eager = play(False)
+    graph_eng, graphed = play(True)
+    off_eng, off = play(True, portion_tokens=0)
+    # shapes: (40,) from the start; (30,) behind 40; (24,) behind 70; (1, 33, 1); (40,) behind 94; the decode step
+    # a shape of portions runs eagerly the first time and from its graph after that
+    assert graph_eng._graphs.captures == 6 and graph_eng._graphs.replays == 3 + 3 + 3 + 2 + 3 + 3
+    assert off_eng._graphs.captures == 1 and off_eng._graphs.replays == 3
+    for i, (a, b, c) in enumerate(zip(eager, graphed, off)):
+        assert a.shape == b.shape and torch.equal(a, b), f"step {i}: the replay differs from the eager step"
+        assert torch.equal(a, c)
+    assert graph_eng.tables.audit() == ""
+
+
 def test_graph_replays_with_library_products_equal_eager_steps(gpu):
     """A decode step of more than 48 requests multiplies through the library product, also inside a captured
     graph (with its workspace): every replay, with eager steps of other shapes between them, gives the eager
