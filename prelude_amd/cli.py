@@ -43,6 +43,8 @@ def build_parser() -> argparse.ArgumentParser:
     g = ap.add_mutually_exclusive_group()
     g.add_argument("--cuda-graph", "--hip-graph", dest="hip_graph", action="store_true", default=True)
     g.add_argument("--no-cuda-graph", "--no-hip-graph", dest="hip_graph", action="store_false")
+    ap.add_argument("--hip-graph-portion-tokens", type=int, default=1024,
+                    help="small steps with prompt portions are replayed from graphs up to this many tokens (0: never)")
     ap.add_argument("--no-weight-tiles", dest="weight_tiles", action="store_false", default=True,
                     help="keep no second, tiled copy of the weights for decode steps (saves their memory)")
     ap.add_argument("--no-overlap-steps", dest="overlap_steps", action="store_false", default=True,
@@ -87,7 +89,8 @@ def main(argv=None) -> int:
                        max_running_requests=args.max_running_requests, max_total_tokens=args.max_total_tokens,
                        decode_reservation_cap=args.decode_reservation_cap,
                        decode_priority_max_remaining_tokens=args.decode_priority_max_remaining_tokens,
-                       hip_graph=args.hip_graph, overlap_steps=args.overlap_steps, weight_tiles=args.weight_tiles)
+                       hip_graph=args.hip_graph, hip_graph_portion_tokens=args.hip_graph_portion_tokens,
+                       overlap_steps=args.overlap_steps, weight_tiles=args.weight_tiles)
     if args.random_weights:
         cfg_path = os.path.join(model, "config.json") if os.path.isdir(model) else model
         with open(cfg_path, "r", encoding="utf-8") as f:
