@@ -27,7 +27,6 @@
 namespace pa {
 
 constexpr int kMidMaxM = 128;
-constexpr int kMidMaxWaves = 8;
 
 struct MidFrag {
   bf16x8 lo, hi;
