@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import dataclasses
 import re
-from typing import Any, Callable, Dict, List, Mapping, Optional, Sequence
+from typing import Any, Callable, List, Mapping, Optional, Sequence
 
 
 class UnknownArchitecture(ValueError):

@@ -12,13 +12,12 @@ always returns one row per request.
 from __future__ import annotations
 
 import dataclasses
-import os
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
 
-from ..cache.manager import (CacheError, OutOfPages, PageTables, allocate_storage, bytes_per_token, pages_per_group,
+from ..cache.manager import (CacheError, PageTables, allocate_storage, bytes_per_token, pages_per_group,
                              plan_groups, state_bytes_per_slot)
 from ..config.engine_config import EngineConfig
 from ..config.model_config import read_config_json

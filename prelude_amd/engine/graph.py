@@ -40,7 +40,7 @@ from __future__ import annotations
 
 import collections
 import dataclasses
-from typing import Sequence, Tuple
+from typing import Sequence
 
 import torch
 

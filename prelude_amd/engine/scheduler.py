@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import dataclasses
-from typing import List, Tuple
+from typing import List
 
 import numpy as np
 

@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..parts import Block, KVCacheSpec, Part, StateSpec, TensorReq, build_part
+from ..parts import Block, Part, StateSpec, TensorReq, build_part
 from ..parts.base import PartError, _REGISTRY
 from .spec import ModelSpec, PartSpec
 

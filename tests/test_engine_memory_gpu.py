@@ -1,12 +1,9 @@
 """How the engine sizes what it allocates: the page pools from a measured step, a pool of its own size per cache
 group, a bounded cache of captured decode steps."""
-import json
-
 import numpy as np
 import pytest
 import torch
 
-import plain_model as pm
 from helpers import check, model_folder, reference_logits
 
 pytestmark = pytest.mark.gpu

@@ -4,9 +4,6 @@ framework's files.  The toy model also names a layer twice in its run order and 
 It is no model of anyone's: a decaying sum as mixer, beside the framework's attention in the other layer.
 """
 import dataclasses
-import os
-
-import numpy as np
 import pytest
 import torch
 
