@@ -261,8 +261,10 @@ SKINNY_MAX_ROWS = 16   # above this the library product is faster (the kernel it
 # which the streaming kernel measured faster -- [6144, 2560] and [2560, 4096] to 48 rows (11 against 19 us at 32),
 # [6144, 4096] to 32 rows (15 against 19 us); weights beyond that go to the library, as do rows of 8192 columns or
 # more -- unless they are very long: [5120, 25600] takes the library 143 to 155 us at 24 to 64 rows, the streaming
-# kernel 67 to 118
-TILED_LIMITS = ((48, 1 << 24), (32, 1 << 25))
+# kernel 67 to 118.  Inside a captured step, where no launch waits for the host, the library's floor is 11 us and
+# the order is the same: [4096, 1024] takes the streaming kernel 4.6 to 8.0 us at 17 to 64 rows, [6144, 2560] 11.6
+# to 14.4 at 17 to 48 rows against 12.5 to 15.5
+TILED_LIMITS = ((64, 1 << 23), (48, 1 << 24), (32, 1 << 25))
 TILED_LONG_ROWS = 16384
 
 
@@ -380,6 +382,11 @@ MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns,
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
 MID_SLICED_LONG_K = 8192
+# A reader that wants a tensor gets the slices too, added by a kernel of their own, where the pair is still ahead of
+# the library: large weights ([10240, 5120] inside a captured step: 24.2 to 26.9 us at 24 to 64 rows against 28.4 to
+# 32.4, 33.7 and 38.6 at 96 and 128 rows against 36.1 and 40.4; [6144, 4096] and [6144, 2560] are within a
+# microsecond either way and stay with the library)
+MID_SUMMED_MIN_ELEMENTS = 40 << 20
 MID_PRODUCTS = True    # ``set_mid_products``: off sends these products where they went without this kernel (measurements)
 
 
@@ -478,6 +485,11 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
             return gemm_mid(x, tiles, bias, slices=s)
     if m <= SKINNY_MAX_ROWS and k % 8 == 0:
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
+    if (MID_PRODUCTS and tiles is not None and bias is None and k % 8 == 0 and n % 4 == 0 and m <= GEMM_MID_MAX_ROWS
+            and out_dtype in (None, torch.bfloat16) and n * k >= MID_SUMMED_MIN_ELEMENTS and k < TILED_LONG_ROWS):
+        s = gemm_mid_slices(n, k)
+        if s >= MID_MIN_SLICES:
+            return gemm_mid(x, tiles, slices=s).materialize()
     if MID_PRODUCTS and tiles is not None and k % 8 == 0 and m <= GEMM_MID_MAX_ROWS:
         if n >= MID_WIDE_ROWS and m <= (MID_WIDE_MAX_M if k <= MID_WIDE_SHORT_K else MID_WIDE_MAX_M // 2):
             return gemm_mid(x, tiles, bias, out_dtype)

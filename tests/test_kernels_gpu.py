@@ -239,6 +239,18 @@ def test_gemm_mid_refuses_and_is_dispatched(gpu):
     close(K().as_tensor(got), x.double().cpu() @ w.double().cpu().T, torch.bfloat16)
     assert isinstance(K().linear(x[:8].contiguous(), lw, slices_ok=True), torch.Tensor)      # few rows: the streaming kernel
     assert isinstance(K().linear(x.float(), w.float(), slices_ok=True), torch.Tensor)      # 32-bit: the plain product
+    # a large weight whose reader wants a tensor: the slices and a kernel that adds them, the same bits as asked for
+    # directly; a small weight stays with the streaming kernel up to 64 rows
+    wl = (torch.randn(10240, 5120, generator=torch.Generator().manual_seed(8)) * 0.03).to(torch.bfloat16).to(gpu)
+    ll = K().LinearWeight(wl, K().pack_tiles(wl))
+    xl = rnd(56, 5120, dtype=torch.bfloat16, seed=9).to(gpu)
+    got = K().linear(xl, ll)
+    assert torch.equal(got, K().gemm_mid(xl, ll.tiles, slices=K().gemm_mid_slices(10240, 5120)).materialize())
+    close(got, xl.double().cpu() @ wl.double().cpu().T, torch.bfloat16)
+    ws = rnd(4096, 1024, dtype=torch.bfloat16, seed=10, scale=0.05).to(gpu)
+    ls = K().LinearWeight(ws, K().pack_tiles(ws))
+    xs = rnd(64, 1024, dtype=torch.bfloat16, seed=11).to(gpu)
+    assert torch.equal(K().linear(xs, ls), K().gemm_skinny(xs, ls.tiles))
     # the gated product beyond 16 rows: activation in this kernel's epilogue (the same bits as asked for directly)
     wg = rnd(1216, 520, dtype=torch.bfloat16, seed=5, scale=0.05).to(gpu)
     lg = K().LinearWeight(wg, K().pack_tiles(wg))
