@@ -440,7 +440,9 @@ class Engine:
         returns is then the graph's own and is overwritten by the next such step.
         """
         if self._graphs is not None and self._graphs.eligible(entries, starts):
-            return self._graphs.run(entries, starts, carried)
+            logits = self._graphs.run(entries, starts, carried)
+            if logits is not None:
+                return logits
         batch = self.build_batch(entries, starts, carried=carried)
         return self.forward(batch, any(batch.fresh_host))
 

@@ -66,6 +66,10 @@ def portion_tokens_worth_a_graph(matrix_elements: int, layers: int, element_byte
     return int(min(cap, host * PRODUCT_OPS_PER_SECOND / (2.0 * matrix_elements)))
 
 
+class NotCaptured(RuntimeError):
+    """A step ran in its warm-up but its capture as a graph failed."""
+
+
 @dataclasses.dataclass
 class _Captured:
     graph: torch.cuda.CUDAGraph
@@ -85,6 +89,7 @@ class DecodeGraphs:
         self.portion_tokens = int(portion_tokens)
         self._graphs: "collections.OrderedDict[tuple, _Captured]" = collections.OrderedDict()
         self._seen: "collections.OrderedDict[tuple, None]" = collections.OrderedDict()
+        self._refused: "collections.OrderedDict[tuple, None]" = collections.OrderedDict()   # shapes whose capture failed
         self._pool = None
         self.replays = 0
         self.captures = 0
@@ -104,6 +109,8 @@ class DecodeGraphs:
         key = self._key(entries, starts)
         if key in self._graphs:
             return True
+        if key in self._refused:
+            return False
         if key in self._seen:
             del self._seen[key]
             return True
@@ -131,7 +138,10 @@ class DecodeGraphs:
         page = self.engine.page_size
         return K.decode_context_bound(max(ends), page) // page
 
-    def run(self, entries: Sequence, starts: Sequence[int], carried=None) -> torch.Tensor:
+    def run(self, entries: Sequence, starts: Sequence[int], carried=None):
+        """The step's logits from its graph, captured first if need be.  None if the step has portions and its
+        capture failed (no memory for its activations, say): the caller then runs it directly, as it will every
+        later step of that shape.  A step of single tokens has no such way out: its failure is the caller's."""
         eng = self.engine
         key = self._key(entries, starts)
         stride = key[-1]
@@ -142,7 +152,15 @@ class DecodeGraphs:
                 torch.cuda.synchronize(eng.device)
                 self._graphs.popitem(last=False)
                 self.evictions += 1
-            cap = self._capture(entries, starts, stride, carried)
+            try:
+                cap = self._capture(entries, starts, stride, carried)
+            except NotCaptured:
+                if max(len(e.tokens) for e in entries) == 1:
+                    raise
+                self._refused[key] = None
+                while len(self._refused) > self.SEEN_SHAPES:
+                    self._refused.popitem(last=False)
+                return None
             self._graphs[key] = cap
         else:
             self._graphs.move_to_end(key)
@@ -165,16 +183,23 @@ class DecodeGraphs:
         saved = [c.snapshot(batch.state_slots) for c in stateful]
         side = torch.cuda.Stream(device=eng.device)
         side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            eng.forward(batch)
-        torch.cuda.current_stream().wait_stream(side)
-        for c, rows in zip(stateful, saved):
-            c.restore(batch.state_slots, rows)
+        try:
+            with torch.cuda.stream(side):
+                eng.forward(batch)
+        finally:
+            torch.cuda.current_stream().wait_stream(side)
+            for c, rows in zip(stateful, saved):
+                c.restore(batch.state_slots, rows)
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        if self._pool is None:
-            self._pool = torch.cuda.graph_pool_handle()
-        with torch.cuda.graph(graph, pool=self._pool):
-            logits = eng.forward(batch)
+        # The warm-up ran the same launches, so what fails from here on is the capture itself (its pool's memory, an
+        # operation that cannot be recorded): the step can still run directly.
+        try:
+            graph = torch.cuda.CUDAGraph()
+            if self._pool is None:
+                self._pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._pool):
+                logits = eng.forward(batch)
+        except Exception as e:
+            raise NotCaptured(f"a step of {[len(e_.tokens) for e_ in entries]} tokens could not be captured: {e}") from e
         self.captures += 1
         return _Captured(graph, buffer, logits, stride)

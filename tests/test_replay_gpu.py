@@ -374,6 +374,51 @@ def test_graph_replays_of_steps_with_portions_equal_eager_steps(gpu):
     assert graph_eng.tables.audit() == ""
 
 
+def test_a_step_with_portions_whose_capture_fails_runs_directly(gpu, monkeypatch):
+    """The capture of a step with portions is an extra: if it fails (here: made to), the step runs directly and
+    gives the direct run's logits, its shape is not tried again, and decode steps are captured as ever."""
+    import contextlib
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    from prelude_amd.engine import graph as graph_module
+    folder, cfg, _ = model_folder("b")
+    rng = np.random.default_rng(14)
+    seqs = [rng.integers(0, cfg["vocab_size"], size=60).tolist() for _ in range(4)]
+
+    def play(hip_graph, break_portions):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=512,
+                                                         hip_graph=hip_graph))
+        if break_portions:
+            real = torch.cuda.graph
+
+            @contextlib.contextmanager
+            def refusing(graph, pool=None):
+                if eng._graphs.captures >= 0 and refusing.portions:
+                    raise torch.cuda.OutOfMemoryError("no memory for this capture (made up by the test)")
+                with real(graph, pool=pool):
+                    yield
+            refusing.portions = True
+            monkeypatch.setattr(graph_module.torch.cuda, "graph", refusing)
+        outs = []
+        for r in range(4):
+            outs.append(eng.step([StepEntry(r, seqs[r][:40], [39])]).cpu())     # the same shape four times
+        if break_portions:
+            refusing.portions = False
+        for k in range(3):
+            outs.append(eng.step([StepEntry(r, [seqs[r][40 + k]], [0]) for r in range(4)]).cpu())
+        if break_portions:
+            monkeypatch.undo()
+        return eng, outs
+
+    eager_eng, eager = play(False, False)
+    graph_eng, graphed = play(True, True)
+    assert graph_eng._graphs.captures == 1 and graph_eng._graphs.replays == 3       # the decode step only
+    assert len(graph_eng._graphs._refused) == 1
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.equal(a, b), f"step {i}"
+    assert graph_eng.tables.audit() == ""
+
+
 def test_graph_replays_with_library_products_equal_eager_steps(gpu):
     """A decode step of more than 48 requests multiplies through the library product, also inside a captured
     graph (with its workspace): every replay, with eager steps of other shapes between them, gives the eager
