@@ -100,7 +100,7 @@ class DecodeGraphs:
         portions from the second time its shape is met (the first time only remembers the shape)."""
         if not 1 <= len(entries) <= self.max_batch:
             return False
-        if all(len(e.tokens) == 1 and len(e.want) == 1 and int(e.want[0]) == 0 for e in entries):
+        if self._single_tokens(entries):
             return True
         if self.portion_tokens <= 0 or sum(len(e.tokens) for e in entries) > self.portion_tokens:
             return False
@@ -119,13 +119,18 @@ class DecodeGraphs:
             self._seen.popitem(last=False)
         return False
 
+    @staticmethod
+    def _single_tokens(entries: Sequence) -> bool:
+        return all(len(e.tokens) == 1 and len(e.want) == 1 and int(e.want[0]) == 0 for e in entries)
+
     def _key(self, entries: Sequence, starts: Sequence[int]) -> tuple:
         counts = tuple(len(e.tokens) for e in entries)
         stride = self._stride_for([s + c for s, c in zip(starts, counts)])
-        if max(counts) == 1:
+        if self._single_tokens(entries):
             return (len(entries), stride)
+        # any other step (portions, or single tokens some of which want no logits): its own kind of key
         portions = [i for i, c in enumerate(counts) if c > 1]
-        level = min(starts[i] for i in portions) >= max(counts)
+        level = bool(portions) and min(starts[i] for i in portions) >= max(counts)
         return (counts, sum(len(e.want) for e in entries), level, stride)
 
     def owns(self, t: torch.Tensor) -> bool:
@@ -155,7 +160,7 @@ class DecodeGraphs:
             try:
                 cap = self._capture(entries, starts, stride, carried)
             except NotCaptured:
-                if max(len(e.tokens) for e in entries) == 1:
+                if self._single_tokens(entries):
                     raise
                 self._refused[key] = None
                 while len(self._refused) > self.SEEN_SHAPES:

@@ -357,6 +357,8 @@ def test_graph_replays_of_steps_with_portions_equal_eager_steps(gpu):
         for r in range(4):
             feed([(r, 40, True)])                    # 40 tokens again, behind 94 or 95: a shape of its own
         feed([(7, 37, True)])                        # a shape that comes once
+        for _ in range(2):                           # single tokens, one of which wants no logits: no decode step's
+            feed([(0, 1, True), (1, 1, False), (2, 1, True)])   # graph fits that; met, then captured as a shape of its own
         for _ in range(3):
             feed([(r, 1, True) for r in range(8)])   # decode steps: captured at once, as ever
         return eng, outs
@@ -364,9 +366,10 @@ def test_graph_replays_of_steps_with_portions_equal_eager_steps(gpu):
     eager_eng, eager = play(False)
     graph_eng, graphed = play(True)
     off_eng, off = play(True, portion_tokens=0)
-    # shapes: (40,) from the start; (30,) behind 40; (24,) behind 70; (1, 33, 1); (40,) behind 94; the decode step
+    # shapes: (40,) from the start; (30,) behind 40; (24,) behind 70; (1, 33, 1); (40,) behind 94; (1, 1, 1) with two
+    # rows wanted; the decode step
     # a shape of portions runs eagerly the first time and from its graph after that
-    assert graph_eng._graphs.captures == 6 and graph_eng._graphs.replays == 3 + 3 + 3 + 2 + 3 + 3
+    assert graph_eng._graphs.captures == 7 and graph_eng._graphs.replays == 3 + 3 + 3 + 2 + 3 + 1 + 3
     assert off_eng._graphs.captures == 1 and off_eng._graphs.replays == 3
     for i, (a, b, c) in enumerate(zip(eager, graphed, off)):
         assert a.shape == b.shape and torch.equal(a, b), f"step {i}: the replay differs from the eager step"
