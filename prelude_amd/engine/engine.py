@@ -410,6 +410,7 @@ class Engine:
         max_pre = max([counts[i] for i in pre], default=0)
         min_pre = min([starts[i] for i in pre], default=0)
         level = bool(pre) and min_pre >= max_pre
+        replayable = bool(dec) and self._graphs is not None and total <= self._graphs.portion_tokens
         G = len(self.group_specs)
         bt = view("block_tables").view(G, n, stride) if G else None
         sl = view("slots").view(G, total) if G else None
@@ -425,10 +426,13 @@ class Engine:
                          n_decode=len(dec), n_prefill=len(pre), max_prefill_q=max_pre,
                          # with fixed buffers the launch shapes must not follow the data.  The fewest tokens behind
                          # a portion only says whether every portion has its own length behind it; the decode
-                         # kernels are bound by what the tables can hold, and without fixed buffers by the step's
-                         # longest sequence of either kind, which rounds to the same bound.
+                         # kernels are bound by what the tables can hold.  A step small enough to be replayed one
+                         # day is bound the same way when it runs directly (by its longest sequence of either
+                         # kind, which rounds to the table's width), so that both give the same bits; a larger
+                         # step by its decoding sequences alone, which keeps its workspace small.
                          min_prefill_prefix=((max_pre if level else 0) if fixed else min_pre),
-                         max_decode_context=(stride * self.page_size if fixed else (max(ends) if dec else 0)))
+                         max_decode_context=(stride * self.page_size if fixed else
+                                             (max(ends) if replayable else max([ends[i] for i in dec], default=0))))
 
     def run(self, entries: Sequence[StepEntry], starts: Sequence[int],
             carried: Optional[torch.Tensor] = None) -> torch.Tensor:
