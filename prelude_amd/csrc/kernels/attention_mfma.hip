@@ -1057,9 +1057,11 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // and need no pairing, which doubles the workgroups there are to hand out
   const bool level = min_prefix >= max_q_len;
   const bool wide_ok = can_stage && group % (gt_best * 2) == 0;   // eight wavefronts: two groups of gt_best heads
-  if (wide_ok && workgroups(paired, gt_best, 2) >= enough) {
+  if (wide_ok && workgroups(paired, gt_best, 2) >= enough && tiles > 8) {
     // the most work per staged key that still gives every compute unit a workgroup (measured at head_dim 128,
-    // 32 heads over 8: 4,096 tokens 171 against 186 us, 8,192 tokens 624 against 648)
+    // 32 heads over 8: 4,096 tokens 171 against 186 us, 8,192 tokens 624 against 648); not for many short prompts,
+    // whose workgroups are over after a few blocks (16 prompts of 512 tokens: 66 against 70 us with four
+    // wavefronts a workgroup, 32 of 256: 51 against 60)
     hw = 2;
   } else if (level && workgroups(0, gt_best, wide_ok ? 2 : 1) >= enough) {
     paired = 0;   // 2,048 tokens behind 6,144: 297 against 342 us
