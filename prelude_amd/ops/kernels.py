@@ -373,12 +373,14 @@ GEMM_MID_MAX_ROWS = 128
 # 128 rows).  Cut into slices, for a reader that adds them, wherever the weight's shape gives two slices or more:
 # [2560, 4096] at 64 rows 9.2 against the library's 14.7 us, [2560, 9728] 14.4 against 28, [4096, 12288] 28 against
 # 37, [5120, 25600] 50 against 155 (and 73 against 179 at 128 rows).  Uncut for very wide weights with 32-bit output
-# (the head: at 64 rows and 2,560 columns 196 us where the library takes 176 and a conversion pass of 20; with longer
-# rows the library is ahead from 48 rows on).  The gated product with its activation in the epilogue: see
+# (the head; figures at MID_WIDE_MAX_M).  The gated product with its activation in the epilogue: see
 # ``linear_silu_mul``.
 MID_MIN_SLICES = 2
 MID_WIDE_ROWS = 65536
-MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns, half of it beyond
+MID_WIDE_MAX_M = 128           # ... for rows of up to MID_WIDE_SHORT_K columns, half of it beyond (inside a captured
+#                                step the head takes it 214 against the library's 230 us at 96 rows and 236 against
+#                                249 at 128 for 2,560 columns, 290 against 315 and 331 against 339 for 4,096, and
+#                                290 against 311 at 48 rows and 308 against 330 at 64 for 5,120)
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
 MID_SLICED_LONG_K = 8192
