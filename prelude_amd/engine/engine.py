@@ -92,8 +92,8 @@ class Engine:
         self._set_cache(pages, state_slots)
         # decode steps as HIP graphs, in the serving type, for models none of whose parts says it cannot be replayed
         if config.hip_graph and model.graph_safe and self.dtype == torch.bfloat16:
-            from .graph import DecodeGraphs
-            self._graphs = DecodeGraphs(self, config.hip_graph_max_bs, config.hip_graph_cache_size,
+            from .graph import StepGraphs
+            self._graphs = StepGraphs(self, config.hip_graph_max_bs, config.hip_graph_cache_size,
                                         self._graph_portion_tokens())
 
     def _chunk_cap(self) -> int:

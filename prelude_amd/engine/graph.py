@@ -78,7 +78,7 @@ class _Captured:
     stride: int
 
 
-class DecodeGraphs:
+class StepGraphs:
 
     SEEN_SHAPES = 512   # shapes of steps with portions remembered as met once
 
