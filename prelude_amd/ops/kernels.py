@@ -384,6 +384,7 @@ MID_WIDE_MAX_M = 128           # ... for rows of up to MID_WIDE_SHORT_K columns,
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
 MID_SLICED_LONG_K = 8192
+MID_SLICED_SHORT_ROWS = 24     # ... and up to here small weights with shorter rows stay with the streaming kernel
 # A reader that wants a tensor gets the slices too, added by a kernel of their own, where the pair is still ahead of
 # the library: large weights ([10240, 5120] inside a captured step: 24.2 to 26.9 us at 24 to 64 rows against 28.4 to
 # 32.4, 33.7 and 38.6 at 96 and 128 rows against 36.1 and 40.4; [6144, 4096] and [6144, 2560] are within a
@@ -480,7 +481,11 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     # the other way round), from 17 rows on everywhere
     sliced = (MID_PRODUCTS and slices_ok and tiles is not None and k % 8 == 0 and n % 4 == 0 and m <= GEMM_MID_MAX_ROWS
               and out_dtype in (None, torch.bfloat16)
-              and (m > SKINNY_MAX_ROWS or (m >= MID_SLICED_MIN_ROWS and k >= MID_SLICED_LONG_K)))
+              and (m > SKINNY_MAX_ROWS or (m >= MID_SLICED_MIN_ROWS and k >= MID_SLICED_LONG_K))
+              # just beyond 16 rows a small weight with short rows is still the streaming kernel's (inside a captured
+              # step, with the norm that reads it: [4096, 4096] 13.3 and 14.4 us at 17 and 24 rows against 16.8 in
+              # slices, [2560, 4096] 12.5 and 13.7 against 13.3 and 13.9; from 32 rows on the slices are ahead)
+              and not (m <= MID_SLICED_SHORT_ROWS and k < MID_SLICED_LONG_K and _tiled_beyond_16(m, n, k)))
     if sliced:
         s = gemm_mid_slices(n, k)
         if s >= MID_MIN_SLICES:
