@@ -377,10 +377,10 @@ GEMM_MID_MAX_ROWS = 128
 # ``linear_silu_mul``.
 MID_MIN_SLICES = 2
 MID_WIDE_ROWS = 65536
-MID_WIDE_MAX_M = 128           # ... for rows of up to MID_WIDE_SHORT_K columns, half of it beyond (inside a captured
-#                                step the head takes it 214 against the library's 230 us at 96 rows and 236 against
-#                                249 at 128 for 2,560 columns, 290 against 315 and 331 against 339 for 4,096, and
-#                                290 against 311 at 48 rows and 308 against 330 at 64 for 5,120)
+MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns, half of it beyond.  (Alone inside a
+#                                captured graph the head is ahead of the library up to 128 rows, 214 against 230 us at
+#                                96 rows of 2,560 columns; in the decode step of 112 requests it is not: 7,380 against
+#                                7,640 tok/s.  The step decides.)
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
 MID_SLICED_LONG_K = 8192
