@@ -233,6 +233,45 @@ def test_drawn_workloads_change_no_token(gpu, seed):
     assert tight.engine.tables.audit() == "" and tight.engine.tables.num_requests() == 0
 
 
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_WORKLOADS", "6")))))   # widen for a hunt
+def test_drawn_workloads_replayed_from_graphs_change_no_token(gpu, seed):
+    """The same in bfloat16 with steps replayed from graphs (decode steps, and small steps with prompt portions once
+    their shape has come twice) against the same engine with every step run directly: a replay gives the direct
+    run's bits, so every request gets the same tokens, greedy or drawn, with overlapped steps and tokens carried
+    on the device, few pages and evictions."""
+    import numpy as np
+    from prelude_amd import LLM
+    from prelude_amd.sampling.sampler import SamplingParams
+    rng = np.random.default_rng(5000 + seed)
+    name = ["a", "b", "c"][seed % 3]
+    folder, cfg, _ = model_folder(name)
+    page = int(rng.choice([8, 16]))
+    n = int(rng.integers(4, 13))
+    room = cfg["max_position_embeddings"]
+    # few different lengths, so that shapes of steps come back
+    pool = [int(rng.integers(1, min(100, room - 45))) for _ in range(3)]
+    lengths = [int(rng.choice(pool)) for _ in range(n)]
+    prompts = prompts_for(cfg, lengths, 70 + seed)
+    max_new = int(rng.integers(2, 30))
+    params = [SamplingParams(temperature=0.0) if rng.random() < 0.5 else
+              SamplingParams(temperature=float(rng.choice([0.6, 1.0])), top_k=int(rng.choice([0, 5])) or None,
+                             top_p=float(rng.choice([1.0, 0.9])), seed=int(rng.integers(0, 1000))) for _ in range(n)]
+    total = sum(-(-(m + max_new) // page) * page for m in lengths)
+    longest = -(-(max(lengths) + max_new) // page) * page
+    common = dict(dtype="bfloat16", page_size=page, max_cache_tokens=int(rng.integers(longest + page, max(longest + 2 * page, total))),
+                  max_num_batched_tokens=int(rng.choice([48, 128, 512])), max_running_requests=int(rng.integers(2, 9)),
+                  overlap_steps=bool(rng.integers(0, 2)))
+    direct = LLM(folder, hip_graph=False, **common)
+    want = direct.generate(prompts, max_tokens=max_new, sampling_params=params)
+    replayed = LLM(folder, hip_graph=True, **common)
+    got = replayed.generate(prompts, max_tokens=max_new, sampling_params=params)
+    for i, (g, w_) in enumerate(zip(got, want)):
+        assert g.token_ids == w_.token_ids and g.finish_reason == w_.finish_reason, \
+            f"seed {seed}, request {i} of {n}: {g.token_ids} ({g.finish_reason}) against {w_.token_ids} ({w_.finish_reason})"
+    assert replayed.engine._graphs.replays > 0
+    assert replayed.engine.tables.audit() == "" and replayed.engine.tables.num_requests() == 0
+
+
 def test_tokens_are_handed_over_as_they_come(gpu):
     from prelude_amd import LLM
     folder, cfg, _ = model_folder("a")
