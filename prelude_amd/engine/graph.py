@@ -40,6 +40,8 @@ from __future__ import annotations
 
 import collections
 import dataclasses
+import gc
+import weakref
 from typing import Sequence
 
 import torch
@@ -83,7 +85,7 @@ class StepGraphs:
     SEEN_SHAPES = 512   # shapes of steps with portions remembered as met once
 
     def __init__(self, engine, max_batch: int, cache_size: int = 32, portion_tokens: int = 0):
-        self.engine = engine
+        self.engine = weakref.proxy(engine)   # the engine owns this object: no cycle, so both go when the engine is let go
         self.max_batch = int(max_batch)
         self.cache_size = max(1, int(cache_size))
         self.portion_tokens = int(portion_tokens)
@@ -198,6 +200,11 @@ class StepGraphs:
         torch.cuda.synchronize()
         # The warm-up ran the same launches, so what fails from here on is the capture itself (its pool's memory, an
         # operation that cannot be recorded): the step can still run directly.
+        # No cyclic garbage collection while the stream is being captured: a collection runs the destructors of
+        # whatever dead cycles the process holds, and the destructor of an earlier engine's graph waits for the
+        # device, which is not allowed during a capture and ends the process.  What is dead stays so until after.
+        collecting = gc.isenabled()
+        gc.disable()
         try:
             graph = torch.cuda.CUDAGraph()
             if self._pool is None:
@@ -206,5 +213,8 @@ class StepGraphs:
                 logits = eng.forward(batch)
         except Exception as e:
             raise NotCaptured(f"a step of {[len(e_.tokens) for e_ in entries]} tokens could not be captured: {e}") from e
+        finally:
+            if collecting:
+                gc.enable()
         self.captures += 1
         return _Captured(graph, buffer, logits, stride)

@@ -422,6 +422,47 @@ def test_a_step_with_portions_whose_capture_fails_runs_directly(gpu, monkeypatch
     assert graph_eng.tables.audit() == ""
 
 
+def test_no_garbage_is_collected_while_a_step_is_captured(gpu):
+    """A collection inside a capture would run the destructors of dead cycles there, an earlier engine's graphs among
+    them, whose destructor waits for the device: not allowed while a stream is captured.  So the collector is off
+    exactly while a step is recorded and on again afterwards, also when the capture fails; and an engine that is let
+    go takes its graphs with it at once, with no cycle left for a collection to find."""
+    import gc
+    import weakref
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    folder, cfg, _ = model_folder("a")
+    rng = np.random.default_rng(15)
+    seqs = [rng.integers(0, cfg["vocab_size"], size=40).tolist() for _ in range(2)]
+    eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=256, hip_graph=True))
+    seen = []
+    forward = eng.forward
+
+    def watching(*args):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return forward(*args)
+    eng.forward = watching
+    assert gc.isenabled()
+    for r in range(2):
+        eng.step([StepEntry(r, seqs[r][:30], [29])])
+    for k in range(3):
+        eng.step([StepEntry(r, [seqs[r][30 + k]], [0]) for r in range(2)])
+    assert eng._graphs.captures == 2      # the portion's shape at its second sighting, the decode step
+    assert (True, False) in seen and (False, True) in seen
+    assert all(collecting != capturing for capturing, collecting in seen), seen
+    assert gc.isenabled()
+    del eng.forward       # the class's own again
+
+    graphs = weakref.ref(eng._graphs)
+    captured = [weakref.ref(c.graph) for c in eng._graphs._graphs.values()]
+    gc.disable()
+    try:
+        del eng, forward, watching
+        assert graphs() is None and all(c() is None for c in captured)
+    finally:
+        gc.enable()
+
+
 def test_graph_replays_with_library_products_equal_eager_steps(gpu):
     """A decode step of more than 48 requests multiplies through the library product, also inside a captured
     graph (with its workspace): every replay, with eager steps of other shapes between them, gives the eager
