@@ -55,7 +55,7 @@ def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides
 
 
 def release_memory():
-    """An engine and its captured graphs refer to one another: collect the cycle before the next engine is built."""
+    """Gives the last engine's device memory back before the next engine is built (the caller has dropped it)."""
     import gc
     import torch
     gc.collect()

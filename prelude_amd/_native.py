@@ -38,7 +38,6 @@ _KERNEL_API = {
     "pa_device_arch": (I, [c_char_p, I]),
     "pa_num_compute_units": (I, []),
     "pa_stream_read": (I, [P, P, c_long, P, I]),
-    "pa_overlap_probe": (I, [P, I, I, I, I, P]),
     "pa_embed_gather": (I, [P, I, P, P, P, I, I, I]),
     "pa_carry_tokens": (I, [P, P, P, P, P, I, I, I]),
     "pa_zero_fresh_rows": (I, [P, P, c_long, P, P, I, I]),

@@ -1,6 +1,6 @@
 """Times single kernels against their rooflines on one MI355X.
 
-    python -m prelude_amd.bench_kernels [stream] [overlap] [gemm] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
+    python -m prelude_amd.bench_kernels [stream] [gemm] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
 
 Each line gives the kernel's time (device events around repeated launches,
 operands rotated over copies larger than the caches where the kernel streams
@@ -61,23 +61,6 @@ def bench_stream(dev, shape) -> None:
         out = torch.zeros(blocks, dtype=torch.int32, device=dev)
         us = timeit(lambda i: check(kernels().pa_stream_read(K._stream(), buf.data_ptr(), nbytes, out.data_ptr(), blocks)), 1, iters=10)
         line(f"read 8 GB, {blocks} workgroups of 256 threads", us, nbytes=nbytes)
-
-
-def bench_overlap(dev, shape) -> None:
-    """Whether a SIMD's matrix products and vector instructions run at the same time: an attention step's 34 MFMAs
-    and its 64 vector instructions (16 exponentials), two wavefronts a SIMD, alone and together (probes.hip)."""
-    from ._native import check, kernels
-    out = torch.zeros(512, device=dev)
-    iters, blocks = 2000, int(kernels().pa_num_compute_units())
-    cycles = 2.0 * iters * 34 * 16       # a SIMD's matrix pipe: two wavefronts, 34 products of 16 cycles an iteration
-    cases = ((4, 0, "products only"), (5, 0, "vector work only"), (0, 0, "both, every wavefront in the same order"),
-             (1, 0, "both, a barrier after each phase"), (2, 0, "both, a SIMD's two wavefronts in opposite phases"),
-             (3, 0, "opposite phases, the products at raised priority"),
-             (0, 1, "accumulation registers: same order"), (2, 1, "accumulation registers: opposite phases"))
-    for order, acc, name in cases:
-        us = timeit(lambda i: check(kernels().pa_overlap_probe(K._stream(), order, acc, iters, blocks, out.data_ptr())), 1, iters=5)
-        busy = "" if order == 5 else f"   matrix pipe busy {100 * cycles / (us * 1e-6 * 2.4e9):3.0f} % (at 2.4 GHz)"
-        print(f"{name:52s} {us:9.1f} us{busy}", flush=True)
 
 
 def bench_gemm(dev, shape) -> None:
@@ -191,7 +174,7 @@ def bench_sampling(dev, shape) -> None:
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
-    ap.add_argument("what", nargs="*", help="stream, overlap, gemm, decode, prefill, elementwise, sampling (default: all)")
+    ap.add_argument("what", nargs="*", help="stream, gemm, decode, prefill, elementwise, sampling (default: all)")
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -199,11 +182,11 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     shape = SHAPES[args.shape]
-    todo = args.what or ["stream", "overlap", "gemm", "decode", "prefill", "elementwise", "sampling"]
+    todo = args.what or ["stream", "gemm", "decode", "prefill", "elementwise", "sampling"]
     print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
           f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
     for name in todo:
-        {"stream": bench_stream, "overlap": bench_overlap, "gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
+        {"stream": bench_stream, "gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
          "sampling": bench_sampling}[name](dev, shape)
     return 0
 

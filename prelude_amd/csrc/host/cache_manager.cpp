@@ -30,7 +30,25 @@ void PagePool::grab(int page) {
 // A page that is free has lost its claim, or has just become free: its run may be whole again.
 void PagePool::page_is_unclaimed_and_free(int page) {
   const int r = page / run_;
-  if (++unclaimed_free_[r] == run_len(r) && run_ > 1) runs_.push_back({r, ++run_stamp_[r]});
+  if (++unclaimed_free_[r] == run_len(r) && run_ > 1) {
+    runs_.push_back({r, ++run_stamp_[r]});
+    if (runs_.size() > queue_limit(unclaimed_free_.size())) {
+      std::deque<Entry> live;
+      for (const Entry& e : runs_)
+        if (e.stamp == run_stamp_[e.index]) live.push_back(e);
+      runs_.swap(live);
+    }
+  }
+}
+
+// The queues are only ever popped where a hand-out falls through to them; a pool whose requests keep finding the
+// page behind their last one would let void entries pile up for good.  Past twice the number of things they can
+// validly hold, the void ones are dropped (the order of the others stays): constant work per page on average.
+void PagePool::drop_void_entries() {
+  std::deque<Entry> live;
+  for (const Entry& e : free_)
+    if (e.stamp == stamp_[e.index] && !held_[e.index]) live.push_back(e);
+  free_.swap(live);
 }
 
 int PagePool::take(int64_t owner, int after) {
@@ -73,6 +91,7 @@ bool PagePool::give(int page) {
   held_[page] = 0;
   ++free_count_;
   free_.push_back({page, ++stamp_[page]});
+  if (free_.size() > queue_limit(held_.size())) drop_void_entries();
   page_is_unclaimed_and_free(page);
   return true;
 }
@@ -102,6 +121,8 @@ std::string PagePool::check() const {
   if (free_pages != free_count_) return "the count of free pages is off";
   for (size_t r = 0; r < count.size(); ++r)
     if (count[r] != unclaimed_free_[r]) return "run " + std::to_string(r) + ": the count of unclaimed free pages is off";
+  if (free_.size() > queue_limit(held_.size()) || runs_.size() > queue_limit(unclaimed_free_.size()))
+    return "a queue holds " + std::to_string(std::max(free_.size(), runs_.size())) + " entries, most of them void";
   // every free page can still be reached through the queue
   std::vector<uint8_t> queued(capacity(), 0);
   for (const Entry& e : free_)

@@ -62,6 +62,8 @@ class PagePool {
   int run_len(int r) const { return std::min(run_, capacity() - r * run_); }
   void grab(int page);
   void page_is_unclaimed_and_free(int page);
+  void drop_void_entries();
+  static size_t queue_limit(size_t things) { return 2 * things + 16; }   // entries a queue may hold, void ones included
 
   int run_;
   int free_count_ = 0;

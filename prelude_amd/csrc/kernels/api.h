@@ -14,9 +14,6 @@ int pa_num_compute_units();
 // A kernel that only reads: `bytes` (a multiple of 16) from src by `blocks` workgroups; out holds a word per
 // workgroup.  For measuring the rate at which this device streams memory.
 int pa_stream_read(void* stream, const void* src, long bytes, void* out, int blocks);
-// A measurement: a phase of matrix products and a phase of vector work, `iters` times, in the order `order`
-// (probes.hip) with the accumulators in the vector (0) or the accumulation registers (1); out: 512 floats.
-int pa_overlap_probe(void* stream, int order, int accumulators, int iters, int blocks, void* out);
 // out[t, :] = table[ids[t], :]
 int pa_embed_gather(void* stream, int dtype, const int* ids, const void* table, void* out, int tokens, int hidden,
                     int vocab);

@@ -222,8 +222,9 @@ __device__ __forceinline__ void move_reference(HeadState<HD>& st, float mx_lane,
   constexpr int OT = HeadState<HD>::OT;
   const float mx = xor_max16_32(mx_lane);
   const bool moved = mx > st.lim;   // from -inf any finite score; -inf against -inf is false
-  // 2^((m_before - mx) c); for a column's first keys m_before c counts as 0, and its sums are zero anyway
-  const float alpha = moved ? __builtin_amdgcn_exp2f(-st.shift - mx * c) : 1.0f;
+  // 2^((m_before - mx) c).  A column's first keys rescale nothing (its sums are zero): the factor is 1 there and
+  // not 2^(-mx c), which for a first score far below zero is +inf and would turn the zero sums into NaN
+  const float alpha = moved && st.lim != -INFINITY ? __builtin_amdgcn_exp2f(-st.shift - mx * c) : 1.0f;
   if (moved) {
     st.lim = mx + over;
     st.shift = -mx * c;

@@ -97,13 +97,16 @@ class StepGraphs:
         self.captures = 0
         self.evictions = 0
 
-    def eligible(self, entries: Sequence, starts: Sequence[int] = ()) -> bool:
+    def eligible(self, entries: Sequence, starts: Sequence[int]) -> bool:
         """Whether the step is to be replayed.  A step of single tokens is, from its first time; a step with
-        portions from the second time its shape is met (the first time only remembers the shape)."""
+        portions from the second time its shape is met (the first time only remembers the shape).  A shape whose
+        capture has failed is not tried again."""
         if not 1 <= len(entries) <= self.max_batch:
             return False
+        if len(starts) != len(entries):
+            raise ValueError(f"{len(entries)} entries but {len(starts)} starts")
         if self._single_tokens(entries):
-            return True
+            return self._key(entries, starts) not in self._refused
         if self.portion_tokens <= 0 or sum(len(e.tokens) for e in entries) > self.portion_tokens:
             return False
         if any(len(e.want) > 1 for e in entries):
@@ -146,9 +149,9 @@ class StepGraphs:
         return K.decode_context_bound(max(ends), page) // page
 
     def run(self, entries: Sequence, starts: Sequence[int], carried=None):
-        """The step's logits from its graph, captured first if need be.  None if the step has portions and its
-        capture failed (no memory for its activations, say): the caller then runs it directly, as it will every
-        later step of that shape.  A step of single tokens has no such way out: its failure is the caller's."""
+        """The step's logits from its graph, captured first if need be.  None if its capture failed (no memory
+        for its activations, say): the caller then runs it directly, which gives the same bits, as it will every
+        later step of that shape."""
         eng = self.engine
         key = self._key(entries, starts)
         stride = key[-1]
@@ -162,8 +165,6 @@ class StepGraphs:
             try:
                 cap = self._capture(entries, starts, stride, carried)
             except NotCaptured:
-                if self._single_tokens(entries):
-                    raise
                 self._refused[key] = None
                 while len(self._refused) > self.SEEN_SHAPES:
                     self._refused.popitem(last=False)

@@ -603,7 +603,10 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
-DECODE_SPLIT_KEYS = 256   # keys per split of the decode kernel: fixed, so a token's result never depends on its batch
+# Keys per split of the decode kernel: fixed, so which keys a split sums never depends on the batch.  (The order in
+# which a split's steps are added does, in the last bits: grids of 769 to 1,536 workgroups run with two wavefronts a
+# workgroup instead of four.  Steps of the same size on the same side of those limits give the same bits.)
+DECODE_SPLIT_KEYS = 256
 DECODE_CONTEXT_STEP = 1024   # the longest context of a step counts rounded up to this many tokens (whole pages)
 
 

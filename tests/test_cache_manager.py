@@ -254,6 +254,31 @@ def test_random_orders_lose_nothing(seed):
     assert [t.free_pages(g) for g in range(2)] == [g[0] for g in groups] and t.free_state_slots() == 3
 
 
+def test_a_long_session_does_not_pile_up_stale_queue_entries():
+    """Requests that always find the page behind their last one (a lightly used pool) never make the pool fall
+    back to its first-in first-out queue, which is the only place stale entries used to be dropped: the audit
+    fails when a queue holds more than about twice what it can validly hold, and it must stay fast."""
+    import time
+    t = PageTables(16, [(1024, 0)])
+    for i in range(20000):
+        t.open(i)
+        t.reserve(i, 128)                  # eight pages: a whole run
+        t.commit(i, 128)
+        t.close(i)
+        if i % 5000 == 4999:
+            assert t.audit() == ""
+    t0 = time.time()
+    assert t.audit() == "" and t.free_pages(0) == 1024
+    assert time.time() - t0 < 0.5
+    # with a window pages come back one at a time while the request lives
+    t = PageTables(4, [(64, 8)])
+    t.open(0)
+    for n in range(1, 6000):
+        t.reserve(0, n)
+        t.commit(0, n)
+    assert t.audit() == ""
+
+
 def test_pool_sizes_per_group():
     """A group with a window needs pages for what a window and a portion span, per request that may run; the
     Python rule used to size the pools is the manager's own."""

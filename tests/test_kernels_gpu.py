@@ -111,6 +111,18 @@ def test_gemm_plain_f32(gpu, m, n, k):
     assert torch.equal(one[0], out[m // 2])
 
 
+def test_gemm_plain_f32_sums_long_rows_without_drift(gpu):
+    """A row of 9,728 terms (the widest inner size of the 4B shape): the sixteens are added with a compensated sum,
+    which keeps the error near 1e-7 of the largest output; a plain running sum in 32-bit is off by some 4e-6 there
+    and would fail this.  All terms of one sign, so that rounding cannot cancel."""
+    m, n, k = 4, 96, 9728
+    x, w = rnd(m, k).abs(), rnd(n, k, seed=1).abs()
+    ref = x.double() @ w.double().T
+    out = K().gemm_plain(x.to(gpu), w.to(gpu))
+    err = float((out.double().cpu() - ref).abs().max()) / float(ref.abs().max())
+    assert err < 4e-7, f"relative error {err:.2e} of the largest output"
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 509, 96), (8, 2560, 4096), (40, 331, 80), (300, 192, 96), (64, 6144, 2560)])
 def test_linear_bf16(gpu, m, n, k):
     x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
@@ -620,6 +632,28 @@ def test_mfma_attention_far_key_and_edges(gpu):
             assert (float(out[-1].float().abs().max()) > 50.0) == seen
 
 
+@pytest.mark.parametrize("hd,page,window", [(64, 16, 0), (128, 16, 0), (64, 8, 40), (32, 32, 70), (128, 64, 33)])
+def test_mfma_attention_first_keys_far_below_zero(gpu, hd, page, window):
+    """The first keys a query sees score about -104 (2^-150 as a weight against a reference of 0), the later ones
+    around zero: the first step's rescaling factor must not be formed from nothing (2^150 = inf, times the still
+    empty sums = NaN).  Contexts that end one key into a step of 32, inside the cold stretch and behind it; with a
+    window, queries whose first visible keys are the cold stretch's last ones."""
+    cold = 64
+
+    def trick(i, q, k, v):
+        q[:, :, 0] = 12.0
+        k[:, :, 0] = 0
+        k[:cold, :, 0] = -104.0 * math.sqrt(hd) / 12.0
+
+    seqs = [(300, 1), (33, 1), (65, 1), (97, 1), (64, 1), (300, 300), (200, 50), (70, 6), (129, 1)]
+    out, ref = paged_case(gpu, torch.bfloat16, 4, 2, hd, page, seqs, window, seed=8, scale_trick=trick, kernel="mfma")
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.bfloat16)
+    out, ref = paged_case(gpu, torch.float32, 4, 2, hd, page, seqs, window, seed=8, scale_trick=trick)
+    assert not bool(torch.isnan(out).any())
+    close(out, ref, torch.float32, f32=3e-6)
+
+
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0),
                                                    (8, 2, 128, 128, 0), (4, 2, 64, 256, 100)])
 def test_prefill_attention_every_cut(gpu, nh, nkv, hd, page, window):
@@ -791,6 +825,23 @@ def test_mfma_attention_batch_and_page_independence(gpu):
     assert torch.equal(one, other)                               # other page size, other pages
 
 
+def test_decode_attention_on_either_side_of_the_grid_limits(gpu):
+    """The same sequence alone (128 workgroups: four wavefronts a workgroup), among eight (1,024: two) and among
+    thirteen (1,664: four again).  Which keys a split sums is the same in all three; the order in which a split's
+    steps are added is not, so the results agree to rounding, not to the bit, across the limits -- and to the bit
+    on the same side of them."""
+    first = (4096, 1)
+    outs = []
+    for others in (0, 7, 12):
+        seqs = [first] + [(4000 - 50 * i, 1) for i in range(others)]
+        out, ref = paged_case(gpu, torch.bfloat16, 32, 8, 128, 16, seqs, 0, seed=21, kernel="mfma")
+        close(out, ref, torch.bfloat16)
+        outs.append((out[0].double().cpu(), ref[0]))
+    (a, ref), (b, _), (c, _) = outs
+    assert torch.equal(a, c)                                  # four wavefronts both times
+    assert float((a - b).abs().max()) <= tol(torch.bfloat16, ref)
+
+
 @pytest.mark.parametrize("nh,nkv,hd,page,window,norm,ctxs", [
     (32, 8, 128, 16, 0, True, [1, 17, 256, 257, 700, 33, 512]), (8, 8, 64, 8, 0, True, [1, 17, 256, 257, 700, 33, 512]),
     (16, 1, 128, 64, 40, True, [1, 17, 256, 257, 700, 33, 512]), (4, 2, 64, 16, 0, False, [1, 17, 256, 257, 700, 33, 512]),
@@ -804,6 +855,13 @@ def test_decode_attention_takes_the_raw_projection(gpu, nh, nkv, hd, page, windo
     assert not K().attention_decode_fused_supported(nh, nkv, hd, hd // 2, page)      # partial rotation
     assert not K().attention_decode_fused_supported(34, 2, 128, 128, 16)             # more than 16 heads per KV head
     assert not K().attention_decode_fused_supported(4, 2, 96, 96, 16)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,window,norm", [(8, 2, 128, 16, 0, True), (4, 4, 64, 8, 0, False),
+                                                         (8, 1, 128, 32, 40, True)])
+def test_decode_attention_of_the_raw_projection_with_first_keys_far_below_zero(gpu, nh, nkv, hd, page, window, norm):
+    """As ``test_mfma_attention_first_keys_far_below_zero``, for the kernel that norms and rotates its own query."""
+    raw_projection_case(gpu, nh, nkv, hd, page, window, norm, [300, 33, 65, 97, 66, 40, 129, 4096], cold=64)
 
 
 @pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_ATTENTION", "10")) // 2)))
@@ -820,35 +878,54 @@ def test_drawn_raw_projection_in_grids_of_two_wavefronts(gpu, seed):
     raw_projection_case(gpu, nh, nkv, hd, page, window, bool(seed % 2), ctxs)
 
 
-def raw_projection_case(gpu, nh, nkv, hd, page, window, norm, ctxs):
+def raw_projection_case(gpu, nh, nkv, hd, page, window, norm, ctxs, cold=0):
+    """``cold`` > 0: the first ``cold`` keys of every sequence score about -104 against its query (the heads of a
+    KV head then share one query, so that one key can be that cold for all of them)."""
     eps = 1e-6
     t = len(ctxs)
     listed = [i for i in range(t) if i != 5]           # the sixth sequence is not in the list
     g = torch.Generator().manual_seed(3)
+    group = nh // nkv
+    scale = 1.0 / math.sqrt(hd)
+    qkv = (2.0 * torch.randn(t, (nh + 2 * nkv) * hd, generator=g)).to(torch.bfloat16)
+    if cold:
+        heads = qkv[:, : nh * hd].reshape(t, nkv, group, hd)
+        heads[:] = heads[:, :, :1]
+    qw = (1.0 + 0.2 * rnd(hd, seed=1)) if norm else None
+    kw = (1.0 + 0.2 * rnd(hd, seed=2)) if norm else None
+    cos, sin = pm.rope_tables(hd, max(ctxs), 10000.0, torch.float32)
+    # what the plain functions make of the projection: normed, rotated queries and keys, values as they are
+    rq, rk, rv = qk_reference(qkv, qw, kw, cos, sin, torch.tensor([c - 1 for c in ctxs]), nh, nkv, hd, hd, eps)
     total_pages = sum(-(-c // page) for c in ctxs) + 2
     perm = torch.randperm(total_pages, generator=g).tolist()
     stride = max(-(-c // page) for c in ctxs)
     table = torch.full((t, stride), -1, dtype=torch.int32)
     kc = torch.zeros(total_pages, nkv, page, hd, dtype=torch.bfloat16)
     vc = torch.zeros(total_pages, nkv, hd, page, dtype=torch.bfloat16)
-    slots = []
+    slots, plain = [], []
     for i, c in enumerate(ctxs):
         for p in range(-(-c // page)):
             table[i, p] = perm.pop()
         hist = c - 1                                   # keys before the token's own
+        k_hist = torch.randn(hist, nkv, hd, generator=g)
+        v_hist = torch.randn(hist, nkv, hd, generator=g).to(torch.bfloat16)
+        if cold:
+            qdir = rq[i, ::group].float()              # [nkv, hd]: the query all heads of a KV head share
+            k_hist[:cold] = -104.0 / scale * qdir / (qdir * qdir).sum(-1, keepdim=True)
+        k_hist = k_hist.to(torch.bfloat16)
         for p in range(-(-hist // page)):
             n, ph = min(page, hist - p * page), int(table[i, p])
-            kc[ph, :, :n] = torch.randn(nkv, n, hd, generator=g).to(torch.bfloat16)
-            vc[ph, :, :, :n] = torch.randn(nkv, hd, n, generator=g).to(torch.bfloat16)
+            kc[ph, :, :n] = k_hist[p * page: p * page + n].transpose(0, 1)
+            vc[ph, :, :, :n] = v_hist[p * page: p * page + n].permute(1, 2, 0)
         slots.append(int(table[i, (c - 1) // page]) * page + (c - 1) % page)
-    qkv = (2.0 * torch.randn(t, (nh + 2 * nkv) * hd, generator=g)).to(torch.bfloat16)
-    qw = (1.0 + 0.2 * rnd(hd, seed=1)) if norm else None
-    kw = (1.0 + 0.2 * rnd(hd, seed=2)) if norm else None
-    cos, sin = pm.rope_tables(hd, max(ctxs), 10000.0, torch.float32)
+        # the plain attention of the token over its history and its own key and value (as the cache will hold them)
+        keys = torch.cat([k_hist.double(), rk[i: i + 1].to(torch.bfloat16).double()])
+        values = torch.cat([v_hist.double(), rv[i: i + 1]])
+        plain.append(pm.attention(rq[i: i + 1].to(torch.bfloat16).double(), keys, values, scale, window=window or None,
+                                  q_offset=c - 1)[0])
     dev = lambda x: None if x is None else x.to(gpu)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
     pos, sl, seqs, cu, cl = i32([c - 1 for c in ctxs]), i32(slots), i32(listed), i32(list(range(t + 1))), i32(ctxs)
-    scale = 1.0 / math.sqrt(hd)
     assert K().attention_decode_fused_supported(nh, nkv, hd, hd, page)
     # the two kernels
     k1, v1 = kc.to(gpu), vc.to(gpu)
@@ -859,8 +936,11 @@ def raw_projection_case(gpu, nh, nkv, hd, page, window, norm, ctxs):
     k2, v2 = kc.to(gpu), vc.to(gpu)
     out2 = K().attention_decode_fused(dev(qkv), dev(qw), dev(kw), dev(cos), dev(sin), sl, eps, k2, v2, dev(table),
                                       seqs, cu, cl, nh, max(ctxs), window, scale)
+    assert not bool(torch.isnan(out2[listed]).any()) and not bool(torch.isnan(out1[listed]).any())
     for i in listed:
         close(out2[i], out1[i].double().cpu(), torch.bfloat16)
+        close(out2[i], plain[i], torch.bfloat16)       # and each against the plain functions, not only one another
+        close(out1[i], plain[i], torch.bfloat16)
         ph, off = slots[i] // page, slots[i] % page
         assert torch.equal(v2[ph, :, :, off], v1[ph, :, :, off])
         close(k2[ph, :, off], k1[ph, :, off].double().cpu(), torch.bfloat16)

@@ -237,6 +237,111 @@ def test_one_layer_by_hand():
     assert torch.allclose(got, want, atol=1e-5)     # the angle goes through float32 in the plain implementation
 
 
+def _library_model(cfg, w, toks):
+    """The whole decoder put together from library routines only (``F.embedding``, ``F.linear``, ``F.rms_norm``,
+    ``F.silu``, ``F.scaled_dot_product_attention`` with its own default scale and its own causal mask,
+    ``repeat_interleave`` for the grouped heads) and the rotation in the form the reference's test fixes,
+    x * cat(cos, cos) + rotate_half(x) * cat(sin, sin) (crates/prelude-core/tests/tensor_ops.rs:1684-1691).  It
+    shares no function with the plain implementation: what it pins is the wiring -- which norm goes where, that
+    values are not normed, the scale 1 / sqrt(head_dim), both residual sums, the final norm, the head."""
+    w = {k: v.double() for k, v in w.items()}
+    nh, nkv, hd, hid = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["hidden_size"]
+    eps, bias = cfg["rms_norm_eps"], cfg["attention_bias"]
+    toks = torch.as_tensor(toks)
+    s = toks.shape[0]
+    # the angle in 32-bit, as the reference forms it (crates/prelude-core/src/models/commons/attn_utils.rs:39-49)
+    inv_freq = (1.0 / torch.tensor(cfg["rope_theta"], dtype=D).pow(torch.arange(0, hd, 2, dtype=D) / hd).float()).float()
+    ang = torch.outer(torch.arange(s, dtype=torch.float32), inv_freq).double()
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1)[:, None, :], torch.cat([ang.sin(), ang.sin()], -1)[:, None, :]
+    x = F.embedding(toks, w["model.embed_tokens.weight"])
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        a = p + "self_attn."
+        b = (lambda n: w[a + n + ".bias"]) if bias else (lambda n: None)
+        h = F.rms_norm(x, (hid,), w[p + "input_layernorm.weight"], eps)
+        q = F.linear(h, w[a + "q_proj.weight"], b("q_proj")).view(s, nh, hd)
+        k = F.linear(h, w[a + "k_proj.weight"], b("k_proj")).view(s, nkv, hd)
+        v = F.linear(h, w[a + "v_proj.weight"], b("v_proj")).view(s, nkv, hd)
+        q = F.rms_norm(q, (hd,), w[a + "q_norm.weight"], eps)
+        k = F.rms_norm(k, (hd,), w[a + "k_norm.weight"], eps)
+        q = q * cos + _rotate_half(q) * sin
+        k = k * cos + _rotate_half(k) * sin
+        k, v = k.repeat_interleave(nh // nkv, dim=1), v.repeat_interleave(nh // nkv, dim=1)
+        window = pm.layer_window(cfg, i)
+        if window is None:
+            o = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        else:
+            r, c = torch.arange(s)[:, None], torch.arange(s)[None, :]
+            o = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1),
+                                               attn_mask=(c <= r) & (c > r - window))
+        x = x + F.linear(o.transpose(0, 1).reshape(s, nh * hd), w[a + "o_proj.weight"], b("o_proj"))
+        h = F.rms_norm(x, (hid,), w[p + "post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    x = F.rms_norm(x, (hid,), w["model.norm.weight"], eps)
+    return F.linear(x, w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"])
+
+
+def test_model_is_the_library_routines_wired_together(tiny):
+    cfg, w = tiny
+    toks = torch.randint(0, cfg["vocab_size"], (60,)).tolist()
+    got, want = pm.forward(cfg, w, toks), _library_model(cfg, w, toks)
+    assert float((got - want).abs().max()) < 1e-9 * max(1.0, float(want.abs().max()))
+    # each of these plausible mistakes moves the library model's logits by far more than that bound, so the
+    # agreement above is not one that any wiring would reach
+    p = "model.layers.0.self_attn."
+    swapped = dict(w)
+    swapped[p + "q_norm.weight"], swapped[p + "k_norm.weight"] = w[p + "k_norm.weight"], w[p + "q_norm.weight"]
+    assert float((_library_model(cfg, swapped, toks) - want).abs().max()) > 1e-5
+
+
+def _attention_block_inputs(cfg, seed):
+    w = {k: v.double() for k, v in pm.random_weights(cfg, seed=seed, std=0.3, norm_std=0.3).items()}
+    h = torch.randn(9, cfg["hidden_size"], dtype=D)
+    cos_t, sin_t = pm.rope_tables(cfg["head_dim"], 16, cfg["rope_theta"], D)
+    return w, h, cos_t[:9], sin_t[:9]
+
+
+def test_values_are_not_normed():
+    """Scaling W_v by c scales the block's output by c (o_proj is linear): a norm on V would undo the scale."""
+    cfg = dict(pm.tiny_config_b(), num_hidden_layers=1)
+    w, h, cos, sin = _attention_block_inputs(cfg, 3)
+    base = pm.attention_block(cfg, w, 0, h, cos, sin)
+    w2 = dict(w)
+    w2["model.layers.0.self_attn.v_proj.weight"] = 3.0 * w["model.layers.0.self_attn.v_proj.weight"]
+    assert torch.allclose(pm.attention_block(cfg, w2, 0, h, cos, sin), 3.0 * base, atol=1e-10)
+    # ... while queries and keys are: scaling W_q or W_k changes nothing (up to eps)
+    for name in ("q_proj", "k_proj"):
+        w3 = dict(w)
+        w3[f"model.layers.0.self_attn.{name}.weight"] = 5.0 * w[f"model.layers.0.self_attn.{name}.weight"]
+        assert torch.allclose(pm.attention_block(cfg, w3, 0, h, cos, sin), base, rtol=1e-4, atol=1e-4)
+
+
+def test_heads_are_independent_and_keep_their_kv_head():
+    """With o_proj the identity the block's output is the heads side by side.  Exchanging two query heads of one
+    KV head exchanges their outputs and touches no other head; exchanging the two KV heads exchanges the outputs of
+    their groups only if the query heads go with them."""
+    cfg = dict(pm.tiny_config_a(), num_hidden_layers=1)              # 4 heads over 2 KV heads, 4 * 16 = hidden
+    w, h, cos, sin = _attention_block_inputs(cfg, 4)
+    p = "model.layers.0.self_attn."
+    w[p + "o_proj.weight"] = torch.eye(64, dtype=D)
+    base = pm.attention_block(cfg, w, 0, h, cos, sin).reshape(9, 4, 16)
+    w2 = dict(w)
+    wq = w[p + "q_proj.weight"].reshape(4, 16, 64)
+    w2[p + "q_proj.weight"] = wq[[1, 0, 2, 3]].reshape(64, 64)       # heads 0 and 1 share KV head 0
+    out = pm.attention_block(cfg, w2, 0, h, cos, sin).reshape(9, 4, 16)
+    assert torch.allclose(out, base[:, [1, 0, 2, 3]], atol=1e-12)
+    w3 = dict(w)
+    w3[p + "q_proj.weight"] = wq[[2, 3, 0, 1]].reshape(64, 64)       # the groups exchanged, KV heads with them
+    for name in ("k_proj", "v_proj"):
+        w3[p + name + ".weight"] = w[p + name + ".weight"].reshape(2, 16, 64)[[1, 0]].reshape(32, 64)
+    out = pm.attention_block(cfg, w3, 0, h, cos, sin).reshape(9, 4, 16)
+    assert torch.allclose(out, base[:, [2, 3, 0, 1]], atol=1e-12)
+    w4 = dict(w3)
+    w4[p + "q_proj.weight"] = w[p + "q_proj.weight"]                 # KV heads exchanged alone: other results
+    assert not torch.allclose(pm.attention_block(cfg, w4, 0, h, cos, sin).reshape(9, 4, 16), base, atol=1e-3)
+
+
 def test_tied_head_uses_the_embedding():
     cfg = pm.tiny_config_a()
     w = pm.random_weights(cfg, seed=2)

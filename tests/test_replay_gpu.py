@@ -248,6 +248,22 @@ def test_trace_run_program_from_a_bare_config(gpu, tmp_path):
     assert float(np.abs(np.fromfile(out2 / "0.f32", dtype="<f4").reshape(-1, cfg["vocab_size"]) - load(0)).max()) > 1e-3
 
 
+def test_a_seed_names_one_model_on_the_cpu_and_on_the_gpu(gpu):
+    """The random-weights mode draws the same values wherever it draws: what ``--write-model`` puts into a folder
+    from the CPU is what ``--random-weights`` alone draws on the device."""
+    from prelude_amd.weights import random_tensors, random_tensors_on_device
+    import plain_model as pm
+    cfg = pm.tiny_config_c()
+    host = random_tensors(cfg, 7, std=0.05, norm_std=0.02, dtype=torch.float32, device="cpu")
+    dev = random_tensors_on_device(cfg, 7, gpu, std=0.05, norm_std=0.02, dtype=torch.float32)
+    assert set(host) == set(dev)
+    for name in host:
+        assert torch.equal(host[name], dev[name].cpu()), name
+    host16 = random_tensors(cfg, 7, dtype=torch.bfloat16, device="cpu")
+    dev16 = random_tensors_on_device(cfg, 7, gpu, dtype=torch.bfloat16)
+    assert all(torch.equal(host16[n].float(), dev16[n].cpu().float().to(torch.bfloat16).float()) for n in host16)
+
+
 def test_graph_replays_equal_eager_steps(gpu):
     """Decode steps replayed from HIP graphs, with eager work (prompt portions, other batch sizes) between the
     replays: every replay gives the logits of the eager step, bit for bit."""
@@ -377,9 +393,9 @@ def test_graph_replays_of_steps_with_portions_equal_eager_steps(gpu):
     assert graph_eng.tables.audit() == ""
 
 
-def test_a_step_with_portions_whose_capture_fails_runs_directly(gpu, monkeypatch):
-    """The capture of a step with portions is an extra: if it fails (here: made to), the step runs directly and
-    gives the direct run's logits, its shape is not tried again, and decode steps are captured as ever."""
+def test_a_step_whose_capture_fails_runs_directly(gpu, monkeypatch):
+    """The capture of a step is an extra: if it fails (here: made to), the step runs directly and gives the direct
+    run's logits, its shape is not tried again, and other shapes are captured as ever."""
     import contextlib
     from prelude_amd.config import EngineConfig
     from prelude_amd.engine import Engine, StepEntry
@@ -410,13 +426,17 @@ def test_a_step_with_portions_whose_capture_fails_runs_directly(gpu, monkeypatch
         for k in range(3):
             outs.append(eng.step([StepEntry(r, [seqs[r][40 + k]], [0]) for r in range(4)]).cpu())
         if break_portions:
+            refusing.portions = True
+        for k in range(2):    # a decode step of another batch size whose capture fails as well: it runs directly too
+            outs.append(eng.step([StepEntry(r, [seqs[r][43 + k]], [0]) for r in range(2)]).cpu())
+        if break_portions:
             monkeypatch.undo()
         return eng, outs
 
     eager_eng, eager = play(False, False)
     graph_eng, graphed = play(True, True)
-    assert graph_eng._graphs.captures == 1 and graph_eng._graphs.replays == 3       # the decode step only
-    assert len(graph_eng._graphs._refused) == 1
+    assert graph_eng._graphs.captures == 1 and graph_eng._graphs.replays == 3       # the decode step of four only
+    assert len(graph_eng._graphs._refused) == 2
     for i, (a, b) in enumerate(zip(eager, graphed)):
         assert torch.equal(a, b), f"step {i}"
     assert graph_eng.tables.audit() == ""
