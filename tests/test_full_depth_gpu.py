@@ -1,11 +1,9 @@
 """The whole Qwen3-4B shape (36 layers, vocabulary 151,936, random weights) against the plain implementation, in
 32-bit and in bfloat16: whole prompts, portions down to two tokens, and single tokens.  The plain implementation
-takes a minute or two on the CPU and tens of GB of memory for it, so this runs only when asked for:
-
-    PRELUDE_AMD_FULL_DEPTH=1 python -m pytest tests/test_full_depth_gpu.py -m gpu -x -q
+takes about a minute on the CPU and some 50 GB of host memory for it (the weights once in 32-bit, once in
+64-bit), so the test is skipped only where the host has less than that to spare.
 """
 import gc
-import os
 
 import numpy as np
 import pytest
@@ -14,9 +12,23 @@ import torch
 import plain_model as pm
 from helpers import tolerance
 
+HOST_BYTES_NEEDED = 56 << 30
+
+
+def _host_memory_available() -> int:
+    try:
+        with open("/proc/meminfo") as f:
+            for line in f:
+                if line.startswith("MemAvailable:"):
+                    return int(line.split()[1]) * 1024
+    except OSError:
+        pass
+    return 0
+
+
 pytestmark = [pytest.mark.gpu,
-              pytest.mark.skipif(os.environ.get("PRELUDE_AMD_FULL_DEPTH") != "1",
-                                 reason="minutes of CPU time for the plain implementation: set PRELUDE_AMD_FULL_DEPTH=1")]
+              pytest.mark.skipif(_host_memory_available() < HOST_BYTES_NEEDED,
+                                 reason="the plain implementation of a 4 G parameter model needs 56 GB of host memory")]
 
 QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936, hidden_size=2560,
                 intermediate_size=9728, num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8,
@@ -26,7 +38,7 @@ QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_si
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_all_layers_of_the_4b_shape(gpu, dtype):
+def test_all_layers_of_the_4b_shape(gpu, dtype, capsys):
     from prelude_amd.config import EngineConfig
     from prelude_amd.engine import Engine, StepEntry
     from prelude_amd.weights import random_tensors_on_device
@@ -34,23 +46,27 @@ def test_all_layers_of_the_4b_shape(gpu, dtype):
     torch_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
     n = 160
     toks = np.random.default_rng(3).integers(0, cfg["vocab_size"], size=n).tolist()
+
+    def say(line):            # past pytest's capture: a minute without a line would look like a hang from outside
+        with capsys.disabled():
+            print(line, flush=True)
     weights = {k: v.float().cpu() for k, v in
                random_tensors_on_device(cfg, 0, gpu, std=0.02, norm_std=0.01, dtype=torch_dtype).items()}
+    say(f"[full depth, {dtype}] the plain implementation over 36 layers on the CPU ...")
     ref = pm.forward(cfg, weights, toks)
-    # The bound.  The suite's own (1e-5 of the largest logit in 32-bit, a tenth of the logits' spread in bfloat16)
-    # was measured on models of two to four layers; through 36 layers the roundings add up further, and how far is
-    # measured here rather than assumed: the plain implementation itself in this precision (every operation rounded
-    # to it) against itself in 64-bit.  The engine, which keeps its norms, softmax and residual sums in 32-bit, has to
-    # be at least that close.
-    plain = float((pm.forward(cfg, weights, toks, dtype=torch_dtype).double() - ref).abs().max())
-    bound = max(tolerance(dtype, ref), plain)
-    print(f"{dtype}: the plain implementation in {dtype} is off by {plain:.3e}; the suite's bound {tolerance(dtype, ref):.3e}")
+    say(f"[full depth, {dtype}] ... done; the engine")
+    # The bound.  In 32-bit the suite's own (1e-5 of the largest logit).  In bfloat16 the suite's tenth of the
+    # logits' spread was measured on models of two to four layers; through 36 layers the roundings add up further:
+    # the engine, which keeps its norms, softmax and residual sums in 32-bit, measured 0.17 to 0.21 of the spread
+    # here, the plain implementation with every operation rounded to bfloat16 0.35.  A
+    # quarter of the spread it is: what a lost split of 256 keys moves a logit by at the least.
+    bound = tolerance(dtype, ref) if dtype == "float32" else 0.25 * float(ref.std())
     del weights
     gc.collect()
 
     def check(got, what):
         err = float((got.double() - ref).abs().max())
-        print(f"{dtype}: {what}: max |engine - plain| = {err:.3e} (bound {bound:.3e}, logits' spread {float(ref.std()):.3f})")
+        say(f"[full depth, {dtype}] {what}: max |engine - plain| = {err:.3e} (bound {bound:.3e}, logits' spread {float(ref.std()):.3f})")
         assert err <= bound, what
 
     eng = Engine.from_config(cfg, EngineConfig(dtype=dtype, page_size=16, max_cache_tokens=3 * 192), seed=0)

@@ -651,7 +651,10 @@ def test_mfma_attention_first_keys_far_below_zero(gpu, hd, page, window):
     close(out, ref, torch.bfloat16)
     out, ref = paged_case(gpu, torch.float32, 4, 2, hd, page, seqs, window, seed=8, scale_trick=trick)
     assert not bool(torch.isnan(out).any())
-    close(out, ref, torch.float32, f32=3e-6)
+    # a cold key's dot product holds one term of 12 x 69 sqrt(hd / 64) = 832 ..: summed in 32-bit it is off by up to
+    # some 2e-4, 2.5e-5 in the exponent, and a query that sees cold keys only weighs them against each other with
+    # that relative error.  The bound follows the inputs' size; a lost or misread key moves the output by O(1).
+    close(out, ref, torch.float32, f32=2e-5)
 
 
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0),

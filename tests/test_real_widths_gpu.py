@@ -157,3 +157,50 @@ def test_decoding_far_into_a_context_from_graphs(gpu):
         check(np.concatenate(got[rid]), ref[s0:s0 + 14], "bfloat16", f"request decoding from position {s0}")
     r.step([], list(starts))
     assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
+@functools.lru_cache(maxsize=None)
+def context_model():
+    """The same widths and small vocabulary for a sequence of 4,100 tokens; the plain implementation in 32-bit (six
+    seconds on the CPU).  Measured with the plain implementation: a split of 256 keys left out of the first
+    layer's attention moves the last positions' logits by 0.9 to 1.3 of their spread wherever the split lies, one
+    left out of the second layer's by 0.05 to 0.15; the plain implementation with every operation rounded to
+    bfloat16 is off by 0.07, and the bound is a tenth of the spread."""
+    from prelude_amd.weights import write_safetensors
+    cfg = dict(wide_config(), vocab_size=4099, eos_token_id=4098, max_position_embeddings=4352)
+    w = pm.random_weights(cfg, seed=9, std=0.02, norm_std=0.02)
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    tmp = tempfile.TemporaryDirectory(prefix="prelude_amd_test_context_")
+    _keep.append(tmp)
+    with open(os.path.join(tmp.name, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(tmp.name, "model.safetensors"), w)
+    toks = torch.randint(0, cfg["vocab_size"], (4100,), generator=torch.Generator().manual_seed(33)).tolist()
+    return tmp.name, toks, pm.forward(cfg, {k: v.float() for k, v in w.items()}, toks, dtype=torch.float32).double()
+
+
+def test_eight_requests_decode_at_4096_tokens_from_graphs(gpu):
+    """The step the benchmark times, against the plain implementation: eight requests with some 4,000 tokens behind
+    them feed one token each, twelve steps, replayed from one captured graph.  Eight KV heads x 16 splits x 8
+    sequences are 1,024 workgroups: the decode attention that takes the raw projection in its two-wavefront form,
+    with the merge of 16 splits.  One request starts on a split's edge (3,840 = 15 x 256), one a token behind it,
+    one on a page's edge (4,000), and the last ends at 4,096 exactly."""
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref = context_model()
+    starts = [3840, 3841, 3900, 4000, 4032, 4070, 4080, 4084]
+    steps = 12
+    r = TraceRunner(folder, "bfloat16", len(starts) * 4160, page_size=16)
+    assert r.engine._graphs is not None
+    for i, s0 in enumerate(starts):
+        for lo in range(0, s0, 2048):
+            r.step([{"id": i, "tokens": toks[lo:min(s0, lo + 2048)], "want": []}])
+    rows = [[] for _ in starts]
+    for k in range(steps):
+        out = r.step([{"id": i, "tokens": [toks[s0 + k]], "want": [0]} for i, s0 in enumerate(starts)])
+        for i in range(len(starts)):
+            rows[i].append(out[i:i + 1])
+    assert r.engine._graphs.replays == steps and r.engine._graphs.captures == 1
+    for i, s0 in enumerate(starts):
+        check(np.concatenate(rows[i]), ref[s0:s0 + steps], "bfloat16", f"request decoding from position {s0}")
+    r.step([], list(range(len(starts))))
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
