@@ -55,6 +55,8 @@ _KERNEL_API = {
     "pa_gemm_mid_parts": (c_long, [I, I, I]),
     "pa_gemm_mid": (I, [P, I, I, P, P, P, P, P, I, I, I, c_long, c_long, I, I]),
     "pa_sum_slices": (I, [P, I, P, P, I, c_long]),
+    "pa_gemm_tall_shape": (None, [I, I, I, I, IP]),
+    "pa_gemm_tall": (I, [P, I, P, P, P, P, P, I, I, I, c_long, c_long, I, I, I]),
     "pa_rmsnorm_slices": (I, [P, I, P, I, c_long, P, P, P, P, I, I, F]),
     "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
     "pa_attn_mfma_supports": (I, [I, I]),

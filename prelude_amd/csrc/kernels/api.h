@@ -69,6 +69,13 @@ int pa_gemm_mid_slices(int n, int k);
 long pa_gemm_mid_parts(int m, int n, int slices);
 int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
                 float* parts, int m, int n, int k, long ldx, long ldc, int slices, int waves);
+// C = X W^T for any number of rows from the weight in tiles, the output tiled both ways (gemm_tall.hip): 16 mt rows
+// of X by 64 nt rows of W a workgroup (mt, nt = 0, 0: the launcher's choice, what pa_gemm_tall_shape puts into
+// out[0], out[1]).  epilogue 0: C (+ bias) in bfloat16; 1: C[m, n/2] = silu(gate) * up.  slices > 1 (epilogue 0): parts
+// [slices, m, n] as pa_gemm_mid leaves them, c not written.
+void pa_gemm_tall_shape(int m, int n, int k, int slices, int* out);
+int pa_gemm_tall(void* stream, int epilogue, const void* x, const void* w, const float* bias, void* c, float* parts,
+                 int m, int n, int k, long ldx, long ldc, int slices, int mt, int nt);
 // out[i] = parts[0, i] + parts[1, i] + ..; out_dtype 0 = float32, 1 = bfloat16; total = rows * columns.
 int pa_sum_slices(void* stream, int out_dtype, const float* parts, void* out, int slices, long total);
 // out[tile][step][half][g][r][8] = w[16 tile + r][64 step + 16 g + 8 half ..], zero-padded: ceil(n/16) * ceil(k/64) * 1024 elements.

@@ -431,6 +431,73 @@ def gemm_mid(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = N
     return out
 
 
+def gemm_tall(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = None, silu_mul_epilogue: bool = False,
+              slices: int = 1, shape=(0, 0)):
+    """x [M, K] @ w[N, K]^T for any number of rows from the weight in tiles, the output tiled both ways: a
+    workgroup owns ``16 * shape[0]`` rows of X and ``64 * shape[1]`` rows of W ((0, 0): the launcher chooses by the
+    product's size; the same bits at every shape).  bfloat16 out; with ``slices`` > 1 a ``SliceSums``."""
+    if not isinstance(w, TiledWeight):
+        raise NativeError("gemm_tall takes the weight in tiles (pack_tiles)")
+    _dev(x, w.data, bias)
+    _f32(bias, "bias")
+    if x.dim() != 2 or x.shape[1] != w.k or x.dtype != torch.bfloat16:
+        raise NativeError(f"gemm_tall: x {tuple(x.shape)} {x.dtype} / w {w.shape}")
+    m, k = x.shape
+    n = w.n
+    if bias is not None and bias.shape != (n,):
+        raise NativeError(f"gemm_tall: bias {tuple(bias.shape)} is not [{n}]")
+    if slices > 1:
+        parts = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+        check(kernels().pa_gemm_tall(_stream(), 0, _ptr(x), _ptr(w.data), _ptr(bias), None, _ptr(parts), m, n, k, k, n,
+                                     slices, int(shape[0]), int(shape[1])))
+        return SliceSums(parts, torch.bfloat16)
+    cols = n // 2 if silu_mul_epilogue else n
+    out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
+    check(kernels().pa_gemm_tall(_stream(), 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out),
+                                 None, m, n, k, k, cols, 1, int(shape[0]), int(shape[1])))
+    return out
+
+
+# Where ``linear`` takes the product tiled both ways (``gemm_tall``) beyond the 128 rows of ``gemm_mid``, measured
+# against the library at the shapes of 4B, 8B and 32B models, weights from memory:
+#  - cut into four slices for a reader that adds them, up to 320 rows everywhere ([2560, 4096] at 256 rows 18.6
+#    against 21.9 us, [2560, 9728] 35.1 against 41.7, [4096, 12288] 46.5 against 54.8, [5120, 25600] 108 against 261)
+#    and up to 576 rows for long rows or large weights ([2560, 9728] at 512 rows 46.8 against 52.6, [4096, 12288]
+#    67.9 against 82.9, [5120, 25600] 163 against 271; [2560, 4096] and [4096, 4096] there are the library's, 24
+#    against 26 and 29 against 30);
+#  - for a reader that wants a tensor, in slices and a kernel that adds them (some 3 us), up to 320 rows ([6144, 2560]
+#    at 256 rows 21.8 + 3 against 31.3, [6144, 4096] 27.9 + 3 against 40.0, [10240, 5120] 49.5 + 3 against 61.3);
+#  - the gated product with its activation in the epilogue for rows shorter than 4,096 columns up to 320 rows
+#    ([19456, 2560]: 37.1 against 43.0 us with the separate kernel at 129 rows, 46.9 against 51.7 at 256; at 512 rows
+#    67.4 against 63.9, and [24576, 4096] 71.9 against 68.2 at 256 rows: the library's).
+TALL_MAX_ROWS = 320
+TALL_LONG_MAX_ROWS = 576       # ... for rows of TALL_LONG_K columns or more, or weights of TALL_LARGE_ELEMENTS
+TALL_LONG_K = 8192
+TALL_LARGE_ELEMENTS = 40 << 20
+TALL_GATED_MAX_K = 4096
+TALL_PRODUCTS = True           # ``set_tall_products``: off sends these products to the library (measurements)
+
+
+def set_tall_products(on: bool) -> None:
+    global TALL_PRODUCTS
+    TALL_PRODUCTS = bool(on)
+
+
+def _tall_slices(k: int) -> int:
+    """Slices of the inner size for ``gemm_tall``: four where every slice still has eight steps of 64 columns."""
+    steps = (k + 63) // 64
+    for s in (4, 2):
+        if steps >= 8 * s and -(-steps // -(-steps // s)) == s:
+            return s
+    return 1
+
+
+def _tall_sliced(m: int, n: int, k: int) -> bool:
+    if not TALL_PRODUCTS or m <= GEMM_MID_MAX_ROWS or k % 8 or n % 4:
+        return False
+    return m <= TALL_MAX_ROWS or (m <= TALL_LONG_MAX_ROWS and (k >= TALL_LONG_K or n * k >= TALL_LARGE_ELEMENTS))
+
+
 LIBRARY_WORKSPACE_BYTES = 76 << 20   # what the library's stream-K kernels may use for partial sums
 _library_workspaces: dict = {}
 
@@ -502,6 +569,12 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
             return gemm_mid(x, tiles, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
+    if tiles is not None and out_dtype in (None, torch.bfloat16) and _tall_sliced(m, n, k):
+        s = _tall_slices(k)
+        if s > 1 and slices_ok:
+            return gemm_tall(x, tiles, bias, slices=s)
+        if s > 1 and m <= TALL_MAX_ROWS:
+            return gemm_tall(x, tiles, bias, slices=s).materialize()
     if k % 8:
         # rows that are no multiple of 16 bytes: neither the streaming kernel's loads nor the library's fast
         # kernels take them; the plain product does (bfloat16 in, 32-bit sums), and only odd toy sizes come here
@@ -562,6 +635,9 @@ def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
             return gemm_mid(x, tiles, silu_mul_epilogue=True)
         if tiles is not None and _gated_tiled(m, tiles.n, k):
             return gemm_skinny(x, tiles, silu_mul_epilogue=True)
+        if (TALL_PRODUCTS and tiles is not None and GEMM_MID_MAX_ROWS < m <= TALL_MAX_ROWS and k < TALL_GATED_MAX_K
+                and tiles.n % 2 == 0):
+            return gemm_tall(x, tiles, silu_mul_epilogue=True)
     return silu_mul(linear(x, w))
 
 

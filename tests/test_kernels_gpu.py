@@ -230,6 +230,97 @@ def test_gemm_mid(gpu, m, n, k, slices):
             assert torch.equal(K().gemm_mid(xd, tiles, bd, slices=slices, waves=waves).parts, ss.parts), f"{waves} wavefronts, slices"
 
 
+@pytest.mark.parametrize("m,n,k,slices", [(129, 2560, 4096, 4), (300, 331, 1000, 1), (256, 200, 4096, 2), (513, 2560, 2560, 1),
+                                          (192, 6144, 2560, 4), (1030, 72, 640, 1), (260, 1000, 2560, 1), (140, 36, 72, 1),
+                                          (576, 2560, 9728, 4), (2, 64, 64, 1)])
+def test_gemm_tall(gpu, m, n, k, slices):
+    """The product tiled both ways (any number of rows, weight in tiles): whole, with bias, with the gated
+    activation in its epilogue, and cut into slices whose 32-bit partial sums the reader adds; at every shape of
+    workgroup the same bits, and a row's result whatever the other rows are."""
+    x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
+    ref = x.double() @ w.double().T
+    xd, bd = x.to(gpu), b.to(gpu)
+    tiles = K().pack_tiles(w.to(gpu))
+    full = K().gemm_tall(xd, tiles)
+    close(full, ref, torch.bfloat16)
+    close(K().gemm_tall(xd, tiles, bd), ref + b.double(), torch.bfloat16)
+    # a row's result does not depend on how many rows there are, nor on which row of a tile it is
+    lone = K().gemm_tall(xd[m - 1:].contiguous(), tiles)
+    assert torch.equal(lone[0], full[m - 1])
+    if m > 70:
+        part = K().gemm_tall(xd[37: 37 + 33].contiguous(), tiles)
+        assert torch.equal(part, full[37: 37 + 33])
+    gated = None
+    if n % 2 == 0:
+        gated = K().gemm_tall(xd, tiles, silu_mul_epilogue=True)
+        close(gated, pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16)
+    ss = None
+    if slices > 1:
+        ss = K().gemm_tall(xd, tiles, bd, slices=slices)
+        assert isinstance(ss, K().SliceSums) and tuple(ss.parts.shape) == (slices, m, n) and ss.dtype == torch.bfloat16
+        whole = ss.parts.double().sum(0).cpu()
+        close(whole, ref + b.double(), torch.float32, f32=2e-5)
+        close(ss.materialize(), ref + b.double(), torch.bfloat16)
+        weight, res = 1 + 0.1 * rnd(n, seed=3), rnd(m, n, dtype=torch.bfloat16, seed=4)
+        resd = res.to(gpu)
+        normed = K().rmsnorm(ss, weight.to(gpu), 1e-5, residual=resd)
+        total = whole + res.double()
+        close(resd, total, torch.bfloat16)
+        close(normed, pm.rms_norm(total, weight.double(), 1e-5), torch.bfloat16)
+    # what lies behind X is not the product's to read: NaN there must not show
+    behind = torch.full((m + 8, k), float("nan"), dtype=torch.bfloat16, device=gpu)
+    behind[:m] = xd
+    got = K().gemm_tall(behind[:m], tiles)
+    assert bool(torch.isfinite(got.float()).all()) and torch.equal(got, full)
+    # the workgroup's shape (which the launcher picks by the product's size) changes no bit
+    for shape in ((4, 2), (4, 3), (8, 2), (8, 3)):
+        assert torch.equal(K().gemm_tall(xd, tiles, shape=shape), full), shape
+        if gated is not None:
+            assert torch.equal(K().gemm_tall(xd, tiles, silu_mul_epilogue=True, shape=shape), gated), shape
+        if ss is not None:
+            assert torch.equal(K().gemm_tall(xd, tiles, bd, slices=slices, shape=shape).parts, ss.parts), shape
+
+
+def test_gemm_tall_refuses_and_is_dispatched(gpu):
+    from prelude_amd._native import NativeError
+    w = rnd(2560, 4096, dtype=torch.bfloat16, seed=1, scale=0.05).to(gpu)
+    tiles = K().pack_tiles(w)
+    x = rnd(256, 4096, dtype=torch.bfloat16).to(gpu)
+    with pytest.raises(NativeError, match="in tiles"):
+        K().gemm_tall(x, w)
+    with pytest.raises(NativeError, match="do not cut into"):
+        K().gemm_tall(x, tiles, slices=60)
+    with pytest.raises(NativeError, match="no kernel of"):
+        K().gemm_tall(x, tiles, shape=(5, 2))
+    with pytest.raises(NativeError, match="no bias"):
+        K().gemm_tall(x, tiles, torch.zeros(2560, device=gpu), silu_mul_epilogue=True)
+    ref = x.double().cpu() @ w.double().cpu().T
+    lw = K().LinearWeight(w, tiles)
+    # a reader that adds slices gets them beyond 128 rows too; one that wants a tensor gets the slices added
+    got = K().linear(x, lw, slices_ok=True)
+    assert isinstance(got, K().SliceSums) and got.parts.shape[0] == 4
+    close(K().as_tensor(got), ref, torch.bfloat16)
+    plain = K().linear(x, lw)
+    assert isinstance(plain, torch.Tensor) and torch.equal(plain, got.materialize())
+    # beyond the rows it is ahead for, the library's product
+    tall = rnd(700, 4096, dtype=torch.bfloat16, seed=5).to(gpu)
+    assert isinstance(K().linear(tall, lw, slices_ok=True), torch.Tensor)
+    # the gated product of short rows: the activation in the epilogue, the same bits as asked for directly
+    wg = rnd(1024, 2560, dtype=torch.bfloat16, seed=6, scale=0.05).to(gpu)
+    lg = K().LinearWeight(wg, K().pack_tiles(wg))
+    xg = rnd(200, 2560, dtype=torch.bfloat16, seed=7).to(gpu)
+    assert torch.equal(K().linear_silu_mul(xg, lg), K().gemm_tall(xg, lg.tiles, silu_mul_epilogue=True))
+    K().set_tall_products(False)
+    try:
+        off = K().linear_silu_mul(xg, lg)
+        assert isinstance(K().linear(x, lw, slices_ok=True), torch.Tensor)
+    finally:
+        K().set_tall_products(True)
+    g = xg.double().cpu() @ wg.double().cpu().T
+    close(off, pm.silu(g[:, 0::2]) * g[:, 1::2], torch.bfloat16)
+    close(K().linear_silu_mul(xg, lg), pm.silu(g[:, 0::2]) * g[:, 1::2], torch.bfloat16)
+
+
 def test_gemm_mid_refuses_and_is_dispatched(gpu):
     from prelude_amd._native import NativeError
     w = rnd(2560, 4096, dtype=torch.bfloat16, seed=1, scale=0.05).to(gpu)
@@ -651,10 +742,12 @@ def test_mfma_attention_first_keys_far_below_zero(gpu, hd, page, window):
     close(out, ref, torch.bfloat16)
     out, ref = paged_case(gpu, torch.float32, 4, 2, hd, page, seqs, window, seed=8, scale_trick=trick)
     assert not bool(torch.isnan(out).any())
-    # a cold key's dot product holds one term of 12 x 69 sqrt(hd / 64) = 832 ..: summed in 32-bit it is off by up to
-    # some 2e-4, 2.5e-5 in the exponent, and a query that sees cold keys only weighs them against each other with
-    # that relative error.  The bound follows the inputs' size; a lost or misread key moves the output by O(1).
-    close(out, ref, torch.float32, f32=2e-5)
+    # A cold key's dot product starts with one term of 104 sqrt(hd); each of the hd additions behind it rounds at
+    # that size (half a unit in the last place: 104 sqrt(hd) 2^-24), which adds up to some sqrt(hd) times that,
+    # times the scale 1 / sqrt(hd), in the exponent: a query that sees cold keys only weighs them against each
+    # other with a relative error of 104 sqrt(hd) 2^-24 (7e-5 at head_dim 128).  The bound follows the inputs' size;
+    # a lost or misread key moves the output by O(1).
+    close(out, ref, torch.float32, f32=104.0 * math.sqrt(hd) * 2.0 ** -24)
 
 
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0),
