@@ -12,9 +12,15 @@ model from the paged cache, greedy argmax on the device, ids back to the host;
 the host prepares a step while the one before it runs, as the engine's
 generation loop does).
 One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is
-a 2,048-token prompt portion; ``roofline`` prices the decode step against HBM
-bandwidth; ``points`` holds batch 1, 32 and 64 at the same context, batch 8 at a context of 32,768 tokens and the
-prefill of 8,192 tokens in one step (tokens a second each).
+a 2,048-token prompt portion (the median of its repetitions); ``roofline`` prices
+the decode step against HBM bandwidth; ``points`` holds, in tokens a second each:
+batch 1, 32 and 64 at the same context; batch 64 again on a pool whose pages were
+handed out, given back and handed out again in a random order of requests
+(``decode_b64_churned``); batch 8 at a context of 32,768 tokens; prompts of 256,
+512 and 8,192 tokens in one step; and at the other shapes the benchmark
+configurations name: batch 8 and a 2,048-token prompt at the 8B shape, a step of
+a 2,048-token portion beside 63 decoding requests at contexts up to 8,192 there
+(``8b_mixed_2048+63``), and batch 8 at the 32B shape.
 """
 from __future__ import annotations
 
@@ -85,7 +91,7 @@ def prefill_requests(engine, batch, length, chunk, vocab, seed):
     return prompts
 
 
-def time_decode(engine, batch, steps, warmup, vocab):
+def time_decode(engine, batch, steps, warmup, vocab, ids=None):
     """Greedy decode steps for `batch` live requests; returns seconds per step.
 
     As in ``LLM.generate``, a step is launched with the previous step's ids
@@ -95,13 +101,14 @@ def time_decode(engine, batch, steps, warmup, vocab):
     from prelude_amd.engine import StepEntry
     from prelude_amd.ops import kernels as K
     state = {"sampled": None, "pending": None, "ids": [1] * batch}
+    rids = list(range(batch)) if ids is None else list(ids)
 
     def one():
         prev = state["sampled"]
         if prev is None:
-            entries = [StepEntry(r, [state["ids"][r]], [0]) for r in range(batch)]
+            entries = [StepEntry(rids[r], [state["ids"][r]], [0]) for r in range(batch)]
         else:
-            entries = [StepEntry(r, [0], [0], carry=r) for r in range(batch)]
+            entries = [StepEntry(rids[r], [0], [0], carry=r) for r in range(batch)]
         logits = engine.step(entries, carried=prev)
         sampled = K.argmax(logits)
         host = torch.empty(batch, dtype=torch.int32, pin_memory=True)
@@ -124,10 +131,56 @@ def time_decode(engine, batch, steps, warmup, vocab):
     return (time.perf_counter() - t0) / steps
 
 
-def decode_point(raw, dtype, batch, context, steps, warmup, layers_note, chunk=2048):
+def churned_requests(engine, batch, length, vocab, seed):
+    """`batch` live requests of `length` tokens on a pool that has been through a session: requests of random
+    lengths are admitted in turn, a random half of them ends, others take their pages, and every request grows in
+    portions of random size in a random order of requests, so that no request's pages lie in one run."""
+    import numpy as np
+    from prelude_amd.engine import StepEntry
+    rng = np.random.default_rng(seed)
+    have = {}
+    next_id = 0
+
+    def grow(rid, upto):
+        while have[rid] < upto:
+            n = int(min(upto - have[rid], rng.integers(48, 400)))
+            engine.step([StepEntry(rid, rng.integers(0, vocab, size=n).tolist(), [])])
+            have[rid] += n
+            yield
+
+    for _ in range(3):                                   # three generations of requests
+        while len(have) < batch:
+            have[next_id] = 0
+            next_id += 1
+        growers = [grow(rid, int(rng.integers(length // 4, length))) for rid in have]
+        while growers:                                   # all of them grow, a portion at a time, in random order
+            i = int(rng.integers(0, len(growers)))
+            if next(growers[i], "done") == "done":
+                growers.pop(i)
+        for rid in rng.permutation(list(have))[: batch // 2].tolist():
+            engine.release(rid)
+            del have[rid]
+    while len(have) < batch:
+        have[next_id] = 0
+        next_id += 1
+    growers = [grow(rid, length) for rid in have]
+    while growers:
+        i = int(rng.integers(0, len(growers)))
+        if next(growers[i], "done") == "done":
+            growers.pop(i)
+    return sorted(have)
+
+
+def decode_point(raw, dtype, batch, context, steps, warmup, layers_note, chunk=2048, churned=False):
     import torch
     total = steps + warmup
     eng = build_engine(raw, dtype, cache_tokens=batch * (context + 64), max_num_batched_tokens=max(8192, chunk))
+    if churned:
+        ids = churned_requests(eng, batch, context - total, raw["vocab_size"], seed=batch)
+        sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"], ids)
+        del eng
+        release_memory()
+        return sec
     prefill_requests(eng, batch, context - total, chunk, raw["vocab_size"], seed=batch)
     sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"])
     del eng
@@ -136,12 +189,13 @@ def decode_point(raw, dtype, batch, context, steps, warmup, layers_note, chunk=2
 
 
 def time_prefill(raw, dtype, tokens, reps):
+    """Seconds a prompt of `tokens` tokens takes in one step, its last logits wanted: the median of `reps` runs."""
     import numpy as np
     import torch
     from prelude_amd.engine import StepEntry
     eng = build_engine(raw, dtype, cache_tokens=(reps + 2) * (tokens + 64), max_num_batched_tokens=max(8192, tokens))
     rng = np.random.default_rng(7)
-    best = None
+    times = []
     for r in range(reps + 1):
         p = rng.integers(0, raw["vocab_size"], size=tokens).tolist()
         torch.cuda.synchronize()
@@ -151,10 +205,10 @@ def time_prefill(raw, dtype, tokens, reps):
         dt = time.perf_counter() - t0
         eng.release(100 + r)
         if r > 0:
-            best = dt if best is None else min(best, dt)
+            times.append(dt)
     del eng
     release_memory()
-    return best
+    return sorted(times)[len(times) // 2]           # the median (the first run, which sets things up, left out)
 
 
 def time_mixed(raw, dtype, chunk, decoding, context, steps, warmup):
@@ -289,7 +343,7 @@ def main() -> int:
               flush=True)
         return 0
     if args.prefill_only:
-        psec = time_prefill(raw, args.dtype, args.prefill_tokens, reps=3)
+        psec = time_prefill(raw, args.dtype, args.prefill_tokens, reps=5)
         print(json.dumps({"prefill_tokens": args.prefill_tokens, "ms": round(psec * 1e3, 3),
                           "tok_per_s": round(args.prefill_tokens / psec, 1)}), flush=True)
         return 0
@@ -314,7 +368,7 @@ def main() -> int:
     }
     if not args.no_prefill:
         T = args.prefill_tokens
-        psec = time_prefill(raw, args.dtype, T, reps=3)
+        psec = time_prefill(raw, args.dtype, T, reps=5)
         nh, hd, L = raw["num_attention_heads"], raw["head_dim"], raw["num_hidden_layers"]
         flops = 2.0 * T * matmul_params + L * 2.0 * nh * hd * T * T + 2.0 * raw["vocab_size"] * raw["hidden_size"]
         out["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
@@ -328,8 +382,25 @@ def main() -> int:
             # further from the default point: a long context (the cache is 3.6 times the weights there) and a long portion
             s = decode_point(raw, args.dtype, 8, 32768, max(8, args.steps // 4), max(2, args.warmup // 4), None, chunk=8192)
             pts["decode_b8_ctx32768"] = round(8 / s, 2)
+            s = decode_point(raw, args.dtype, 64, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), None,
+                             churned=True)
+            pts["decode_b64_churned"] = round(64 / s, 2)
             if not args.no_prefill:
-                pts["prefill_8192"] = round(8192 / time_prefill(raw, args.dtype, 8192, reps=2), 1)
+                pts["prefill_8192"] = round(8192 / time_prefill(raw, args.dtype, 8192, reps=3), 1)
+                for t in (256, 512):
+                    pts[f"prefill_{t}"] = round(t / time_prefill(raw, args.dtype, t, reps=5), 1)
+            if args.shape == "4b" and not args.layers:
+                # the other shapes the benchmark configurations name, at their own points
+                big = dict(SHAPES["8b"])
+                s = decode_point(big, args.dtype, 8, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), None)
+                pts["8b_decode_b8"] = round(8 / s, 2)
+                if not args.no_prefill:
+                    pts["8b_prefill_2048"] = round(2048 / time_prefill(big, args.dtype, 2048, reps=3), 1)
+                s = time_mixed(big, args.dtype, 2048, 63, 8192, 4, 2)
+                pts["8b_mixed_2048+63"] = round((2048 + 63) / s, 1)
+                big = dict(SHAPES["32b"])
+                s = decode_point(big, args.dtype, 8, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), None)
+                pts["32b_decode_b8"] = round(8 / s, 2)
         out["points"] = pts
     print(json.dumps(out), flush=True)
     return 0

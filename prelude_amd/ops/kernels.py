@@ -458,29 +458,33 @@ def gemm_tall(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = 
     return out
 
 
-# Where ``linear`` takes the product tiled both ways (``gemm_tall``) beyond the 128 rows of ``gemm_mid``, measured
-# against the library at the shapes of 4B, 8B and 32B models, weights from memory:
-#  - cut into four slices for a reader that adds them, up to 320 rows everywhere ([2560, 4096] at 256 rows 18.6
-#    against 21.9 us, [2560, 9728] 35.1 against 41.7, [4096, 12288] 46.5 against 54.8, [5120, 25600] 108 against 261)
-#    and up to 576 rows for long rows or large weights ([2560, 9728] at 512 rows 46.8 against 52.6, [4096, 12288]
-#    67.9 against 82.9, [5120, 25600] 163 against 271; [2560, 4096] and [4096, 4096] there are the library's, 24
-#    against 26 and 29 against 30);
-#  - for a reader that wants a tensor, in slices and a kernel that adds them (some 3 us), up to 320 rows ([6144, 2560]
-#    at 256 rows 21.8 + 3 against 31.3, [6144, 4096] 27.9 + 3 against 40.0, [10240, 5120] 49.5 + 3 against 61.3);
-#  - the gated product with its activation in the epilogue for rows shorter than 4,096 columns up to 320 rows
-#    ([19456, 2560]: 37.1 against 43.0 us with the separate kernel at 129 rows, 46.9 against 51.7 at 256; at 512 rows
-#    67.4 against 63.9, and [24576, 4096] 71.9 against 68.2 at 256 rows: the library's).
-TALL_MAX_ROWS = 320
-TALL_LONG_MAX_ROWS = 576       # ... for rows of TALL_LONG_K columns or more, or weights of TALL_LARGE_ELEMENTS
-TALL_LONG_K = 8192
-TALL_LARGE_ELEMENTS = 40 << 20
+# Where ``linear`` takes the product tiled both ways (``gemm_tall``) beyond the 128 rows of ``gemm_mid``.  Alone, with
+# the weights coming from memory, it is ahead of the library for most products of 129 to 320 rows at the shapes of 4B, 8B
+# and 32B models ([2560, 9728] at 256 rows in four slices 35.1 against 41.7 us, [4096, 12288] 46.5 against 54.8,
+# [5120, 25600] 108 against 261; the gated [19456, 2560] 46.9 against 51.7 with the separate activation kernel); what
+# decides is the prompt step it runs in, where the reader of slices pays for them (the norm reads four 32-bit partial
+# sums instead of one bfloat16 tensor) -- a whole prompt through 36 layers, same box, library against this kernel:
+#  - in four slices for the norm that follows, wide outputs only: hidden 4,096 at 129 / 160 / 192 / 256 rows 7.29 /
+#    8.00 / 9.27 / 8.21 against 6.96 / 6.85 / 7.42 / 8.02 ms, level at 320 rows and behind from 384 on; hidden 2,560
+#    5.01 / 5.20 / 5.43 / 6.56 against 5.34 / 5.49 / 5.78 / 6.39: the library's.  The very large weights of a 32B
+#    model (a [5120, 25600] product alone: 163 against 271 us at 512 rows) up to 576 rows;
+#  - the gated product with its activation in the epilogue, rows shorter than 4,096 columns: hidden 2,560 at 129 / 192 /
+#    256 rows 5.01 / 5.43 / 6.56 against 4.76 / 5.23 / 6.34 ms, behind from 288 rows on (6.16 against 6.43);
+#    [24576, 4096] is the library's at every number of rows (256 rows: 68.2 against 71.9 us);
+#  - slices added by a kernel of their own for a reader of tensors (the QKV projection) lost everywhere (hidden
+#    2,560 at 256 rows: 6.56 against 8.01 ms) and are not dispatched.
+TALL_MAX_ROWS = 256
+TALL_SLICED_MIN_N = 4096       # outputs at least this wide go to it in slices for the norm ...
+TALL_HUGE_MAX_ROWS = 576       # ... and weights of TALL_HUGE_ELEMENTS up to this many rows
+TALL_HUGE_ELEMENTS = 100 << 20
 TALL_GATED_MAX_K = 4096
-TALL_PRODUCTS = True           # ``set_tall_products``: off sends these products to the library (measurements)
+TALL_PRODUCTS = 3              # ``set_tall_products``: which of these products ``gemm_tall`` takes (measurements):
+#                                1 in slices for a reader of slices, 2 the gated one
 
 
-def set_tall_products(on: bool) -> None:
+def set_tall_products(on) -> None:
     global TALL_PRODUCTS
-    TALL_PRODUCTS = bool(on)
+    TALL_PRODUCTS = 3 if on is True else int(on)
 
 
 def _tall_slices(k: int) -> int:
@@ -493,9 +497,9 @@ def _tall_slices(k: int) -> int:
 
 
 def _tall_sliced(m: int, n: int, k: int) -> bool:
-    if not TALL_PRODUCTS or m <= GEMM_MID_MAX_ROWS or k % 8 or n % 4:
+    if not TALL_PRODUCTS & 1 or m <= GEMM_MID_MAX_ROWS or k % 8 or n % 4 or n < TALL_SLICED_MIN_N:
         return False
-    return m <= TALL_MAX_ROWS or (m <= TALL_LONG_MAX_ROWS and (k >= TALL_LONG_K or n * k >= TALL_LARGE_ELEMENTS))
+    return m <= TALL_MAX_ROWS or (m <= TALL_HUGE_MAX_ROWS and n * k >= TALL_HUGE_ELEMENTS)
 
 
 LIBRARY_WORKSPACE_BYTES = 76 << 20   # what the library's stream-K kernels may use for partial sums
@@ -527,10 +531,11 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, slices_ok: bool = False):
     """y = x W^T (+ b), W [out, in] as a tensor or a ``LinearWeight``.  float32: our own true 32-bit product.
     bfloat16: few rows our weight-streaming kernel (from the tiled copy if the weight has one), above that the
-    library product or, for the shapes it suits, the product with X staged in LDS; 32-bit accumulation in all.
+    library product or, for the shapes they suit, the products with X staged in LDS (``gemm_mid`` to 128 rows,
+    ``gemm_tall`` beyond); 32-bit accumulation in all.
 
     ``slices_ok``: the caller's reader adds slices itself (``rmsnorm`` does): a narrow weight at 17 to 128 rows
-    then comes back as ``SliceSums`` (the product cut along its inner size, a 32-bit partial sum per slice)
+    (a wide one beyond, see ``TALL_MAX_ROWS``) then comes back as ``SliceSums`` (the product cut along its inner size, a 32-bit partial sum per slice)
     instead of a tensor."""
     tiles = None
     if isinstance(w, LinearWeight):
@@ -569,12 +574,10 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
             return gemm_mid(x, tiles, bias, out_dtype)
     if tiles is not None and _tiled_beyond_16(m, w.shape[0], k):
         return gemm_skinny(x, tiles, bias, out_dtype)
-    if tiles is not None and out_dtype in (None, torch.bfloat16) and _tall_sliced(m, n, k):
+    if tiles is not None and slices_ok and out_dtype in (None, torch.bfloat16) and _tall_sliced(m, n, k):
         s = _tall_slices(k)
-        if s > 1 and slices_ok:
+        if s > 1:
             return gemm_tall(x, tiles, bias, slices=s)
-        if s > 1 and m <= TALL_MAX_ROWS:
-            return gemm_tall(x, tiles, bias, slices=s).materialize()
     if k % 8:
         # rows that are no multiple of 16 bytes: neither the streaming kernel's loads nor the library's fast
         # kernels take them; the plain product does (bfloat16 in, 32-bit sums), and only odd toy sizes come here
@@ -635,7 +638,7 @@ def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
             return gemm_mid(x, tiles, silu_mul_epilogue=True)
         if tiles is not None and _gated_tiled(m, tiles.n, k):
             return gemm_skinny(x, tiles, silu_mul_epilogue=True)
-        if (TALL_PRODUCTS and tiles is not None and GEMM_MID_MAX_ROWS < m <= TALL_MAX_ROWS and k < TALL_GATED_MAX_K
+        if (TALL_PRODUCTS & 2 and tiles is not None and GEMM_MID_MAX_ROWS < m <= TALL_MAX_ROWS and k < TALL_GATED_MAX_K
                 and tiles.n % 2 == 0):
             return gemm_tall(x, tiles, silu_mul_epilogue=True)
     return silu_mul(linear(x, w))

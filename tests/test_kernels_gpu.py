@@ -294,17 +294,17 @@ def test_gemm_tall_refuses_and_is_dispatched(gpu):
         K().gemm_tall(x, tiles, shape=(5, 2))
     with pytest.raises(NativeError, match="no bias"):
         K().gemm_tall(x, tiles, torch.zeros(2560, device=gpu), silu_mul_epilogue=True)
-    ref = x.double().cpu() @ w.double().cpu().T
-    lw = K().LinearWeight(w, tiles)
-    # a reader that adds slices gets them beyond 128 rows too; one that wants a tensor gets the slices added
-    got = K().linear(x, lw, slices_ok=True)
+    # a wide output whose reader adds slices gets them beyond 128 rows too; a narrow one, and a reader that wants a
+    # tensor, the library's product
+    ww = rnd(4096, 4096, dtype=torch.bfloat16, seed=3, scale=0.05).to(gpu)
+    lww = K().LinearWeight(ww, K().pack_tiles(ww))
+    got = K().linear(x, lww, slices_ok=True)
     assert isinstance(got, K().SliceSums) and got.parts.shape[0] == 4
-    close(K().as_tensor(got), ref, torch.bfloat16)
-    plain = K().linear(x, lw)
-    assert isinstance(plain, torch.Tensor) and torch.equal(plain, got.materialize())
-    # beyond the rows it is ahead for, the library's product
+    close(K().as_tensor(got), x.double().cpu() @ ww.double().cpu().T, torch.bfloat16)
+    assert isinstance(K().linear(x, lww), torch.Tensor)
+    assert isinstance(K().linear(x, K().LinearWeight(w, tiles), slices_ok=True), torch.Tensor)
     tall = rnd(700, 4096, dtype=torch.bfloat16, seed=5).to(gpu)
-    assert isinstance(K().linear(tall, lw, slices_ok=True), torch.Tensor)
+    assert isinstance(K().linear(tall, lww, slices_ok=True), torch.Tensor)                  # beyond the rows it is ahead for
     # the gated product of short rows: the activation in the epilogue, the same bits as asked for directly
     wg = rnd(1024, 2560, dtype=torch.bfloat16, seed=6, scale=0.05).to(gpu)
     lg = K().LinearWeight(wg, K().pack_tiles(wg))
@@ -313,7 +313,7 @@ def test_gemm_tall_refuses_and_is_dispatched(gpu):
     K().set_tall_products(False)
     try:
         off = K().linear_silu_mul(xg, lg)
-        assert isinstance(K().linear(x, lw, slices_ok=True), torch.Tensor)
+        assert isinstance(K().linear(x, lww, slices_ok=True), torch.Tensor)
     finally:
         K().set_tall_products(True)
     g = xg.double().cpu() @ wg.double().cpu().T
