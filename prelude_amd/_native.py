@@ -42,7 +42,7 @@ _KERNEL_API = {
     "pa_carry_tokens": (I, [P, P, P, P, P, I, I, I]),
     "pa_zero_fresh_rows": (I, [P, P, c_long, P, P, I, I]),
     "pa_rmsnorm": (I, [P, I, P, P, P, P, P, I, I, F]),
-    "pa_silu_mul": (I, [P, I, P, P, I, I]),
+    "pa_silu_mul": (I, [P, I, P, P, I, I, I]),
     "pa_gather_rows": (I, [P, I, P, P, P, I, I]),
     "pa_add_bias": (I, [P, I, P, P, I, I]),
     "pa_to_f32": (I, [P, I, P, P, c_long]),
@@ -58,14 +58,14 @@ _KERNEL_API = {
     "pa_gemm_tall_shape": (None, [I, I, I, I, IP]),
     "pa_gemm_tall": (I, [P, I, P, P, P, P, P, I, I, I, c_long, c_long, I, I, I]),
     "pa_rmsnorm_slices": (I, [P, I, P, I, c_long, P, P, P, P, I, I, F]),
-    "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
+    "pa_attn_generic": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F]),
     "pa_attn_mfma_supports": (I, [I, I]),
     "pa_attn_decode_workspace": (c_long, [I, I, I, I]),
-    "pa_attn_decode": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I]),
-    "pa_attn_decode_fused": (I, [P, P, P, P, P, P, P, F, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I]),
+    "pa_attn_decode": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I]),
+    "pa_attn_decode_fused": (I, [P, P, P, P, P, P, P, F, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I]),
     "pa_attn_decode_fused_supports": (I, [I, I, I, I, I]),
-    "pa_attn_prefill": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F]),
-    "pa_attn_prefill_cut": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, I]),
+    "pa_attn_prefill": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F]),
+    "pa_attn_prefill_cut": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, I, I, I]),
     "pa_argmax_scratch": (I, [I, I]),
     "pa_argmax": (I, [P, P, P, P, I, I]),
     "pa_argmax_static_capacity": (I, []),

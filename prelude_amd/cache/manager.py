@@ -8,14 +8,11 @@ them.  Beside the pages there is a pool of slots for per-request state of
 fixed size (crates/prelude-core/src/scheduler/components/cache/deltanet_pool.rs:54-173),
 one slot per live request when the model has a mixer that keeps such state.
 
-Layout of a group's pages on the device, per cache slot: K
-``[pages, kv_heads, page_size, head_dim]`` and V transposed
-``[pages, kv_heads, head_dim, page_size]`` -- one (page, head) tile is
-contiguous, so a wavefront streaming a head's keys reads whole lines, and
-both tiles can be loaded straight into matrix-core operands: the contraction
-index (head_dim for Q.K, keys for P.V) is the contiguous one in each
-(the reference keeps ``[pages, page_size, kv_heads, head_dim]`` for both,
-crates/prelude-core/src/scheduler/components/cache/manager.rs:286-329).
+What lies in a page is the mixer's business: every cache specification
+allocates its own storage (``parts.base.PagedCacheSpec.allocate``; keys and
+values: K ``[pages, kv_heads, page_size, head_dim]`` and V transposed, see
+``KVCacheSpec``), the manager only counts bytes, hands out pages and builds
+the tables.
 """
 from __future__ import annotations
 
@@ -27,7 +24,7 @@ import numpy as np
 import torch
 
 from .._native import host
-from ..parts.base import KVCacheSpec, StateSpec
+from ..parts.base import KVLayerCache, PagedCacheSpec, StateLayerCache   # noqa: F401  (the views are re-exported here)
 
 
 class CacheError(RuntimeError):
@@ -181,44 +178,17 @@ class PageTables:
             raise CacheError(self._err())
 
 
-@dataclasses.dataclass
-class KVLayerCache:
-    """What an attention-like mixer gets: its pages and the group whose tables index them."""
-    k: torch.Tensor   # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor   # [pages, kv_heads, value width (head_dim unless the spec says otherwise), page_size]
-    group: int
+def _paged(cs) -> bool:
+    return bool(getattr(cs, "PAGED", False))
 
 
-@dataclasses.dataclass
-class StateLayerCache:
-    """What a mixer with state of fixed size gets: per name a tensor [slots, *shape]."""
-    tensors: Dict[str, torch.Tensor]
-
-    def snapshot(self, state_slots: torch.Tensor) -> Dict[str, torch.Tensor]:
-        """Copies of the slots' rows (``state_slots`` int32 on the device, all >= 0)."""
-        idx = state_slots.to(torch.int64)
-        return {name: t.index_select(0, idx) for name, t in self.tensors.items()}
-
-    def restore(self, state_slots: torch.Tensor, saved: Dict[str, torch.Tensor]) -> None:
-        idx = state_slots.to(torch.int64)
-        for name, t in self.tensors.items():
-            t.index_copy_(0, idx, saved[name])
-
-    def zero_fresh(self, state_slots: torch.Tensor, fresh: torch.Tensor) -> None:
-        """Clears the slots of the step's sequences that start their request; both index arrays are the
-        step's own on the device, so a captured step can carry this."""
-        from ..ops import kernels as K
-        for t in self.tensors.values():
-            K.zero_fresh_rows(t, state_slots, fresh)
-
-
-def plan_groups(cache_specs: Sequence[object]) -> Tuple[List[KVCacheSpec], List[Optional[int]]]:
-    """Groups the model's cache slots: identical key/value specs share a group.
-    Returns the groups' specs and, per cache slot, its group (None for state slots)."""
-    groups: List[KVCacheSpec] = []
+def plan_groups(cache_specs: Sequence[object]) -> Tuple[List[PagedCacheSpec], List[Optional[int]]]:
+    """Groups the model's cache slots: paged specs that compare equal share a group (``PagedCacheSpec``).
+    Returns the groups' specs and, per cache slot, its group (None for slots of per-request state)."""
+    groups: List[PagedCacheSpec] = []
     of_slot: List[Optional[int]] = []
     for cs in cache_specs:
-        if isinstance(cs, KVCacheSpec):
+        if _paged(cs):
             if cs not in groups:
                 groups.append(cs)
             of_slot.append(groups.index(cs))
@@ -229,20 +199,12 @@ def plan_groups(cache_specs: Sequence[object]) -> Tuple[List[KVCacheSpec], List[
 
 def bytes_per_token(cache_specs: Sequence[object], dtype: torch.dtype) -> int:
     el = torch.empty((), dtype=dtype).element_size()
-    return sum(cs.num_kv_heads * (cs.head_dim + cs.v_dim) * el for cs in cache_specs if isinstance(cs, KVCacheSpec))
+    return sum(int(cs.bytes_per_token(el)) for cs in cache_specs if _paged(cs))
 
 
 def state_bytes_per_slot(cache_specs: Sequence[object]) -> int:
     """Bytes one request's state of fixed size takes, over all cache slots that keep such state."""
-    total = 0
-    for cs in cache_specs:
-        if isinstance(cs, StateSpec):
-            for _name, shape, dt in cs.tensors:
-                n = 1
-                for d in shape:
-                    n *= int(d)
-                total += n * torch.empty((), dtype=dt).element_size()
-    return total
+    return sum(int(cs.bytes_per_slot()) for cs in cache_specs if not _paged(cs))
 
 
 def peak_pages(total: int, chunk: int, window: int, page_size: int) -> int:
@@ -254,7 +216,7 @@ def peak_pages(total: int, chunk: int, window: int, page_size: int) -> int:
     return min(pages(total), pages(max(1, chunk) + window - 1) + 1)
 
 
-def pages_per_group(tokens: int, group_specs: Sequence[KVCacheSpec], page_size: int, max_requests: int,
+def pages_per_group(tokens: int, group_specs: Sequence[PagedCacheSpec], page_size: int, max_requests: int,
                     max_request_tokens: int, chunk: int) -> List[int]:
     """Pages each group needs so that live requests can hold ``tokens`` tokens between them: a group that
     sees every key holds them all; one with a window holds per request what the window and a portion span,
@@ -271,16 +233,14 @@ def pages_per_group(tokens: int, group_specs: Sequence[KVCacheSpec], page_size: 
 
 def allocate_storage(cache_specs: Sequence[object], of_slot: Sequence[Optional[int]], pages_per_group: Sequence[int],
                      page_size: int, state_slots: int, dtype: torch.dtype, device: torch.device) -> List[object]:
-    """Device tensors for every cache slot, zero-initialised."""
+    """Device storage for every cache slot, zero-initialised: each specification allocates its own kind
+    (``PagedCacheSpec.allocate`` / ``SlotCacheSpec.allocate``)."""
     out: List[object] = []
     for cs, g in zip(cache_specs, of_slot):
-        if isinstance(cs, KVCacheSpec):
-            n = pages_per_group[g]
-            out.append(KVLayerCache(torch.zeros((n, cs.num_kv_heads, page_size, cs.head_dim), dtype=dtype, device=device),
-                                    torch.zeros((n, cs.num_kv_heads, cs.v_dim, page_size), dtype=dtype, device=device), g))
-        elif isinstance(cs, StateSpec):
-            out.append(StateLayerCache({name: torch.zeros((state_slots, *shape), dtype=dt, device=device)
-                                        for name, shape, dt in cs.tensors}))
+        if not callable(getattr(cs, "allocate", None)):
+            raise CacheError(f"unknown cache specification {cs!r}: it has no allocate()")
+        if _paged(cs):
+            out.append(cs.allocate(pages_per_group[g], page_size, dtype, device, g))
         else:
-            raise CacheError(f"unknown cache specification {cs!r}")
+            out.append(cs.allocate(state_slots, device))
     return out

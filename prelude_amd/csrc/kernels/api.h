@@ -32,8 +32,9 @@ int pa_rmsnorm(void* stream, int dtype, const void* x, void* residual, const flo
 // pa_gemm_mid leaves of a product cut along its inner size): they are added in order as they are loaded.
 int pa_rmsnorm_slices(void* stream, int dtype, const float* parts, int slices, long slice_stride, void* residual,
                       const float* w, void* out, const int* rows, int nrows, int hidden, float eps);
-// out[t, c] = silu(gate_up[t, 2c]) * gate_up[t, 2c + 1]   (columns alternate gate_j, up_j)
-int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter);
+// out[t, c] = act(gate_up[t, 2c]) * gate_up[t, 2c + 1]   (columns alternate gate_j, up_j); act: 0 SiLU, 1 GELU in its
+// tanh form.  The products' gated epilogues take the same choice as epilogue code 1 + act.
+int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter, int act);
 int pa_gather_rows(void* stream, int dtype, const void* x, const int* rows, void* out, int nrows, int width);
 int pa_add_bias(void* stream, int dtype, void* y, const float* b, int tokens, int width);
 int pa_to_f32(void* stream, int dtype, const void* x, float* out, long total);
@@ -82,9 +83,11 @@ int pa_sum_slices(void* stream, int out_dtype, const float* parts, void* out, in
 int pa_pack_tiles(void* stream, const void* w, void* out, int n, int k);
 
 // Paged causal attention, one query token per (seq_of_token[t], positions[t]); window 0 = all keys.
+// softcap (here and in the matrix-core entry points): 0 = none; > 0 bends every scaled score to
+// softcap * tanh(score / softcap) before the softmax.
 int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
                     const int* block_table, int table_stride, const int* seq_of_token, const int* positions, void* out,
-                    int tokens, int nh, int nkv, int hd, int page_size, int window, float scale);
+                    int tokens, int nh, int nkv, int hd, int page_size, int window, float scale, float softcap);
 
 // Matrix-core attention in bfloat16 (K cache [page, nkv, page_size, hd], V cache [page, nkv, hd, page_size]).
 // seq_ids lists the sequences of the step a call handles; cu_q[s] is the first packed token row of sequence s,
@@ -96,26 +99,26 @@ long pa_attn_decode_workspace(int nseq, int nh, int hd, int max_splits);
 int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                    float* workspace, int nseq, int nh, int nkv, int hd, int page_size, int window, float scale,
-                   int split_keys, int max_splits);
+                   float softcap, int split_keys, int max_splits);
 // pa_qknorm_rope_kv + pa_attn_decode in one kernel for steps of single tokens: takes the merged projection,
 // norms and rotates the queries in place of loading them, and writes each token's key and value first.
 int pa_attn_decode_fused(void* stream, const void* qkv, const float* q_weight, const float* k_weight,
                          const float* cos_table, const float* sin_table, const int* slots, float eps,
                          void* kc, void* vc, const int* block_table, int table_stride, const int* seq_ids, const int* cu_q,
                          const int* context_lens, void* out, float* workspace, int nseq, int nh, int nkv, int hd,
-                         int page_size, int window, float scale, int split_keys, int max_splits);
+                         int page_size, int window, float scale, float softcap, int split_keys, int max_splits);
 int pa_attn_decode_fused_supports(int nh, int nkv, int hd, int rot, int page_size);
 int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                     int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                     int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd, int page_size, int window,
-                    float scale);
+                    float scale, float softcap);
 // min_prefix: the fewest keys any sequence has before its portion (0 if unknown), a hint for the cut of the work.
 // The same with the cut of the work given (for tests and measurements): tiles in pairs, heads a wavefront (1, 2, 4),
 // head groups a workgroup (1, 2), keys staged in LDS; -1 leaves one to the launcher.
 int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                         int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                         int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd, int page_size, int window,
-                        float scale, int paired, int heads, int groups, int staged);
+                        float scale, float softcap, int paired, int heads, int groups, int staged);
 
 // out[r] = index of the largest of logits[r, :], the lowest index among equals.
 // scratch: pa_argmax_scratch(rows, vocab) floats (none for narrow rows).

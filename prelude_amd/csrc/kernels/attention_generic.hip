@@ -15,7 +15,8 @@
 // Formula: crates/prelude-core/src/models/qwen3.rs:276-370 and
 // crates/prelude-core/src/ops/traits/attention.rs:10-99 (scores q.k * scale,
 // key c visible to the query at position p when c <= p and, with a window of
-// W keys, c > p - W; softmax in 32-bit; query head h reads KV head h / (nh/nkv)).
+// W keys, c > p - W; softmax in 32-bit; query head h reads KV head h / (nh/nkv)).  The reference's attention has
+// no score cap (qwen3.rs:204); `softcap` > 0 bends the scaled scores to cap * tanh(s / cap) for mixers that want one.
 #include "common.h"
 #include "api.h"
 
@@ -29,7 +30,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, T* __restrict__ out, int nh, int nkv, int hd, int page_size, int window,
-    float scale) {
+    float scale, float softcap) {
   __shared__ float qs[kAttnWaves][kAttnMaxHd];
   __shared__ float ps[kAttnWaves][kWave];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(qs[wave][d], to_f32(kr[d]), dot);
       s = dot * scale;
+      if (softcap != 0.f) s = softcap * tanhf(s / softcap);   // scores bent into (-cap, cap); off: the same bits as ever
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -106,7 +108,7 @@ using namespace pa;
 extern "C" int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
                                const int* block_table, int table_stride, const int* seq_of_token,
                                const int* positions, void* out, int tokens, int nh, int nkv, int hd, int page_size,
-                               int window, float scale) {
+                               int window, float scale, float softcap) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && nh > 0 && nkv > 0 && page_size > 0 && table_stride > 0,
              "attn_generic: bad sizes tokens=%d nh=%d nkv=%d page=%d table_stride=%d", tokens, nh, nkv, page_size,
@@ -114,16 +116,17 @@ extern "C" int pa_attn_generic(void* stream, int dtype, const void* q, const voi
   PA_REQUIRE(nh % nkv == 0, "attn_generic: %d query heads are not a multiple of %d KV heads", nh, nkv);
   PA_REQUIRE(hd > 0 && hd <= kAttnMaxHd, "attn_generic: head_dim %d is outside 1..%d", hd, kAttnMaxHd);
   PA_REQUIRE(window >= 0, "attn_generic: window %d is negative (0 means none)", window);
+  PA_REQUIRE(softcap >= 0.f, "attn_generic: a score cap of %g is negative (0 means none)", (double)softcap);
   dim3 grid(tokens, (nh + kAttnWaves - 1) / kAttnWaves);
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kF32) {
     hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kAttnWaves * kWave), 0, st, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, block_table, table_stride, seq_of_token, positions,
-                       (float*)out, nh, nkv, hd, page_size, window, scale);
+                       (float*)out, nh, nkv, hd, page_size, window, scale, softcap);
   } else if (dtype == kBF16) {
     hipLaunchKernelGGL(attn_generic_kernel<bf16>, grid, dim3(kAttnWaves * kWave), 0, st, (const bf16*)q,
                        (const bf16*)k_cache, (const bf16*)v_cache, block_table, table_stride, seq_of_token, positions,
-                       (bf16*)out, nh, nkv, hd, page_size, window, scale);
+                       (bf16*)out, nh, nkv, hd, page_size, window, scale, softcap);
   } else {
     return pa::fail("attn_generic: unknown element type code %d", dtype);
   }

@@ -45,6 +45,18 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// How raw scores become exponents: 2^(s c - m c) with c = scale log2(e).  With a cap on the scores (cap > 0) a raw
+// score is first bent to cap tanh(s scale / cap) and c is log2(e) alone.  Off (cap == 0) nothing is touched: the
+// same instructions on the same numbers as without the parameter.
+struct ScoreMap {
+  float c;        // exponent per unit of (bent) score
+  float cap;      // 0: none
+  float cap_in;   // scale / cap
+};
+__host__ inline ScoreMap score_map(float scale, float softcap) {
+  return softcap > 0.f ? ScoreMap{kLog2e, softcap, scale / softcap} : ScoreMap{scale * kLog2e, 0.f, 0.f};
+}
+
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
@@ -192,7 +204,7 @@ __device__ __forceinline__ bf16x8 ones8() {
 // `vis(key)` says whether this lane's query may see the key (and the key exists).
 template <int HD, typename Visible>
 __device__ __forceinline__ float scores32(int key0, int g, const KFrag<HD>& kf, const bf16x8* qf, bool masked,
-                                          float* s, Visible vis) {
+                                          const ScoreMap& sm, float* s, Visible vis) {
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     f32x4 acc{0.f, 0.f, 0.f, 0.f};
@@ -200,6 +212,10 @@ __device__ __forceinline__ float scores32(int key0, int g, const KFrag<HD>& kf, 
     for (int ks = 0; ks < KFrag<HD>::KS; ++ks) acc = mfma16(kf.k[t][ks], qf[ks], acc);
 #pragma unroll
     for (int i = 0; i < 4; ++i) s[4 * t + i] = acc[i];
+  }
+  if (sm.cap != 0.f) {   // before the mask: a masked score must stay -inf
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] = sm.cap * tanhf(s[i] * sm.cap_in);
   }
   if (masked) {
 #pragma unroll
@@ -263,15 +279,16 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool valid, int g, bf16
 // reference maximum of one of its columns moved.
 template <int HD, int GT, typename Visible>
 __device__ __forceinline__ void attend32_core(int key0, int g, const KFrag<HD>& kf, const bf16x8* va,
-                                              const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked,
+                                              const bf16x8 (*qf)[(HD + 31) / 32], const ScoreMap& sm, bool masked,
                                               HeadState<HD>* st, Visible vis) {
   constexpr int OT = HeadState<HD>::OT;
   bf16x8 pb[GT];
+  const float c = sm.c;
   const float over = kLazyLog2 / c;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
     float s[8];
-    const float mx = scores32<HD>(key0, g, kf, qf[j], masked, s, vis);
+    const float mx = scores32<HD>(key0, g, kf, qf[j], masked, sm, s, vis);
     if (__any(mx > st[j].lim)) {
       asm volatile("" ::: "memory");  // keep this a branch: as selects it would cost a multiply per output every step
       move_reference<HD>(st[j], mx, c, over);
@@ -291,8 +308,8 @@ __device__ __forceinline__ void attend32_core(int key0, int g, const KFrag<HD>& 
 // arrive under the scores.  `kf` holds the step's K rows, loaded a step ahead.
 template <int HD, int GT, typename Visible>
 __device__ __forceinline__ void attend32(const KeyWalk& w, int key0, int g, int r, const KFrag<HD>& kf,
-                                         const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked, HeadState<HD>* st,
-                                         Visible vis) {
+                                         const bf16x8 (*qf)[(HD + 31) / 32], const ScoreMap& c, bool masked,
+                                         HeadState<HD>* st, Visible vis) {
   constexpr int OT = HeadState<HD>::OT;
   const VChunks vch = v_chunks<HD>(w, key0, g);
   bf16x8 va[OT];
@@ -432,7 +449,7 @@ __global__ __launch_bounds__(WAVES* kWave, 3) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* kc, const bf16* vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_shift, int window, float c,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_shift, int window, ScoreMap c,
     int split_keys, int max_splits, FusedQkv fq, int contiguous) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
@@ -632,8 +649,8 @@ __global__ __launch_bounds__(merge_groups_of(HD) * ((HD + kWave - 1) / kWave * k
 template <int HD, int GT>
 __device__ __forceinline__ void prefill_tile(const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* kc,
                                              const bf16* vc, const int* table, int row0, int q_len, int ctx, int t0,
-                                             int nh, int nkv, int kvh, int head0, int page_shift, int window, float c,
-                                             int g, int r) {
+                                             int nh, int nkv, int kvh, int head0, int page_shift, int window,
+                                             const ScoreMap& c, int g, int r) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
   const int start = ctx - q_len;                // position of the portion's first token
@@ -687,7 +704,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
-    int page_shift, int window, float c, int paired) {
+    int page_shift, int window, ScoreMap c, int paired) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int group = nh / nkv;
@@ -803,7 +820,7 @@ struct Stage {
 // One step over the 32 keys `sub` of the staged block.
 template <int HD, int GT, typename Visible>
 __device__ __forceinline__ void attend32_lds(const StageLds<HD>& lds, int buf, int sub, int key0, int g, int r,
-                                             const bf16x8 (*qf)[(HD + 31) / 32], float c, bool masked,
+                                             const bf16x8 (*qf)[(HD + 31) / 32], const ScoreMap& c, bool masked,
                                              HeadState<HD>* st, Visible vis) {
   constexpr int OT = HeadState<HD>::OT;
   KFrag<HD> kf;
@@ -830,7 +847,7 @@ template <int HD, int GT, int HW>
 __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* __restrict__ q, bf16* __restrict__ out,
                                                  const bf16* kc, const bf16* vc, const int* table, int row0, int q_len,
                                                  int ctx, int tile0, int nh, int nkv, int kvh, int head0, int page_shift,
-                                                 int window, float c, int wave, int g, int r) {
+                                                 int window, const ScoreMap& c, int wave, int g, int r) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
   const int lane = 16 * g + r;
@@ -921,7 +938,7 @@ __global__ __launch_bounds__(256 * HW, 2) void attn_prefill_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int nkv,
-    int page_shift, int window, float c, int paired) {
+    int page_shift, int window, ScoreMap c, int paired) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   StageLds<HD>& lds = *reinterpret_cast<StageLds<HD>*>(lds_raw);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -951,7 +968,7 @@ template <int HD, bool FUSED>
 int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                   float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_shift, int window, float scale,
-                  int split_keys, int max_splits, const FusedQkv& fq) {
+                  float softcap, int split_keys, int max_splits, const FusedQkv& fq) {
   const int qtiles = (nh / nkv + 15) / 16;
   // Up to 1,536 workgroups (what the chip holds at once, below) each XCD gets a contiguous stretch of them; measured
   // in the decode step of a 4B model: batch 8 at 4,096 keys +0.9 %, batch 9 to 12 +0.8 to 1.2 %, batch 2 at 16,384
@@ -971,11 +988,11 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   if (two_wavefronts) {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 2>), grid, dim3(2 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                       part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits, fq, contiguous);
+                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);
   } else {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 4>), grid, dim3(4 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                       part_ml, nh, nkv, page_shift, window, scale * kLog2e, split_keys, max_splits, fq, contiguous);
+                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);
   }
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
@@ -994,7 +1011,7 @@ template <int HD, int GT, int HW>
 int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                           int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                           int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale,
-                          int paired) {
+                          float softcap, int paired) {
   const int tiles = (max_q_len + 63) / 64;
   dim3 grid(nkv * (nh / nkv / (GT * HW)), paired ? (tiles + 1) / 2 : tiles, nseq);
   // the two buffers are more than the 64 KB a kernel may declare: asked for at launch, allowed once per kernel
@@ -1005,27 +1022,27 @@ int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const v
     return pa::fail("attn_prefill: %zu bytes of LDS refused: %s", sizeof(StageLds<HD>), hipGetErrorString(allowed));
   hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, GT, HW>), grid, dim3(256 * HW), sizeof(StageLds<HD>), st,
                      (const bf16*)q, (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q,
-                     context_lens, (bf16*)out, nh, nkv, page_shift, window, scale * kLog2e, paired);
+                     context_lens, (bf16*)out, nh, nkv, page_shift, window, score_map(scale, softcap), paired);
   return check_launch("attn_prefill");
 }
 
 template <int HD, int GT>
 int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                       int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
-                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, int paired,
-                      int hw, bool staged) {
+                      int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, float softcap,
+                      int paired, int hw, bool staged) {
   const int tiles = (max_q_len + 63) / 64;
   dim3 grid(nkv * (nh / nkv / GT), paired ? (tiles + 1) / 2 : tiles, nseq);
   if (staged) {
     if (hw == 2)
       return launch_prefill_staged<HD, GT, 2>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
-                                              nseq, max_q_len, nh, nkv, page_shift, window, scale, paired);
+                                              nseq, max_q_len, nh, nkv, page_shift, window, scale, softcap, paired);
     return launch_prefill_staged<HD, GT, 1>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
-                                            nseq, max_q_len, nh, nkv, page_shift, window, scale, paired);
+                                            nseq, max_q_len, nh, nkv, page_shift, window, scale, softcap, paired);
   }
   hipLaunchKernelGGL((attn_prefill_kernel<HD, GT>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kc,
                      (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, nh, nkv,
-                     page_shift, window, scale * kLog2e, paired);
+                     page_shift, window, score_map(scale, softcap), paired);
   return check_launch("attn_prefill");
 }
 
@@ -1039,7 +1056,7 @@ template <int HD>
 int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
                    int max_q_len, int min_prefix, int nh, int nkv, int page_shift, int window, float scale,
-                   const PrefillCut& want) {
+                   float softcap, const PrefillCut& want) {
   const int group = nh / nkv;
   // How the work is cut: tiles in pairs (an early and a late tile of the causal triangle, so workgroups finish
   // together) and as many heads per wavefront as share the keys and fit the registers (wider heads would not fit
@@ -1111,7 +1128,7 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   PA_REQUIRE(gt <= gt_best, "attn_prefill: %d heads a wavefront, head_dim %d takes up to %d", gt, HD, gt_best);
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
-                                   max_q_len, nh, nkv, page_shift, window, scale, paired, hw, staged)
+                                   max_q_len, nh, nkv, page_shift, window, scale, softcap, paired, hw, staged)
   if constexpr (HD <= 64) {   // four heads' state of a wider head does not fit 256 registers: not built, never chosen
     if (gt == 4) PA_GT(4);
   }
@@ -1160,8 +1177,9 @@ extern "C" long pa_attn_decode_workspace(int nseq, int nh, int hd, int max_split
 extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                               int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                               void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
-                              int window, float scale, int split_keys, int max_splits) {
+                              int window, float scale, float softcap, int split_keys, int max_splits) {
   if (nseq == 0) return 0;
+  PA_REQUIRE(softcap >= 0.f, "attn_decode: a score cap of %g is negative (0 means none)", (double)softcap);
   if (int rc = check_common("attn_decode", nseq, nh, nkv, page_size, table_stride, window)) return rc;
   PA_REQUIRE(split_keys >= 32 && split_keys % 32 == 0, "attn_decode: split of %d keys is not a multiple of 32", split_keys);
   PA_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attn_decode: %d splits", max_splits);
@@ -1171,7 +1189,7 @@ extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const
 #define PA_CALL(HD)                                                                                                  \
   return launch_decode<HD, false>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q,         \
                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, __builtin_ctz(page_size), window, \
-                                  scale, split_keys, max_splits, FusedQkv{})
+                                  scale, softcap, split_keys, max_splits, FusedQkv{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
@@ -1191,8 +1209,9 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
                                     const float* cos_table, const float* sin_table, const int* slots, float eps, void* kc, void* vc, const int* block_table,
                                     int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                                     void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
-                                    int window, float scale, int split_keys, int max_splits) {
+                                    int window, float scale, float softcap, int split_keys, int max_splits) {
   if (nseq == 0) return 0;
+  PA_REQUIRE(softcap >= 0.f, "attn_decode_fused: a score cap of %g is negative (0 means none)", (double)softcap);
   if (int rc = check_common("attn_decode_fused", nseq, nh, nkv, page_size, table_stride, window)) return rc;
   PA_REQUIRE(pa_attn_decode_fused_supports(nh, nkv, hd, hd, page_size), "attn_decode_fused: nh=%d nkv=%d head_dim=%d page=%d are not taken",
              nh, nkv, hd, page_size);
@@ -1206,11 +1225,11 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
   const int shift = __builtin_ctz(page_size);
   if (hd == 64)
     return launch_decode<64, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,
-                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, split_keys,
-                                   max_splits, fq);
+                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, softcap,
+                                   split_keys, max_splits, fq);
   return launch_decode<128, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,
-                                  context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, split_keys,
-                                  max_splits, fq);
+                                  context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, softcap,
+                                  split_keys, max_splits, fq);
 }
 
 // min_prefix: the fewest keys any of the sequences has before its portion (0 if unknown): only a hint for how
@@ -1221,16 +1240,17 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
 extern "C" int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                                    void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
-                                   int page_size, int window, float scale, int paired, int heads, int groups,
-                                   int staged) {
+                                   int page_size, int window, float scale, float softcap, int paired, int heads,
+                                   int groups, int staged) {
   if (nseq == 0) return 0;
   if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
   PA_REQUIRE(max_q_len >= 1 && min_prefix >= 0, "attn_prefill: longest portion %d, shortest prefix %d", max_q_len, min_prefix);
+  PA_REQUIRE(softcap >= 0.f, "attn_prefill: a score cap of %g is negative (0 means none)", (double)softcap);
   PrefillCut cut;
   cut.paired = paired, cut.heads = heads, cut.groups = groups, cut.staged = staged;
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, cut)
+                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, softcap, cut)
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
@@ -1238,13 +1258,14 @@ extern "C" int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, 
 extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                                int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                                void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
-                               int page_size, int window, float scale) {
+                               int page_size, int window, float scale, float softcap) {
   if (nseq == 0) return 0;
   if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
   PA_REQUIRE(max_q_len >= 1 && min_prefix >= 0, "attn_prefill: longest portion %d, shortest prefix %d", max_q_len, min_prefix);
+  PA_REQUIRE(softcap >= 0.f, "attn_prefill: a score cap of %g is negative (0 means none)", (double)softcap);
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale,           \
+                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, softcap,  \
                             PrefillCut{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL

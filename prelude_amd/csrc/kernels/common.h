@@ -19,6 +19,17 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Element type codes shared with the Python side.
 enum DType : int { kF32 = 0, kBF16 = 1 };
 
+// The activation of a gated feed-forward act(gate) * up, by a code shared with the Python side: SiLU
+// x / (1 + e^-x) (crates/prelude-cuda/src/kernels/kernels_src/common/common.cuh:78-80, what the reference's Qwen3
+// is wired to, qwen3.rs:429-447) or GELU in its tanh form 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))) (the
+// reference's Activation::GeluPytorchTanh, crates/prelude-core/src/models/commons/activation.rs:3-25).  The code
+// is the same in every lane, so the choice is a branch, and SiLU's arithmetic is what it was without it.
+enum GateActivation : int { kActSilu = 0, kActGeluTanh = 1, kActCount = 2 };
+__device__ __forceinline__ float gate_activation(float x, int act) {
+  if (act == kActGeluTanh) return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+  return x / (1.0f + expf(-x));
+}
+
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16 v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_f32(float v);

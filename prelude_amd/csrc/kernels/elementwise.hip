@@ -194,16 +194,16 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, const float* __restr
 
 // ---- SiLU(gate) * up over a merged [T, 2I] input whose columns alternate gate_j, up_j ----
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, size_t total) {
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, size_t total, int act) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const float g = to_f32(gate_up[2 * i]);
   const float u = to_f32(gate_up[2 * i + 1]);
-  out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+  out[i] = from_f32<T>(gate_activation(g, act) * u);
 }
 
 // Eight outputs a thread: two 16-byte loads (eight gate/up pairs), one 16-byte store.
-__global__ void silu_mul_vec_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, size_t groups) {
+__global__ void silu_mul_vec_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, size_t groups, int act) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= groups) return;
   const uint4* src = reinterpret_cast<const uint4*>(gate_up) + 2 * i;
@@ -214,8 +214,8 @@ __global__ void silu_mul_vec_kernel(const bf16* __restrict__ gate_up, bf16* __re
   for (int j = 0; j < 4; ++j) {
     const float g0 = (float)a.h[2 * j], u0 = (float)a.h[2 * j + 1];
     const float g1 = (float)b.h[2 * j], u1 = (float)b.h[2 * j + 1];
-    o.h[j] = (bf16)(g0 / (1.0f + expf(-g0)) * u0);
-    o.h[4 + j] = (bf16)(g1 / (1.0f + expf(-g1)) * u1);
+    o.h[j] = (bf16)(gate_activation(g0, act) * u0);
+    o.h[4 + j] = (bf16)(gate_activation(g1, act) * u1);
   }
   reinterpret_cast<uint4*>(out)[i] = o.v;
 }
@@ -347,19 +347,20 @@ extern "C" int pa_rmsnorm_slices(void* stream, int dtype, const float* parts, in
   return rmsnorm_launch(stream, dtype, nullptr, parts, slices, slice_stride, residual, w, out, rows, nrows, hidden, eps);
 }
 
-extern "C" int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter) {
+extern "C" int pa_silu_mul(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter, int act) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && inter > 0, "silu_mul: bad sizes tokens=%d inter=%d", tokens, inter);
+  PA_REQUIRE(act >= 0 && act < kActCount, "silu_mul: unknown activation code %d", act);
   const size_t total = (size_t)tokens * inter;
   if (dtype == kBF16 && inter % 8 == 0) {
     const size_t groups = total / 8;
     hipLaunchKernelGGL(silu_mul_vec_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const bf16*)gate_up, (bf16*)out, groups);
+                       (const bf16*)gate_up, (bf16*)out, groups, act);
     return check_launch("silu_mul");
   }
   const unsigned blocks = (unsigned)((total + 255) / 256);
   PA_DISPATCH(dtype, hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
-                                        (const T*)gate_up, (T*)out, inter, total));
+                                        (const T*)gate_up, (T*)out, inter, total, act));
   return check_launch("silu_mul");
 }
 

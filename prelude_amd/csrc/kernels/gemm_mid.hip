@@ -51,7 +51,7 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
                                                                        const float* __restrict__ bias,
                                                                        TC* __restrict__ c, float* __restrict__ parts,
                                                                        int m, int n, int k, long ldx, long ldc,
-                                                                       int steps_per_slice) {
+                                                                       int steps_per_slice, int act) {
   constexpr int SPC = KC / 64;                  // steps a chunk
   constexpr int CPR = DEPTH / SPC;              // chunks the ring of W steps spans
   static_assert(DEPTH % SPC == 0 && CPR >= 1, "the ring holds whole chunks");
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
         const int nn = nb + 2 * j;
         if (nn + 1 < n) {
           const float gate = acc[t][2 * j], up = acc[t][2 * j + 1];
-          c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate / (1.0f + expf(-gate)) * up);
+          c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate_activation(gate, act) * up);
         }
       }
     } else {
@@ -228,7 +228,7 @@ __global__ void sum_slices_kernel(const float* __restrict__ parts, T* __restrict
 
 template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI>
 int launch_mid(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n, int k,
-               long ldx, long ldc, int slices) {
+               long ldx, long ldc, int slices, int act) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
   const int sps = (steps + slices - 1) / slices;
   constexpr size_t lds = 2 * (size_t)(16 * MT) * (KC + 8) * sizeof(bf16);
@@ -237,7 +237,7 @@ int launch_mid(hipStream_t st, const void* x, const void* w, const float* bias, 
   if (allowed != hipSuccess) return pa::fail("gemm_mid: %zu bytes of LDS refused: %s", lds, hipGetErrorString(allowed));
   dim3 grid((tiles + WN - 1) / WN, (steps + sps - 1) / sps);
   hipLaunchKernelGGL((gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI>), grid, dim3(WN * kWave), lds, st, (const bf16*)x,
-                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps);
+                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps, act);
   return check_launch("gemm_mid");
 }
 
@@ -264,8 +264,8 @@ inline int mid_waves(int n, int slices) {
 
 template <int WN, typename TC, int EPI>
 int launch_mid_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n,
-                  int k, long ldx, long ldc, int slices) {
-#define PA_MID(MT, KC, D) return launch_mid<MT, KC, D, WN, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices)
+                  int k, long ldx, long ldc, int slices, int act) {
+#define PA_MID(MT, KC, D) return launch_mid<MT, KC, D, WN, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act)
   // chunks of 256 columns and a ring of four steps up to 64 rows; 128 columns beyond (LDS holds two chunks);
   // measured over chunk sizes and ring depths at the shapes of a 4B model: within a microsecond of one another
   switch ((m + 15) / 16) {
@@ -282,13 +282,13 @@ int launch_mid_mt(hipStream_t st, const void* x, const void* w, const float* bia
 
 template <typename TC, int EPI>
 int launch_mid_wn(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n,
-                  int k, long ldx, long ldc, int slices, int waves) {
+                  int k, long ldx, long ldc, int slices, int waves, int act = 0) {
   switch (waves ? waves : mid_waves(n, slices)) {
-    case 3: return launch_mid_mt<3, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
-    case 5: return launch_mid_mt<5, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
-    case 6: return launch_mid_mt<6, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
-    case 8: return launch_mid_mt<8, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
-    default: return launch_mid_mt<4, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices);
+    case 3: return launch_mid_mt<3, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act);
+    case 5: return launch_mid_mt<5, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act);
+    case 6: return launch_mid_mt<6, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act);
+    case 8: return launch_mid_mt<8, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act);
+    default: return launch_mid_mt<4, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act);
   }
 }
 
@@ -311,7 +311,7 @@ extern "C" int pa_gemm_mid_slices(int n, int k) {
 extern "C" long pa_gemm_mid_parts(int m, int n, int slices) { return slices <= 1 ? 0 : (long)slices * m * n; }
 
 // C[m, n] = X[m, k] W^T for m <= 128 from the weight in tiles.  slices 1: epilogue 0 writes C (+ bias) as
-// out_dtype (0 float32, 1 bfloat16), epilogue 1 C[m, n/2] = silu(gate) * up.  slices > 1 (epilogue 0 only):
+// out_dtype (0 float32, 1 bfloat16), epilogue 1 + a C[m, n/2] = act_a(gate) * up (GateActivation codes: 1 SiLU, 2 GELU-tanh).  slices > 1 (epilogue 0 only):
 // nothing is written to C; parts [slices, m, n] receives each slice's 32-bit sums (the bias in the first).
 // waves: wavefronts (tiles of 16 rows of W) a workgroup, 3, 4, 5, 6 or 8, or 0 for the launcher's choice; the sums
 // are the same bits at every number.
@@ -336,15 +336,16 @@ extern "C" int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void
     return launch_mid_wn<float, kMidSlices>(st, x, w, bias, nullptr, parts, m, n, k, ldx, ldc, slices, waves);
   }
   PA_REQUIRE(c, "gemm_mid: no output");
-  PA_REQUIRE(epilogue == kMidPlain || (epilogue == kMidSiluMul && n % 2 == 0 && !bias),
-             "gemm_mid: the SiLU*up epilogue needs an even n and no bias");
-  PA_REQUIRE(ldc >= (epilogue == kMidSiluMul ? n / 2 : n), "gemm_mid: output row stride %ld is too small", ldc);
-  if (epilogue == kMidPlain && out_dtype == kBF16)
+  PA_REQUIRE(epilogue >= 0 && epilogue <= kActCount, "gemm_mid: unknown epilogue %d", epilogue);
+  const bool gated = epilogue != kMidPlain;
+  PA_REQUIRE(!gated || (n % 2 == 0 && !bias), "gemm_mid: the gated epilogue needs an even n and no bias");
+  PA_REQUIRE(ldc >= (gated ? n / 2 : n), "gemm_mid: output row stride %ld is too small", ldc);
+  if (!gated && out_dtype == kBF16)
     return launch_mid_wn<bf16, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves);
-  if (epilogue == kMidPlain && out_dtype == kF32)
+  if (!gated && out_dtype == kF32)
     return launch_mid_wn<float, kMidPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves);
-  if (epilogue == kMidSiluMul && out_dtype == kBF16)
-    return launch_mid_wn<bf16, kMidSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves);
+  if (gated && out_dtype == kBF16)
+    return launch_mid_wn<bf16, kMidSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, waves, epilogue - 1);
   return pa::fail("gemm_mid: unsupported output type %d with epilogue %d", out_dtype, epilogue);
 }
 

@@ -92,7 +92,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
                                                                    const bf16* __restrict__ w,
                                                                    const float* __restrict__ bias,
                                                                    TC* __restrict__ c, int m, int n, int k, long ldx,
-                                                                   long ldc) {
+                                                                   long ldc, int act) {
   __shared__ float red[WAVES][NT * MT][kWave][4];
   // the wavefront's number as a scalar: what depends on it (the steps it takes, the loop's end) is then uniform
   // for the compiler too, and a branch on it is a branch, not a mask
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
         const int nn = nb + 2 * j;
         if (nn + 1 < n) {
           const float gate = fin[t][2 * j], up = fin[t][2 * j + 1];
-          c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate / (1.0f + expf(-gate)) * up);
+          c[(size_t)mi * ldc + nn / 2] = from_f32<TC>(gate_activation(gate, act) * up);
         }
       }
     } else {
@@ -267,11 +267,11 @@ constexpr bool skinny_built() {
 
 template <int MT, int NT, int WV, typename TC, int EPI, bool TILED, int DEPTH>
 int launch_skinny_as(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                     long ldx, long ldc) {
+                     long ldx, long ldc, int act) {
   if constexpr (skinny_built<MT, TILED, NT, WV>()) {
     dim3 grid(((n + 15) / 16 + NT - 1) / NT);
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED, DEPTH>), grid, dim3(WV * kWave), 0, st,
-                       (const bf16*)x, (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc);
+                       (const bf16*)x, (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc, act);
     return check_launch("gemm_skinny");
   } else {
     return pa::fail("gemm_skinny: no kernel for %d row tiles with %d tiles a workgroup on %d wavefronts (%s weight)", MT,
@@ -281,10 +281,10 @@ int launch_skinny_as(hipStream_t st, const void* x, const void* w, const float* 
 
 template <int MT, typename TC, int EPI, bool TILED, int DEPTH>
 int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                        long ldx, long ldc) {
+                        long ldx, long ldc, int act) {
   int nt, waves, depth;
   skinny_shape(m, n, k, MT, TILED, &nt, &waves, &depth);
-#define PA_AS(NT, WV) return launch_skinny_as<MT, NT, WV, TC, EPI, TILED, DEPTH>(st, x, w, bias, c, m, n, k, ldx, ldc)
+#define PA_AS(NT, WV) return launch_skinny_as<MT, NT, WV, TC, EPI, TILED, DEPTH>(st, x, w, bias, c, m, n, k, ldx, ldc, act)
 #define PA_WAVES(NT)     \
   switch (waves) {       \
     case 16: PA_AS(NT, 16); \
@@ -304,27 +304,27 @@ int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const floa
 
 template <int MT, typename TC, int EPI, bool TILED>
 int launch_skinny(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                  long ldx, long ldc) {
+                  long ldx, long ldc, int act) {
   // the depth is part of the kernel's type: one step in flight for tiles, kDepth for rows (see skinny_shape)
-  return launch_skinny_depth<MT, TC, EPI, TILED, TILED ? 1 : kDepth>(st, x, w, bias, c, m, n, k, ldx, ldc);
+  return launch_skinny_depth<MT, TC, EPI, TILED, TILED ? 1 : kDepth>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
 }
 
 template <typename TC, int EPI>
 int launch_skinny_mt(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                     long ldx, long ldc, int tiled) {
+                     long ldx, long ldc, int act, int tiled) {
   if (tiled) {
     switch ((m + 15) / 16) {
-      case 1: return launch_skinny<1, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
-      case 2: return launch_skinny<2, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
-      case 3: return launch_skinny<3, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
-      default: return launch_skinny<4, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc);
+      case 1: return launch_skinny<1, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
+      case 2: return launch_skinny<2, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
+      case 3: return launch_skinny<3, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
+      default: return launch_skinny<4, TC, EPI, true>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
     }
   }
   switch ((m + 15) / 16) {
-    case 1: return launch_skinny<1, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
-    case 2: return launch_skinny<2, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
-    case 3: return launch_skinny<3, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
-    default: return launch_skinny<4, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc);
+    case 1: return launch_skinny<1, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
+    case 2: return launch_skinny<2, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
+    case 3: return launch_skinny<3, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
+    default: return launch_skinny<4, TC, EPI, false>(st, x, w, bias, c, m, n, k, ldx, ldc, act);
   }
 }
 
@@ -361,7 +361,8 @@ extern "C" int pa_pack_tiles(void* stream, const void* w, void* out, int n, int 
   return check_launch("pack_tiles");
 }
 
-// tiled 1: w is the weight in tiles (pa_pack_tiles).
+// tiled 1: w is the weight in tiles (pa_pack_tiles).  epilogue 0: C (+ bias); 1 + a: C[m, n/2] = act_a(gate) * up
+// over rows that alternate gate_j, up_j, a one of the GateActivation codes (1: SiLU, 2: GELU in its tanh form).
 extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w,
                               const float* bias, void* c, int m, int n, int k, long ldx, long ldc, int tiled) {
   if (m == 0 || n == 0) return 0;
@@ -369,15 +370,18 @@ extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const v
   PA_REQUIRE(m <= kSkinnyMaxM, "gemm_skinny: %d rows exceed %d", m, kSkinnyMaxM);
   PA_REQUIRE(k % 8 == 0 && ldx % 8 == 0, "gemm_skinny: k=%d and the row stride %ld must be multiples of 8", k, ldx);
   PA_REQUIRE(ldx >= k, "gemm_skinny: row stride %ld is smaller than k=%d", ldx, k);
-  PA_REQUIRE(epilogue == kPlain || (n % 2 == 0 && !bias), "gemm_skinny: the SiLU*up epilogue needs an even n and no bias");
-  PA_REQUIRE(ldc >= (epilogue == kSiluMul ? n / 2 : n), "gemm_skinny: output row stride %ld is too small", ldc);
+  PA_REQUIRE(epilogue >= 0 && epilogue <= kActCount, "gemm_skinny: unknown epilogue %d", epilogue);
+  const bool gated = epilogue != kPlain;
+  const int act = gated ? epilogue - 1 : 0;
+  PA_REQUIRE(!gated || (n % 2 == 0 && !bias), "gemm_skinny: the gated epilogue needs an even n and no bias");
+  PA_REQUIRE(ldc >= (gated ? n / 2 : n), "gemm_skinny: output row stride %ld is too small", ldc);
 
   hipStream_t st = (hipStream_t)stream;
-  if (epilogue == kPlain && out_dtype == kBF16)
-    return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);
-  if (epilogue == kPlain && out_dtype == kF32)
-    return launch_skinny_mt<float, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);
-  if (epilogue == kSiluMul && out_dtype == kBF16)
-    return launch_skinny_mt<bf16, kSiluMul>(st, x, w, bias, c, m, n, k, ldx, ldc, tiled);
+  if (!gated && out_dtype == kBF16)
+    return launch_skinny_mt<bf16, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, act, tiled);
+  if (!gated && out_dtype == kF32)
+    return launch_skinny_mt<float, kPlain>(st, x, w, bias, c, m, n, k, ldx, ldc, act, tiled);
+  if (gated && out_dtype == kBF16)
+    return launch_skinny_mt<bf16, kSiluMul>(st, x, w, bias, c, m, n, k, ldx, ldc, act, tiled);
   return pa::fail("gemm_skinny: unsupported output type %d with epilogue %d", out_dtype, epilogue);
 }

@@ -47,7 +47,7 @@ template <int MT, int NT, int DEPTH, int OCC, typename TC, int EPI>
 __global__ __launch_bounds__(kTallThreads, OCC) void gemm_tall_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias, TC* __restrict__ c,
     float* __restrict__ parts, int m, int n, int k, long ldx, long ldc, int steps_per_slice, int row_tiles,
-    int col_groups) {
+    int col_groups, int act) {
   static_assert(MT % 2 == 0 && DEPTH % 2 == 0, "pieces and buffers are dealt out in twos");
   constexpr int ROWS = 16 * MT;
   constexpr int PIECES = ROWS * 8 / kTallThreads;   // 16-byte pieces of a step a thread stages
@@ -177,11 +177,11 @@ __global__ __launch_bounds__(kTallThreads, OCC) void gemm_tall_kernel(
         TC* dst = c + (size_t)mi * ldc + nb / 2;
         if (nb + 3 < n) {
           const float g0 = acc[t][j][0], u0 = acc[t][j][1], g1 = acc[t][j][2], u1 = acc[t][j][3];
-          dst[0] = from_f32<TC>(g0 / (1.0f + expf(-g0)) * u0);
-          dst[1] = from_f32<TC>(g1 / (1.0f + expf(-g1)) * u1);
+          dst[0] = from_f32<TC>(gate_activation(g0, act) * u0);
+          dst[1] = from_f32<TC>(gate_activation(g1, act) * u1);
         } else if (nb + 1 < n) {
           const float g0 = acc[t][j][0], u0 = acc[t][j][1];
-          dst[0] = from_f32<TC>(g0 / (1.0f + expf(-g0)) * u0);
+          dst[0] = from_f32<TC>(gate_activation(g0, act) * u0);
         }
       } else {
         TC* dst = c + (size_t)mi * ldc + nb;
@@ -200,22 +200,22 @@ __global__ __launch_bounds__(kTallThreads, OCC) void gemm_tall_kernel(
 
 template <int MT, int NT, int DEPTH, int OCC, typename TC, int EPI>
 int launch_tall(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n, int k,
-                long ldx, long ldc, int slices) {
+                long ldx, long ldc, int slices, int act) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
   const int sps = (steps + slices - 1) / slices;
   const int row_tiles = (m + 16 * MT - 1) / (16 * MT);
   const int col_groups = (tiles + kTallWaves * NT - 1) / (kTallWaves * NT);
   dim3 grid((unsigned)((col_groups + 7) / 8 * 8 * row_tiles), (unsigned)((steps + sps - 1) / sps));
   hipLaunchKernelGGL((gemm_tall_kernel<MT, NT, DEPTH, OCC, TC, EPI>), grid, dim3(kTallThreads), 0, st, (const bf16*)x,
-                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps, row_tiles, col_groups);
+                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps, row_tiles, col_groups, act);
   return check_launch("gemm_tall");
 }
 
 template <typename TC, int EPI>
 int launch_tall_shape(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n,
-                      int k, long ldx, long ldc, int slices, int mt, int nt) {
+                      int k, long ldx, long ldc, int slices, int mt, int nt, int act = 0) {
 #define PA_TALL(MT, NT, D, OCC) \
-  if (mt == MT && nt == NT) return launch_tall<MT, NT, D, OCC, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices)
+  if (mt == MT && nt == NT) return launch_tall<MT, NT, D, OCC, TC, EPI>(st, x, w, bias, c, parts, m, n, k, ldx, ldc, slices, act)
   // a ring of two steps: four and six measured the same (the loop is not waiting for the loads' latency)
   PA_TALL(4, 2, 2, 2);
   PA_TALL(4, 3, 2, 2);
@@ -258,7 +258,7 @@ extern "C" void pa_gemm_tall_shape(int m, int n, int k, int slices, int* out) {
 }
 
 // C[m, n] = X[m, k] W^T from the weight in tiles, any m.  slices 1: epilogue 0 writes C (+ bias) in bfloat16,
-// epilogue 1 C[m, n/2] = silu(gate) * up.  slices > 1 (epilogue 0 only): nothing is written to C; parts
+// epilogue 1 + a C[m, n/2] = act_a(gate) * up (GateActivation codes: 1 SiLU, 2 GELU-tanh).  slices > 1 (epilogue 0 only): nothing is written to C; parts
 // [slices, m, n] receives each slice's 32-bit sums (the bias in the first).  mt, nt: the workgroup's shape (tiles
 // of 16 rows of X a workgroup, tiles of 16 rows of W a wavefront), or 0, 0 for the launcher's choice; the sums are
 // the same bits at every shape.
@@ -285,10 +285,11 @@ extern "C" int pa_gemm_tall(void* stream, int epilogue, const void* x, const voi
     return launch_tall_shape<float, kTallSlices>(st, x, w, bias, nullptr, parts, m, n, k, ldx, ldc, slices, mt, nt);
   }
   PA_REQUIRE(c, "gemm_tall: no output");
-  PA_REQUIRE(epilogue == kTallPlain || (epilogue == kTallSiluMul && n % 2 == 0 && !bias),
-             "gemm_tall: the SiLU*up epilogue needs an even n and no bias");
-  PA_REQUIRE(ldc >= (epilogue == kTallSiluMul ? n / 2 : n), "gemm_tall: output row stride %ld is too small", ldc);
-  if (epilogue == kTallPlain)
+  PA_REQUIRE(epilogue >= 0 && epilogue <= kActCount, "gemm_tall: unknown epilogue %d", epilogue);
+  const bool gated = epilogue != kTallPlain;
+  PA_REQUIRE(!gated || (n % 2 == 0 && !bias), "gemm_tall: the gated epilogue needs an even n and no bias");
+  PA_REQUIRE(ldc >= (gated ? n / 2 : n), "gemm_tall: output row stride %ld is too small", ldc);
+  if (!gated)
     return launch_tall_shape<bf16, kTallPlain>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, mt, nt);
-  return launch_tall_shape<bf16, kTallSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, mt, nt);
+  return launch_tall_shape<bf16, kTallSiluMul>(st, x, w, bias, c, nullptr, m, n, k, ldx, ldc, 1, mt, nt, epilogue - 1);
 }

@@ -166,7 +166,7 @@ class Engine:
         total = 0
         for cs, g in zip(specs, self._group_of_slot):
             if g is not None:
-                total += pages[g] * self.page_size * cs.num_kv_heads * (cs.head_dim + cs.v_dim) * el
+                total += pages[g] * self.page_size * int(cs.bytes_per_token(el))
         return total
 
     def _decide_cache_tokens(self, specs, state_slots: int) -> int:

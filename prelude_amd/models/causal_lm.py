@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..parts import Block, Part, StateSpec, TensorReq, build_part
+from ..parts import Block, Part, TensorReq, build_part
 from ..parts.base import PartError, _REGISTRY
 from .spec import ModelSpec, PartSpec
 
@@ -23,7 +23,7 @@ from .spec import ModelSpec, PartSpec
 class CacheSlot:
     """What one run of a layer keeps between steps."""
     run: int                    # index in the run order that owns (writes) it
-    spec: object                # KVCacheSpec | StateSpec
+    spec: object                # a PagedCacheSpec (keys and values, or a kind of the mixer's own) | a SlotCacheSpec
 
 
 class CausalLM:
@@ -125,7 +125,7 @@ class CausalLM:
     # ---- what the cache manager must provide ------------------------------
     @property
     def needs_state(self) -> bool:
-        return any(isinstance(c.spec, StateSpec) for c in self.cache_slots)
+        return any(not getattr(c.spec, "PAGED", False) for c in self.cache_slots)
 
     @property
     def graph_safe(self) -> bool:

@@ -145,14 +145,26 @@ def _rmsnorm_slices(x, weight: torch.Tensor, eps: float, residual: Optional[torc
     return out
 
 
-def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(gate) * up for gate_up [T, 2I] whose columns alternate gate_j, up_j -> [T, I]."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}   # codes of the kernels' gated epilogues (common.h)
+
+
+def gate_activation_code(name: str) -> int:
+    try:
+        return GATE_ACTIVATIONS[name]
+    except KeyError:
+        raise NativeError(f"gated activation {name!r} is not one of {sorted(GATE_ACTIVATIONS)}") from None
+
+
+def silu_mul(gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """act(gate) * up for gate_up [T, 2I] whose columns alternate gate_j, up_j -> [T, I]; ``activation`` is
+    ``"silu"`` or ``"gelu_tanh"``, here and in the gated epilogues of the products."""
+    act = gate_activation_code(activation)
     _dev(gate_up)
     if gate_up.dim() != 2 or gate_up.shape[1] % 2:
         raise NativeError(f"silu_mul: input {tuple(gate_up.shape)} is not [T, 2I]")
     inter = gate_up.shape[1] // 2
     out = torch.empty((gate_up.shape[0], inter), dtype=gate_up.dtype, device=gate_up.device)
-    check(kernels().pa_silu_mul(_stream(), _code(gate_up), _ptr(gate_up), _ptr(out), gate_up.shape[0], inter))
+    check(kernels().pa_silu_mul(_stream(), _code(gate_up), _ptr(gate_up), _ptr(out), gate_up.shape[0], inter, act))
     return out
 
 
@@ -327,12 +339,14 @@ def prepare_weight(w: torch.Tensor) -> LinearWeight:
 
 
 def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
-                out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False) -> torch.Tensor:
+                out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False,
+                activation: str = "silu") -> torch.Tensor:
     """x [M <= 64, K] @ w[N, K]^T in bfloat16 on the matrix cores, streaming w once.
 
     ``w`` is a tensor [N, K] or a ``TiledWeight``.  With
     ``silu_mul_epilogue`` the rows of w alternate gate_j, up_j and the
-    result is silu(gate) * up, [M, N/2]."""
+    result is act(gate) * up, [M, N/2], act being ``activation``."""
+    epi = 1 + gate_activation_code(activation) if silu_mul_epilogue else 0
     tiled = isinstance(w, TiledWeight)
     wt = w.data if tiled else w
     _dev(x, wt, bias)
@@ -346,7 +360,7 @@ def gemm_skinny(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
         raise NativeError(f"gemm_skinny: bias {tuple(bias.shape)} is not [{n}]")
     cols = n // 2 if silu_mul_epilogue else n
     out = torch.empty((m, cols), dtype=out_dtype, device=x.device)
-    check(kernels().pa_gemm_skinny(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(wt),
+    check(kernels().pa_gemm_skinny(_stream(), _CODES[out_dtype], epi, _ptr(x), _ptr(wt),
                                    _ptr(bias), _ptr(out), m, n, k, k, cols, 1 if tiled else 0))
     return out
 
@@ -404,12 +418,14 @@ def gemm_mid_slices(n: int, k: int) -> int:
 
 
 def gemm_mid(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = None,
-             out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False, slices: int = 1, waves: int = 0):
+             out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False, slices: int = 1, waves: int = 0,
+             activation: str = "silu"):
     """x [M <= 128, K] @ w[N, K]^T from the weight in tiles, X staged through LDS; with ``slices`` > 1 the result
     is a ``SliceSums`` (one 32-bit partial sum per slice of K) instead of a tensor.  ``waves``: wavefronts a
     workgroup (3, 4, 5, 6, 8; 0 lets the launcher choose by the weight's shape; the same bits at every number)."""
     if not isinstance(w, TiledWeight):
         raise NativeError("gemm_mid takes the weight in tiles (pack_tiles)")
+    epi = 1 + gate_activation_code(activation) if silu_mul_epilogue else 0
     _dev(x, w.data, bias)
     _f32(bias, "bias")
     if x.dim() != 2 or x.shape[1] != w.k or x.dtype != torch.bfloat16:
@@ -426,18 +442,19 @@ def gemm_mid(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = N
         return SliceSums(parts, out_dtype)
     cols = n // 2 if silu_mul_epilogue else n
     out = torch.empty((m, cols), dtype=out_dtype, device=x.device)
-    check(kernels().pa_gemm_mid(_stream(), _CODES[out_dtype], 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w.data),
+    check(kernels().pa_gemm_mid(_stream(), _CODES[out_dtype], epi, _ptr(x), _ptr(w.data),
                                 _ptr(bias), _ptr(out), None, m, n, k, k, cols, 1, waves))
     return out
 
 
 def gemm_tall(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = None, silu_mul_epilogue: bool = False,
-              slices: int = 1, shape=(0, 0)):
+              slices: int = 1, shape=(0, 0), activation: str = "silu"):
     """x [M, K] @ w[N, K]^T for any number of rows from the weight in tiles, the output tiled both ways: a
     workgroup owns ``16 * shape[0]`` rows of X and ``64 * shape[1]`` rows of W ((0, 0): the launcher chooses by the
     product's size; the same bits at every shape).  bfloat16 out; with ``slices`` > 1 a ``SliceSums``."""
     if not isinstance(w, TiledWeight):
         raise NativeError("gemm_tall takes the weight in tiles (pack_tiles)")
+    epi = 1 + gate_activation_code(activation) if silu_mul_epilogue else 0
     _dev(x, w.data, bias)
     _f32(bias, "bias")
     if x.dim() != 2 or x.shape[1] != w.k or x.dtype != torch.bfloat16:
@@ -453,7 +470,7 @@ def gemm_tall(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = 
         return SliceSums(parts, torch.bfloat16)
     cols = n // 2 if silu_mul_epilogue else n
     out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
-    check(kernels().pa_gemm_tall(_stream(), 1 if silu_mul_epilogue else 0, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out),
+    check(kernels().pa_gemm_tall(_stream(), epi, _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out),
                                  None, m, n, k, k, cols, 1, int(shape[0]), int(shape[1])))
     return out
 
@@ -622,31 +639,41 @@ def _gated_tiled(m: int, n: int, k: int) -> bool:
     return n * k <= GATED_TILED_ELEMENTS and k < 8192 and (m <= GATED_TILED_ROWS or (m <= 32 and k >= GATED_TILED_LONG_K))
 
 
-def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) for a weight [2I, K] whose rows alternate gate_j, up_j."""
+def linear_gated(x: torch.Tensor, w, activation: str = "silu") -> torch.Tensor:
+    """act(x Wg^T) * (x Wu^T) for a weight [2I, K] whose rows alternate gate_j, up_j; ``activation`` is ``"silu"``
+    or ``"gelu_tanh"`` (the same kernels, another epilogue code)."""
+    gate_activation_code(activation)
     m, k = x.shape
     if x.dtype == torch.bfloat16 and k % 8 == 0:
         tiles = w.tiles if isinstance(w, LinearWeight) else None
         if m <= SKINNY_MAX_ROWS:
             if (MID_PRODUCTS and tiles is not None and tiles.n * k <= GATED_TILED_ELEMENTS
                     and m >= (GATED_MID_MIN_ROWS if k < GATED_TILED_LONG_K else 1)):
-                return gemm_mid(x, tiles, silu_mul_epilogue=True)
+                return gemm_mid(x, tiles, silu_mul_epilogue=True, activation=activation)
             if isinstance(w, LinearWeight):
                 w = tiles if tiles is not None and m <= 16 else w.rows
-            return gemm_skinny(x, w, silu_mul_epilogue=True)
+            return gemm_skinny(x, w, silu_mul_epilogue=True, activation=activation)
         if MID_PRODUCTS and tiles is not None and m <= GEMM_MID_MAX_ROWS and tiles.n * k <= GATED_TILED_ELEMENTS:
-            return gemm_mid(x, tiles, silu_mul_epilogue=True)
+            return gemm_mid(x, tiles, silu_mul_epilogue=True, activation=activation)
         if tiles is not None and _gated_tiled(m, tiles.n, k):
-            return gemm_skinny(x, tiles, silu_mul_epilogue=True)
+            return gemm_skinny(x, tiles, silu_mul_epilogue=True, activation=activation)
         if (TALL_PRODUCTS & 2 and tiles is not None and GEMM_MID_MAX_ROWS < m <= TALL_MAX_ROWS and k < TALL_GATED_MAX_K
                 and tiles.n % 2 == 0):
-            return gemm_tall(x, tiles, silu_mul_epilogue=True)
-    return silu_mul(linear(x, w))
+            return gemm_tall(x, tiles, silu_mul_epilogue=True, activation=activation)
+    return silu_mul(linear(x, w), activation)
+
+
+def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
+    """``linear_gated`` with SiLU, the reference's own feed-forward (crates/prelude-core/src/models/qwen3.rs:429-447)."""
+    return linear_gated(x, w, "silu")
 
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
-                      seq_of_token: torch.Tensor, positions: torch.Tensor, window: int, scale: float) -> torch.Tensor:
-    """Paged causal attention, any mix of portions and decode tokens.
+                      seq_of_token: torch.Tensor, positions: torch.Tensor, window: int, scale: float,
+                      softcap: float = 0.0) -> torch.Tensor:
+    """Paged causal attention, any mix of portions and decode tokens.  ``softcap`` > 0 (here and in the other
+    attention entry points) bends every scaled score to ``softcap * tanh(score / softcap)`` before the softmax;
+    0, the default, leaves the scores alone (the same bits as without the parameter).
 
     q [T, nh, hd]; K cache [pages, nkv, page, hd], V cache [pages, nkv, hd, page]; block_table int32 [B, stride];
     seq_of_token / positions int32 [T].  window 0 = all keys.
@@ -665,7 +692,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     out = torch.empty_like(q)
     check(kernels().pa_attn_generic(_stream(), _code(q), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
                                     block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out), t, nh,
-                                    k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale)))
+                                    k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale), float(softcap)))
     return out
 
 
@@ -710,7 +737,7 @@ def mfma_attention_supported(head_dim: int, page_size: int) -> bool:
 
 
 def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_context: int,
-                     window: int, scale: float, every_seq: bool = False) -> None:
+                     window: int, scale: float, every_seq: bool = False, softcap: float = 0.0) -> None:
     """Matrix-core attention for the sequences ``seq_ids`` (each feeding one token); writes their rows of ``out``.
     ``every_seq``: ``seq_ids`` is 0, 1, .. (a step of single tokens only); the kernels then count for themselves
     instead of reading it, which is one trip to memory less before their first key."""
@@ -727,7 +754,7 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_le
                                    block_table.shape[1], None if every_seq else _ptr(seq_ids), _ptr(cu_q),
                                    _ptr(context_lens), _ptr(out),
                                    _ptr(ws), n, nh, k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale),
-                                   DECODE_SPLIT_KEYS, max_splits))
+                                   float(softcap), DECODE_SPLIT_KEYS, max_splits))
 
 
 def attention_decode_fused_supported(nh: int, nkv: int, hd: int, rot: int, page_size: int) -> bool:
@@ -736,7 +763,7 @@ def attention_decode_fused_supported(nh: int, nkv: int, hd: int, rot: int, page_
 
 def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float, k_cache, v_cache,
                            block_table, seq_ids, cu_q, context_lens, nh: int, max_context: int, window: int,
-                           scale: float, every_seq: bool = False) -> torch.Tensor:
+                           scale: float, every_seq: bool = False, softcap: float = 0.0) -> torch.Tensor:
     """``qknorm_rope_kv`` and ``attention_decode`` in one kernel, for a step in which every sequence feeds one
     token: takes the merged projection [T, (nh + 2 nkv) * hd], writes the tokens' keys and values into the caches
     and returns the attention output [T, nh, hd].  A token's position is its sequence's context length less one.
@@ -766,12 +793,12 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
                                          _ptr(block_table), block_table.shape[1],
                                          None if every_seq else _ptr(seq_ids), _ptr(cu_q),
                                          _ptr(context_lens), _ptr(out), _ptr(ws), n, nh, nkv, hd, page, int(window),
-                                         float(scale), DECODE_SPLIT_KEYS, max_splits))
+                                         float(scale), float(softcap), DECODE_SPLIT_KEYS, max_splits))
     return out
 
 
 def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_q_len: int,
-                      window: int, scale: float, cut=None, min_prefix: int = 0) -> None:
+                      window: int, scale: float, cut=None, min_prefix: int = 0, softcap: float = 0.0) -> None:
     """Matrix-core attention for the sequences ``seq_ids`` (portions of several tokens); writes their rows of ``out``.
 
     ``min_prefix`` is the fewest keys any of the sequences has before its portion: a hint for how the launcher
@@ -786,7 +813,7 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_l
         return
     args = (_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_ids),
             _ptr(cu_q), _ptr(context_lens), _ptr(out), n, int(max_q_len), int(min_prefix), nh, k_cache.shape[1], hd,
-            k_cache.shape[2], int(window), float(scale))
+            k_cache.shape[2], int(window), float(scale), float(softcap))
     if cut is None:
         check(kernels().pa_attn_prefill(*args))
     else:
@@ -794,7 +821,7 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_l
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int,
-              scale: float) -> torch.Tensor:
+              scale: float, softcap: float = 0.0) -> torch.Tensor:
     """Attention of one step over one cache group; picks the kernel for the sizes at hand.
 
     ``group`` is the step's ``GroupStep`` of the cache group, ``step`` the ``StepBatch``.
@@ -808,12 +835,13 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
         if step.n_decode:
             attention_decode(q, k_cache, v_cache, group.block_table, step.decode_seqs, step.cu_q, step.context_lens,
                              out, step.max_decode_context, window, scale,
-                             every_seq=step.n_prefill == 0 and step.n_decode == step.num_seqs)
+                             every_seq=step.n_prefill == 0 and step.n_decode == step.num_seqs, softcap=softcap)
         if step.n_prefill:
             attention_prefill(q, k_cache, v_cache, group.block_table, step.prefill_seqs, step.cu_q, step.context_lens,
-                              out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix)
+                              out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix, softcap=softcap)
         return out
-    return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale)
+    return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale,
+                             softcap)
 
 
 def logprobs(logits: torch.Tensor, ids: torch.Tensor, k: int = 0):

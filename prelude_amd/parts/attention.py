@@ -26,7 +26,7 @@ class GQAAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, norm_eps: float = 1e-6,
                  qk_norm: bool = True, bias: bool = False, window: int = 0, position: Optional[str] = None,
-                 rotary_dim: Optional[int] = None, scale: Optional[float] = None):
+                 rotary_dim: Optional[int] = None, scale: Optional[float] = None, score_cap: float = 0.0):
         if num_heads % num_kv_heads:
             raise PartError(f"gqa_attention: {num_heads} heads are not a multiple of {num_kv_heads} KV heads")
         # what the kernels take: the matrix-core attention has head sizes of its own (others go to the generic
@@ -38,6 +38,11 @@ class GQAAttention(Mixer):
         self.position = position
         self.rotary_dim = (head_dim if rotary_dim is None else int(rotary_dim)) if position else 0
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        # > 0: scaled scores are bent to cap * tanh(score / cap) before the softmax (the reference's Qwen3 has none,
+        # qwen3.rs:204; a parameter for mixers of other models)
+        self.score_cap = float(score_cap or 0.0)
+        if self.score_cap < 0:
+            raise PartError(f"gqa_attention: a score cap of {score_cap} is negative")
         self.rope = None
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = None
 
@@ -94,7 +99,8 @@ class GQAAttention(Mixer):
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
             o = K.attention_decode_fused(qkv, self.q_norm, self.k_norm, cos, sin, g.slots, self.norm_eps,
                                          cache.k, cache.v, g.block_table, step.decode_seqs, step.cu_q, step.context_lens,
-                                         nh, step.max_decode_context, self.window, self.scale, every_seq=True)
+                                         nh, step.max_decode_context, self.window, self.scale, every_seq=True,
+                                         softcap=self.score_cap)
             return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)
         if write_cache:
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
@@ -105,5 +111,5 @@ class GQAAttention(Mixer):
             qx = K.linear(x, self.w_qkv.first_rows(nh * hd), bq)
             q = K.qknorm_rope_kv(qx, self.q_norm, None, cos, sin, step.positions, None, None, None, nh, 0, hd,
                                  self.rotary_dim, self.norm_eps)
-        o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale)
+        o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale, self.score_cap)
         return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)

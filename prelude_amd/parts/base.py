@@ -12,7 +12,8 @@ Categories and the interface each must have:
 ``mixer``/``ffn`` may return their last product as ``ops.kernels.SliceSums`` (``linear(..., slices_ok=True)``):
               only a norm reads it, and one that says ``TAKES_SLICE_SUMS`` adds the slices itself
 ``position``  ``prepare(device)``; what it offers (tables) is between it and the mixers that name it
-``mixer``     ``cache_spec()`` -> ``KVCacheSpec`` | ``StateSpec`` | ``None``;
+``mixer``     ``cache_spec()`` -> a ``PagedCacheSpec`` (``KVCacheSpec`` or a kind of the mixer's own) | a
+              ``SlotCacheSpec`` (``StateSpec``) | ``None``;
               ``forward(x, step, cache, write_cache=True)``
 ``ffn``       ``forward(x)``
 ``block``     ``forward(hidden, residual, step, cache, write_cache) -> (hidden, residual)``
@@ -42,11 +43,82 @@ class TensorReq:
     kind: str = MATRIX
 
 
+class PagedCacheSpec:
+    """What a mixer keeps per token, in pages: the interface the cache manager works with.
+
+    A kind of its own is a frozen dataclass derived from this.  Mixers whose specs compare equal share a *group*:
+    one pool of pages and one block table per request (each mixer still has its own storage behind those
+    tables).  ``window`` > 0 says that a token looks back over that many places only, its own included; pages a
+    window has passed are given back while the request lives.  Keys and values (``KVCacheSpec``) are one such
+    kind; a mixer that keeps something else per token -- one latent vector, say -- brings its own.
+    """
+    PAGED = True
+    window: int = 0
+
+    def bytes_per_token(self, element_size: int) -> int:
+        """Bytes a token takes in this mixer's storage, for an engine element of ``element_size`` bytes."""
+        raise NotImplementedError
+
+    def allocate(self, pages: int, page_size: int, dtype: torch.dtype, device: torch.device, group: int):
+        """Zeroed storage for ``pages`` pages of ``page_size`` tokens: the object the mixer's ``forward`` gets as
+        ``cache``.  It carries ``group``, the index of the step's ``GroupStep`` (block table, slot numbers)."""
+        raise NotImplementedError
+
+
+class SlotCacheSpec:
+    """What a mixer keeps per request, of fixed size: a slot of every tensor it names.  ``allocate`` returns the
+    object the mixer's ``forward`` gets as ``cache``; it must offer ``zero_fresh(state_slots, fresh)`` (clears the
+    rows of starting requests on the device) and, to be replayed from graphs, ``snapshot`` / ``restore``."""
+    PAGED = False
+
+    def bytes_per_slot(self) -> int:
+        raise NotImplementedError
+
+    def allocate(self, slots: int, device: torch.device):
+        raise NotImplementedError
+
+
+@dataclasses.dataclass
+class KVLayerCache:
+    """What an attention-like mixer gets: its pages and the group whose tables index them."""
+    k: torch.Tensor   # [pages, kv_heads, page_size, head_dim]
+    v: torch.Tensor   # [pages, kv_heads, value width (head_dim unless the spec says otherwise), page_size]
+    group: int
+
+
+@dataclasses.dataclass
+class StateLayerCache:
+    """What a mixer with state of fixed size gets: per name a tensor [slots, *shape]."""
+    tensors: Dict[str, torch.Tensor]
+
+    def snapshot(self, state_slots: torch.Tensor) -> Dict[str, torch.Tensor]:
+        """Copies of the slots' rows (``state_slots`` int32 on the device, all >= 0)."""
+        idx = state_slots.to(torch.int64)
+        return {name: t.index_select(0, idx) for name, t in self.tensors.items()}
+
+    def restore(self, state_slots: torch.Tensor, saved: Dict[str, torch.Tensor]) -> None:
+        idx = state_slots.to(torch.int64)
+        for name, t in self.tensors.items():
+            t.index_copy_(0, idx, saved[name])
+
+    def zero_fresh(self, state_slots: torch.Tensor, fresh: torch.Tensor) -> None:
+        """Clears the slots of the step's sequences that start their request; both index arrays are the
+        step's own on the device, so a captured step can carry this."""
+        from ..ops import kernels as K
+        for t in self.tensors.values():
+            K.zero_fresh_rows(t, state_slots, fresh)
+
+
 @dataclasses.dataclass(frozen=True)
-class KVCacheSpec:
+class KVCacheSpec(PagedCacheSpec):
     """Keys and values per token, in pages.  ``window`` = keys looked back over, own included; 0 = all.
     ``value_dim``: the width of a value where it is not the key's (None: ``head_dim``); mixers with the same
-    heads, widths and window share a group of pages."""
+    heads, widths and window share a group of pages.
+
+    Layout per cache slot: K ``[pages, kv_heads, page_size, head_dim]`` and V transposed
+    ``[pages, kv_heads, value width, page_size]``, so that both Q.K and P.V read their contraction index
+    contiguously (the reference keeps ``[pages, page_size, kv_heads, head_dim]`` for both,
+    crates/prelude-core/src/scheduler/components/cache/manager.rs:286-329)."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
@@ -56,11 +128,32 @@ class KVCacheSpec:
     def v_dim(self) -> int:
         return self.head_dim if self.value_dim is None else self.value_dim
 
+    def bytes_per_token(self, element_size: int) -> int:
+        return self.num_kv_heads * (self.head_dim + self.v_dim) * element_size
+
+    def allocate(self, pages, page_size, dtype, device, group):
+        return KVLayerCache(torch.zeros((pages, self.num_kv_heads, page_size, self.head_dim), dtype=dtype, device=device),
+                            torch.zeros((pages, self.num_kv_heads, self.v_dim, page_size), dtype=dtype, device=device),
+                            group)
+
 
 @dataclasses.dataclass(frozen=True)
-class StateSpec:
+class StateSpec(SlotCacheSpec):
     """State of fixed size per request: name -> (shape, element type).  Zeroed when a request starts."""
     tensors: Tuple[Tuple[str, Tuple[int, ...], torch.dtype], ...]
+
+    def bytes_per_slot(self) -> int:
+        total = 0
+        for _name, shape, dt in self.tensors:
+            n = 1
+            for d in shape:
+                n *= int(d)
+            total += n * torch.empty((), dtype=dt).element_size()
+        return total
+
+    def allocate(self, slots, device):
+        return StateLayerCache({name: torch.zeros((slots, *shape), dtype=dt, device=device)
+                                for name, shape, dt in self.tensors})
 
 
 class Part:

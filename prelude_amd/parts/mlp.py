@@ -5,6 +5,10 @@ crates/prelude-core/src/models/qwen3.rs:383-448; silu(x) = x / (1 + e^-x) in
 Gate and up are one matrix [2I, H] here with rows alternating gate_j, up_j:
 one product yields each (gate_j, up_j) pair side by side, so the activation
 is the epilogue of that product for few rows and a pairwise kernel otherwise.
+The reference's Qwen3 is wired to SiLU whatever ``hidden_act`` says
+(qwen3.rs:429-447); the activation is a parameter here (SiLU, or GELU in its
+tanh form: crates/prelude-core/src/models/commons/activation.rs:3-25), one
+epilogue code in the same kernels.
 """
 from __future__ import annotations
 
@@ -19,9 +23,10 @@ class GatedMLP(FeedForward):
     GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
-        if activation != "silu":
-            raise PartError(f"gated_mlp: activation {activation!r} is not supported (silu)")
+        if activation not in K.GATE_ACTIVATIONS:
+            raise PartError(f"gated_mlp: activation {activation!r} is not one of {sorted(K.GATE_ACTIVATIONS)}")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation = activation
         self.gate_up = None
         self.down = None
 
@@ -37,4 +42,4 @@ class GatedMLP(FeedForward):
         self.down = K.prepare_weight(tensors["down_proj.weight"])
 
     def forward(self, x):
-        return K.linear(K.linear_silu_mul(x, self.gate_up), self.down, slices_ok=True)
+        return K.linear(K.linear_gated(x, self.gate_up, self.activation), self.down, slices_ok=True)

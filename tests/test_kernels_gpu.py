@@ -573,7 +573,26 @@ def test_qknorm_rope_refuses_bad_sizes(gpu):
 
 
 # ---- attention over the paged cache --------------------------------------------------------------
-def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None, kernel="generic", cut=None):
+def capped_plain_attention(q, k, v, scale, cap, window=None, q_offset=0):
+    """``pm.attention`` with the scaled scores bent to cap * tanh(s / cap) before the mask: the cap is no formula of
+    the reference's Qwen3 (no softcap there, crates/prelude-core/src/models/qwen3.rs:204), so its plain form lives here."""
+    sq, nh, hd = q.shape
+    sk, nkv, _ = k.shape
+    out = torch.empty_like(q)
+    qi = torch.arange(sq).reshape(sq, 1) + q_offset
+    ki = torch.arange(sk).reshape(1, sk)
+    allowed = ki <= qi
+    if window is not None:
+        allowed &= ki > qi - window
+    for h in range(nh):
+        s = (q[:, h] @ k[:, h // (nh // nkv)].T) * scale
+        s = (cap * torch.tanh(s / cap)).masked_fill(~allowed, float("-inf"))
+        out[:, h] = torch.softmax(s, dim=-1) @ v[:, h // (nh // nkv)]
+    return out
+
+
+def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=None, kernel="generic", cut=None,
+               softcap=0.0):
     """seqs: list of (context_len, q_len): the last q_len tokens of each context are this step's queries.
     Pages are handed out in a scrambled order.  Returns (engine output, plain output)."""
     g = torch.Generator().manual_seed(seed)
@@ -606,8 +625,12 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
         qs.append(q)
         seq_of += [i] * ql
         pos += list(range(ctx - ql, ctx))
-        refs.append(pm.attention(q.double(), k.double(), v.double(), 1.0 / math.sqrt(hd), window=window or None,
-                                 q_offset=ctx - ql))
+        if softcap:
+            refs.append(capped_plain_attention(q.double(), k.double(), v.double(), 1.0 / math.sqrt(hd), softcap,
+                                               window=window or None, q_offset=ctx - ql))
+        else:
+            refs.append(pm.attention(q.double(), k.double(), v.double(), 1.0 / math.sqrt(hd), window=window or None,
+                                     q_offset=ctx - ql))
     q = torch.cat(qs).to(dtype)
     if kernel == "mfma":
         i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
@@ -620,19 +643,19 @@ def paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=0, scale_trick=
         out = torch.full_like(qd, float("nan"))
         ctxs = i32([c for c, _ in seqs])
         K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, out, max([seqs[i][0] for i in dec], default=0),
-                             window, 1.0 / math.sqrt(hd))
+                             window, 1.0 / math.sqrt(hd), softcap=softcap)
         if dec and not pre:   # a step of single tokens: the kernels may count the sequences themselves, same bits
             again = torch.full_like(qd, float("nan"))
             K().attention_decode(qd, kd, vd, td, i32(dec), i32(cu), ctxs, again, max(seqs[i][0] for i in dec), window,
-                                 1.0 / math.sqrt(hd), every_seq=True)
+                                 1.0 / math.sqrt(hd), every_seq=True, softcap=softcap)
             assert torch.equal(again, out)
         K().attention_prefill(qd, kd, vd, td, i32(pre), i32(cu), ctxs, out, max([seqs[i][1] for i in pre], default=0),
                               window, 1.0 / math.sqrt(hd), cut=cut,
-                              min_prefix=min([seqs[i][0] - seqs[i][1] for i in pre], default=0))
+                              min_prefix=min([seqs[i][0] - seqs[i][1] for i in pre], default=0), softcap=softcap)
         return out, torch.cat(refs)
     out = K().attention_generic(q.to(gpu), kc.to(dtype).to(gpu), vc.to(dtype).to(gpu), table.to(gpu),
                                 torch.tensor(seq_of, dtype=torch.int32, device=gpu),
-                                torch.tensor(pos, dtype=torch.int32, device=gpu), window, 1.0 / math.sqrt(hd))
+                                torch.tensor(pos, dtype=torch.int32, device=gpu), window, 1.0 / math.sqrt(hd), softcap)
     return out, torch.cat(refs)
 
 
@@ -721,6 +744,64 @@ def test_mfma_attention_far_key_and_edges(gpu):
             out, ref = paged_case(gpu, torch.bfloat16, 2, 1, hd, 16, seqs, 20, scale_trick=trick2, kernel="mfma")
             close(out, ref, torch.bfloat16)
             assert (float(out[-1].float().abs().max()) > 50.0) == seen
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,window,cap", [(8, 2, 128, 16, 0, 2.0), (6, 2, 48, 8, 50, 0.7), (4, 4, 64, 32, 0, 30.0),
+                                                       (5, 1, 40, 4, 0, 1.0)])
+def test_attention_with_capped_scores(gpu, nh, nkv, hd, page, window, cap):
+    """A cap on the scores (cap * tanh(scaled score / cap) before the mask and the softmax) in every attention
+    kernel: generic (both precisions), matrix-core decode with its splits, prefill staged and not.  Queries are
+    made long so that most scores lie beyond the cap; without the cap the outputs differ by far more than the bound."""
+    def trick(i, q, k, v):
+        q *= 3.0
+
+    seqs = [(70, 70), (130, 1), (33, 7), (1, 1), (700, 1), (300, 150), (513, 1)]
+    for dtype in DT:
+        out, ref = paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=31, scale_trick=trick, softcap=cap)
+        close(out, ref, dtype, f32=3e-6)
+        plain, other = paged_case(gpu, dtype, nh, nkv, hd, page, seqs, window, seed=31, scale_trick=trick)
+        assert float((other - ref).abs().max()) > 20 * tol(dtype, ref) or cap > 10
+    if K().mfma_attention_supported(hd, page):
+        out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=31, scale_trick=trick,
+                              kernel="mfma", softcap=cap)
+        assert not bool(torch.isnan(out).any())
+        close(out, ref, torch.bfloat16)
+        if page >= 8:
+            direct, _ = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, window, seed=31, scale_trick=trick,
+                                   kernel="mfma", softcap=cap, cut=(-1, -1, -1, 0))
+            close(direct, ref, torch.bfloat16)
+    from prelude_amd._native import NativeError
+    with pytest.raises(NativeError, match="negative"):
+        paged_case(gpu, torch.float32, nh, nkv, hd, page, [(5, 1)], 0, softcap=-1.0)
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+def test_gated_activation_in_every_epilogue(gpu, activation):
+    """act(gate) * up with the activation chosen by a code: the pairwise kernel (both precisions) and the gated
+    epilogues of the three products, each against the library's own function of that name in 64-bit."""
+    import torch.nn.functional as F
+    act = (lambda x: F.silu(x)) if activation == "silu" else (lambda x: F.gelu(x, approximate="tanh"))
+    for dtype in DT:
+        for tokens, inter in ((5, 160), (3, 7), (37, 1000)):
+            gu = rnd(tokens, 2 * inter, dtype=dtype, scale=2.0)
+            ref = act(gu[:, 0::2].double()) * gu[:, 1::2].double()
+            close(K().silu_mul(gu.to(gpu), activation), ref, dtype, f32=3e-6)
+    n, k = 1000, 2560
+    w = rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05)
+    tiles = K().pack_tiles(w.to(gpu))
+    lw = K().LinearWeight(w.to(gpu), tiles)
+    for m, product in ((8, K().gemm_skinny), (40, K().gemm_mid), (200, K().gemm_tall)):
+        x = rnd(m, k, dtype=torch.bfloat16, seed=m)
+        g = x.double() @ w.double().T
+        ref = act(g[:, 0::2]) * g[:, 1::2]
+        close(product(x.to(gpu), tiles, silu_mul_epilogue=True, activation=activation), ref, torch.bfloat16)
+        close(K().linear_gated(x.to(gpu), lw, activation), ref, torch.bfloat16)
+    x = rnd(600, k, dtype=torch.bfloat16, seed=9)          # many rows: the library's product and the pairwise kernel
+    g = x.double() @ w.double().T
+    close(K().linear_gated(x.to(gpu), lw, activation), act(g[:, 0::2]) * g[:, 1::2], torch.bfloat16)
+    from prelude_amd._native import NativeError
+    with pytest.raises(NativeError, match="not one of"):
+        K().silu_mul(rnd(2, 8).to(gpu), "relu")
 
 
 @pytest.mark.parametrize("hd,page,window", [(64, 16, 0), (128, 16, 0), (64, 8, 40), (32, 32, 70), (128, 64, 33)])
