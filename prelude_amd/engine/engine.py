@@ -156,7 +156,7 @@ class Engine:
         from .graph import portion_tokens_worth_a_graph
         if not (self.config.hip_graph and self.model.graph_safe_portions and self.dtype == torch.bfloat16):
             return 0
-        return portion_tokens_worth_a_graph(self.model.matrix_elements(), len(self.model.spec.order), 2,
+        return portion_tokens_worth_a_graph(self.model.matrix_elements(), self.model.launches_per_step(), 2,
                                             int(self.config.hip_graph_portion_tokens))
 
     def _cache_bytes(self, tokens: int, specs) -> int:

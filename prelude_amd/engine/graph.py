@@ -47,22 +47,23 @@ from typing import Sequence
 import torch
 
 
-# What a step with portions is taken to cost, to tell where its capture pays: the host some ten launches a layer
-# at 8 us each; the device the weights streamed once at 4 TB/s or, beyond a few tokens, two operations per matrix
-# element and token at 0.4 PFLOP/s (what the library's products reach at some hundred rows).
-HOST_SECONDS_PER_LAYER = 10 * 8e-6
+# What a step with portions is taken to cost, to tell where its capture pays: the host 8 us for each launch the
+# model's parts count for themselves (``Part.LAUNCHES``); the device the weights streamed once at 4 TB/s or, beyond
+# a few tokens, two operations per matrix element and token at 0.4 PFLOP/s (what the library's products reach at
+# some hundred rows).
+HOST_SECONDS_PER_LAUNCH = 8e-6
 STREAM_BYTES_PER_SECOND = 4e12
 PRODUCT_OPS_PER_SECOND = 0.4e15
 
 
-def portion_tokens_worth_a_graph(matrix_elements: int, layers: int, element_bytes: int, cap: int) -> int:
+def portion_tokens_worth_a_graph(matrix_elements: int, launches: int, element_bytes: int, cap: int) -> int:
     """Up to how many tokens a step with portions is replayed from a graph: as long as the host's launches are
     estimated to take longer than the device's work, and never beyond ``cap``.  (Measured: a 28-layer model of
     0.6 G elements takes 2.04 instead of 2.51 ms for a prompt of 128 tokens; a 36-layer model of 4 G elements is
     bound by the device at 512 tokens, 7.3 ms either way, and gains nothing from the capture.)"""
     if cap <= 0 or matrix_elements <= 0:
         return max(cap, 0)
-    host = layers * HOST_SECONDS_PER_LAYER
+    host = launches * HOST_SECONDS_PER_LAUNCH
     if matrix_elements * element_bytes / STREAM_BYTES_PER_SECOND >= host:
         return 0
     return int(min(cap, host * PRODUCT_OPS_PER_SECOND / (2.0 * matrix_elements)))

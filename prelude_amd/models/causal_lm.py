@@ -122,6 +122,15 @@ class CausalLM:
                     total += n
         return total
 
+    def launches_per_step(self) -> int:
+        """Kernel launches of one step, about: every run's block by its parts' own counts, and the embedding, the
+        final norm and the head."""
+        total = self.embedding.LAUNCHES + self.final_norm.LAUNCHES + self.head.LAUNCHES
+        for r in self.spec.order:
+            b = self.blocks[r.layer]
+            total += b.launches() if hasattr(b, "launches") else 1
+        return total
+
     # ---- what the cache manager must provide ------------------------------
     @property
     def needs_state(self) -> bool:

@@ -22,6 +22,7 @@ from .base import MATRIX, NORM, VECTOR, KVCacheSpec, Mixer, PartError, TensorReq
 
 @register_part("mixer", "gqa_attention")
 class GQAAttention(Mixer):
+    LAUNCHES = 4   # merged projection, norm + rotation + cache write, attention, output projection
     GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, norm_eps: float = 1e-6,

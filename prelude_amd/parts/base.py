@@ -171,6 +171,9 @@ class Part:
     # positions the portions start at, the pages and the state slots are (these it reads on the device).  False
     # by default: a part has to say so itself.
     GRAPH_SAFE_PORTIONS = False
+    # Kernel launches one ``forward`` of this part costs the host, about: what a model's parts add up to says up
+    # to how many tokens a step with portions is bound by the host's launches and worth replaying from a graph.
+    LAUNCHES = 1
 
     def tensors(self) -> Dict[str, TensorReq]:
         """Local tensor name -> what is required of it."""
@@ -224,9 +227,14 @@ class PositionEncoding(Part):
 class Block(Part):
     """An arrangement of parts.  ``SLOTS`` names the sub-parts it is built from: slot -> category."""
     SLOTS: Dict[str, str] = {}
+    LAUNCHES = 0   # of the arrangement itself; its sub-parts count their own
 
     def forward(self, hidden, residual, step, cache, write_cache: bool = True):
         raise NotImplementedError
+
+    def launches(self) -> int:
+        """Kernel launches of one run of this block: its own and those of the parts in its slots."""
+        return self.LAUNCHES + sum(getattr(self, slot).LAUNCHES for slot in self.SLOTS)
 
 
 # ---------------------------------------------------------------------------

@@ -20,6 +20,7 @@ from .base import MATRIX, FeedForward, PartError, TensorReq, register_part
 
 @register_part("ffn", "gated_mlp")
 class GatedMLP(FeedForward):
+    LAUNCHES = 3   # gate and up in one product, activation * up, down
     GRAPH_SAFE_PORTIONS = True   # launches follow the step's shape alone; tokens, positions and pages are read on the device
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):

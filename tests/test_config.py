@@ -104,11 +104,11 @@ def test_where_a_step_with_portions_is_worth_a_graph():
     matrix elements, none where streaming the weights alone takes longer than the launches; never beyond the
     configured number, and the matrix elements are counted from the model's own tensors."""
     from prelude_amd.engine.graph import portion_tokens_worth_a_graph as worth
-    assert 600 < worth(int(0.6e9), 28, 2, 1024) < 900
-    assert worth(int(0.6e9), 28, 2, 256) == 256
-    assert 100 < worth(int(4.0e9), 36, 2, 1024) < 200
-    assert worth(int(8.2e9), 36, 2, 1024) == 0
-    assert worth(int(0.6e9), 28, 2, 0) == 0
+    assert 600 < worth(int(0.6e9), 28 * 9 + 3, 2, 1024) < 900
+    assert worth(int(0.6e9), 28 * 9 + 3, 2, 256) == 256
+    assert 100 < worth(int(4.0e9), 36 * 9 + 3, 2, 1024) < 200
+    assert worth(int(8.2e9), 36 * 9 + 3, 2, 1024) == 0
+    assert worth(int(0.6e9), 28 * 9 + 3, 2, 0) == 0
     from prelude_amd.models.causal_lm import CausalLM
     from prelude_amd.config import resolve_architecture
     for cfg in (pm.tiny_config_a(), pm.tiny_config_b(), pm.tiny_config_c()):
@@ -118,3 +118,5 @@ def test_where_a_step_with_portions_is_worth_a_graph():
         want = sum(a * b for name, (a, *rest) in shapes.items() for b in rest
                    if name != "model.embed_tokens.weight" or cfg["tie_word_embeddings"])
         assert model.matrix_elements() == want and model.graph_safe_portions
+        # the launches are the parts' own counts: two norms, a mixer of four and a feed-forward of three a layer
+        assert model.launches_per_step() == 9 * cfg["num_hidden_layers"] + 3
