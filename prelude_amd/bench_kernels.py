@@ -1,6 +1,6 @@
 """Times single kernels against their rooflines on one MI355X.
 
-    python -m prelude_amd.bench_kernels [stream] [gemm] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
+    python -m prelude_amd.bench_kernels [stream] [gemm] [tall] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
 
 Each line gives the kernel's time (device events around repeated launches,
 operands rotated over copies larger than the caches where the kernel streams
@@ -102,6 +102,32 @@ def bench_gemm(dev, shape) -> None:
         del rows, tiles, weights_of
 
 
+def bench_tall(dev, shape) -> None:
+    """Products of 129 to 1,024 rows: the kernel tiled both ways (``gemm_tall``: in four slices of K for o and down,
+    which the norm after them adds; with the activation in its epilogue for gate_up) beside the library (with
+    its separate activation kernel for gate_up), weights rotated over 600 MB so that they come from memory.  Which
+    of the two a step takes is ``ops.kernels.linear``'s choice, made from whole prompt steps, not from these."""
+    h, inter, nh, nkv, hd, vocab = shape
+    weights = {"qkv": ((nh + 2 * nkv) * hd, h), "o": (h, nh * hd), "gate_up (act*up)": (2 * inter, h), "down": (h, inter)}
+    for name, (n, k) in weights.items():
+        copies = max(2, int(600e6 // (n * k * 2)))
+        rows = [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        tiles = [K.pack_tiles(w) for w in rows]
+        gated = name.startswith("gate_up")
+        slices = K._tall_slices(k) if name in ("o", "down") else 1
+        for m in (129, 192, 256, 384, 512, 1024):
+            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            flops = 2.0 * m * n * k
+            us = timeit(lambda i: K.gemm_tall(x, tiles[i], silu_mul_epilogue=gated, slices=slices), copies, iters=20)
+            line(f"gemm {name} [{n}x{k}] M={m} tall" + (f" in {slices} slices" if slices > 1 else ""), us, flops=flops)
+            if gated:
+                us = timeit(lambda i: K.silu_mul(K.gemm_library(x, rows[i])), copies, iters=20)
+            else:
+                us = timeit(lambda i: K.gemm_library(x, rows[i]), copies, iters=20)
+            line(f"gemm {name} [{n}x{k}] M={m} library" + (" + act*up" if gated else ""), us, flops=flops)
+        del rows, tiles
+
+
 def bench_decode(dev, shape, page: int = 16) -> None:
     _, _, nh, nkv, hd, _ = shape
     for batch, ctx in ((1, 4096), (8, 512), (8, 4096), (8, 32768), (64, 4096)):
@@ -174,7 +200,7 @@ def bench_sampling(dev, shape) -> None:
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
-    ap.add_argument("what", nargs="*", help="stream, gemm, decode, prefill, elementwise, sampling (default: all)")
+    ap.add_argument("what", nargs="*", help="stream, gemm, tall, decode, prefill, elementwise, sampling (default: all)")
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -182,11 +208,11 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     shape = SHAPES[args.shape]
-    todo = args.what or ["stream", "gemm", "decode", "prefill", "elementwise", "sampling"]
+    todo = args.what or ["stream", "gemm", "tall", "decode", "prefill", "elementwise", "sampling"]
     print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
           f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
     for name in todo:
-        {"stream": bench_stream, "gemm": bench_gemm, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
+        {"stream": bench_stream, "gemm": bench_gemm, "tall": bench_tall, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
          "sampling": bench_sampling}[name](dev, shape)
     return 0
 

@@ -439,6 +439,27 @@ def test_drawn_products(gpu, seed):
         parts = K().gemm_mid(x3d, tiles, bd, slices=c, waves=waves).parts
         err = float((parts.double().sum(0).cpu() - ref3 - b.double()).abs().max())
         assert err <= tol(torch.float32, ref3, f32=2e-5), f"{what}, rows {m3}, {waves} wavefronts, {c} slices: max error {err:.3e}"
+    # the product tiled both ways, at a drawn number of rows, shape of workgroup, activation and number of slices
+    m4 = int(rng.choice([1, 129, 192, 256, 257, int(rng.integers(1, 700))]))
+    x4 = rnd(m4, k, dtype=torch.bfloat16, seed=seed + 7)
+    x4d = x4.to(gpu)
+    ref4 = x4.double() @ w.double().T
+    shape = [(0, 0), (4, 2), (4, 3), (8, 2), (8, 3)][int(rng.integers(0, 5))]
+    activation = ["silu", "gelu_tanh"][int(rng.integers(0, 2))]
+    gate4 = pm.silu(ref4[:, 0::2]) if activation == "silu" else torch.nn.functional.gelu(ref4[:, 0::2], approximate="tanh")
+    for name, got, want in (
+            ("tall", K().gemm_tall(x4d, tiles, shape=shape), ref4),
+            ("tall, bias", K().gemm_tall(x4d, tiles, bd, shape=shape), ref4 + b.double()),
+            (f"tall, {activation}*up", K().gemm_tall(x4d, tiles, silu_mul_epilogue=True, shape=shape, activation=activation),
+             gate4 * ref4[:, 1::2])):
+        assert tuple(got.shape) == tuple(want.shape), f"{what}, rows {m4}, shape {shape}, {name}: shape {tuple(got.shape)}"
+        err = float((got.double().cpu() - want).abs().max())
+        assert err <= tol(torch.bfloat16, want), f"{what}, rows {m4}, shape {shape}, {name}: max error {err:.3e}"
+    if cuts:
+        c = int(rng.choice(cuts))
+        parts = K().gemm_tall(x4d, tiles, bd, slices=c, shape=shape).parts
+        err = float((parts.double().sum(0).cpu() - ref4 - b.double()).abs().max())
+        assert err <= tol(torch.float32, ref4, f32=2e-5), f"{what}, rows {m4}, shape {shape}, {c} slices: max error {err:.3e}"
     # many rows through the dispatcher (the library product beyond the streaming kernel's rows)
     m2 = int(rng.integers(65, 400))
     x2 = rnd(m2, k, dtype=torch.bfloat16, seed=seed + 3)

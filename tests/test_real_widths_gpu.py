@@ -101,6 +101,30 @@ def test_twenty_requests_decode_together(gpu):
     assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
 
 
+@pytest.mark.parametrize("batch", [33, 64, 100, 128])
+def test_many_requests_decode_together(gpu, batch):
+    """Decode steps of 33 to 128 requests at the real widths: the products of 17 to 128 rows (X through LDS, the
+    narrow ones in slices of K that the norm adds, the gated one with its activation in the epilogue), the head at
+    up to 64 rows through the same kernel and beyond through the library, the decode attention over that many
+    sequences; up to 64 requests are replayed from a graph after the first step, more are launched directly."""
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref, _ = wide_model()
+    r = TraceRunner(folder, "bfloat16", batch * 112, page_size=16)
+    starts = [2 + (7 * i) % 88 for i in range(batch)]
+    for i, s in enumerate(starts):
+        r.step([{"id": f"r{i}", "tokens": toks[:s], "want": []}])
+    rows = [[] for _ in starts]
+    steps = 4
+    for k in range(steps):
+        out = r.step([{"id": f"r{i}", "tokens": [toks[s + k]], "want": [0]} for i, s in enumerate(starts)])
+        for i in range(batch):
+            rows[i].append(out[i:i + 1])
+    for i, s in enumerate(starts):
+        check(np.concatenate(rows[i]), ref[s:s + steps], "bfloat16", f"request {i} of {batch} from position {s}")
+    r.step([], [f"r{i}" for i in range(batch)])
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
 def test_greedy_generation_at_real_widths(gpu):
     from prelude_amd import LLM
     folder, toks, _, w64 = wide_model()
