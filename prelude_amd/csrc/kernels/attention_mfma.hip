@@ -445,7 +445,7 @@ __device__ __forceinline__ void fused_load_q(const FusedQkv& f, const bf16* qrow
 }
 
 template <int HD, bool FUSED, int WAVES>
-__global__ __launch_bounds__(WAVES* kWave, 3) void attn_decode_kernel(
+__global__ __launch_bounds__(WAVES* kWave, WAVES == 8 ? 1 : 3) void attn_decode_kernel(
     const bf16* __restrict__ q, const bf16* kc, const bf16* vc,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
@@ -453,8 +453,10 @@ __global__ __launch_bounds__(WAVES* kWave, 3) void attn_decode_kernel(
     int split_keys, int max_splits, FusedQkv fq, int contiguous) {
   constexpr int OT = HD / 16;
   constexpr int KS = (HD + 31) / 32;
-  __shared__ float lds_o[WAVES][16][HD + 1];
-  __shared__ float lds_ml[WAVES][16][2];
+  // eight wavefronts (grids of at most a workgroup a compute unit, groups of up to eight heads) keep eight query rows
+  constexpr int QR = WAVES == 8 ? 8 : 16;
+  __shared__ float lds_o[WAVES][QR][HD + 1];
+  __shared__ float lds_ml[WAVES][QR][2];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int group = nh / nkv;
@@ -522,14 +524,16 @@ __global__ __launch_bounds__(WAVES* kWave, 3) void attn_decode_kernel(
   }
   // merge the wavefronts through LDS; maxima leave in the log2 domain (raw maximum times c)
   const float l_wave = st[0].l[0];
-  if (g == 0) {
+  if (g == 0 && r < QR) {
     lds_ml[wave][r][0] = st[0].reference();
     lds_ml[wave][r][1] = l_wave;
   }
+  if (r < QR) {
 #pragma unroll
-  for (int t = 0; t < OT; ++t)
+    for (int t = 0; t < OT; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_o[wave][r][16 * t + 4 * g + i] = st[0].o[t][i];
+      for (int i = 0; i < 4; ++i) lds_o[wave][r][16 * t + 4 * g + i] = st[0].o[t][i];
+  }
   __syncthreads();
   const int nq = group - qt * 16 < 16 ? group - qt * 16 : 16;
   for (int e = threadIdx.x; e < nq * HD; e += blockDim.x) {
@@ -984,8 +988,16 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   // measured 1 to 2 % slower with two.  With two wavefronts a split's steps are added in another order (wavefront w
   // takes the steps w, w + 2, .. instead of w, w + 4, ..), so a token's sums can differ in their last bits between
   // steps whose grids fall on either side of these limits; what else is in the batch changes nothing beyond that.
+  // A grid of at most one workgroup a compute unit (one sequence of 4,096 keys: 128) runs with eight, a step of
+  // 32 keys each: batch 1 of a 4B model 2.518 -> 2.499 ms a step, batch 2 (256 workgroups) level; with eight up to
+  // 512 workgroups batch 3 and 4 lose 4 %.
   const bool two_wavefronts = total > 768 && total <= 1536;
-  if (two_wavefronts) {
+  const bool eight_wavefronts = total <= 256 && nh / nkv <= 8 && split_keys == 256;
+  if (eight_wavefronts) {
+    hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 8>), grid, dim3(8 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
+                       (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
+                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);
+  } else if (two_wavefronts) {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 2>), grid, dim3(2 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
                        part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);

@@ -1024,20 +1024,22 @@ def test_mfma_attention_batch_and_page_independence(gpu):
 
 
 def test_decode_attention_on_either_side_of_the_grid_limits(gpu):
-    """The same sequence alone (128 workgroups: four wavefronts a workgroup), among eight (1,024: two) and among
-    thirteen (1,664: four again).  Which keys a split sums is the same in all three; the order in which a split's
-    steps are added is not, so the results agree to rounding, not to the bit, across the limits -- and to the bit
-    on the same side of them."""
+    """The same sequence alone and beside one other (128 and 256 workgroups: eight wavefronts a workgroup), among
+    eight (1,024: two), among six and among thirteen (768 and 1,664: four).  Which keys a split sums is the same in
+    all of them; the order in which a split's steps are added is not, so the results agree to rounding, not to the
+    bit, across the limits -- and to the bit on the same side of them."""
     first = (4096, 1)
     outs = []
-    for others in (0, 7, 12):
+    for others in (0, 1, 7, 5, 12):
         seqs = [first] + [(4000 - 50 * i, 1) for i in range(others)]
         out, ref = paged_case(gpu, torch.bfloat16, 32, 8, 128, 16, seqs, 0, seed=21, kernel="mfma")
         close(out, ref, torch.bfloat16)
         outs.append((out[0].double().cpu(), ref[0]))
-    (a, ref), (b, _), (c, _) = outs
-    assert torch.equal(a, c)                                  # four wavefronts both times
-    assert float((a - b).abs().max()) <= tol(torch.bfloat16, ref)
+    (a, ref), (a2, _), (b, _), (c, _), (c2, _) = outs
+    assert torch.equal(a, a2)                                 # eight wavefronts both times
+    assert torch.equal(c, c2)                                 # four wavefronts both times
+    for x, y in ((a, b), (a, c), (b, c)):
+        assert float((x - y).abs().max()) <= tol(torch.bfloat16, ref)
 
 
 @pytest.mark.parametrize("nh,nkv,hd,page,window,norm,ctxs", [
