@@ -1087,17 +1087,42 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // and need no pairing, which doubles the workgroups there are to hand out
   const bool level = min_prefix >= max_q_len;
   const bool wide_ok = can_stage && group % (gt_best * 2) == 0;   // eight wavefronts: two groups of gt_best heads
-  if (wide_ok && workgroups(paired, gt_best, 2) >= enough && tiles > 8) {
+  const int gt_half = gt_best >= 2 ? gt_best / 2 : 1;
+  const bool half_ok = can_stage && gt_best >= 2 && group % (gt_half * 2) == 0;
+  // Pairs are workgroups of one length, so they come in rounds, and a last round that is half empty costs as much
+  // as a full one: pairs pay where the rounds are full (or many).  Unpaired, the tiles are of every length from one
+  // block to the whole context, the longest are handed out first, and from one and a half workgroups a compute
+  // unit on they balance out by themselves.  Measured, 32 heads over 8 of 128: 1,536 tokens as 384 pairs of a head
+  // a wavefront 47.2 us, unpaired with eight wavefronts 36.5; 3,072 tokens as 384 pairs 134.3, unpaired with two
+  // heads a wavefront 105.0; 2,048 and 4,096 tokens, whose pairs are one full round, 53.0 and 144.5 paired against
+  // 55.0 and 150.1.
+  // (7,168 tokens, 448 pairs: 466 against 437 us unpaired; three prompts of 1,024, 192 pairs: 50.4 against 57.2 --
+  // short tiles carry a workgroup's fixed cost less well, so one round that is three quarters full still counts)
+  auto full_rounds = [&](long w, long slots) {
+    return (w >= slots && (w % slots == 0 || w >= 4 * slots)) || (tiles <= 16 && 4 * w >= 3 * slots && w <= slots);
+  };
+  const long spread = enough * 3 / 2;
+  if (wide_ok && tiles > 8 && full_rounds(workgroups(1, gt_best, 2), enough)) {
     // the most work per staged key that still gives every compute unit a workgroup (measured at head_dim 128,
     // 32 heads over 8: 4,096 tokens 171 against 186 us, 8,192 tokens 624 against 648); not for many short prompts,
     // whose workgroups are over after a few blocks (16 prompts of 512 tokens: 66 against 70 us with four
     // wavefronts a workgroup, 32 of 256: 51 against 60)
     hw = 2;
+  } else if (wide_ok && tiles > 8 && !level && workgroups(0, gt_best, 2) >= spread) {
+    paired = 0, hw = 2;
   } else if (level && workgroups(0, gt_best, wide_ok ? 2 : 1) >= enough) {
     paired = 0;   // 2,048 tokens behind 6,144: 297 against 342 us
     hw = wide_ok ? 2 : 1;
   } else if (level && can_stage && group % 2 == 0 && workgroups(0, 1, 2) >= enough) {
     paired = 0, gt = 1, hw = 2;   // 1,024 tokens behind 7,168: 205 against 293 us
+  } else if (half_ok && tiles > 8 && full_rounds(workgroups(1, gt_half, 2), enough)) {
+    gt = gt_half, hw = 2;         // 2,048 tokens: 256 pairs of eight wavefronts, a head each
+  } else if (half_ok && tiles > 8 && workgroups(0, gt_half, 2) >= spread) {
+    paired = 0, gt = gt_half, hw = 2;
+  } else if (half_ok && workgroups(0, gt_half, 2) == enough) {
+    // exactly one workgroup of eight wavefronts a compute unit, two wavefronts a SIMD and one round (two prompts
+    // of 512 tokens: 16.0 us against 17.7 as pairs of four wavefronts)
+    paired = 0, gt = gt_half, hw = 2;
   } else {
     if (workgroups(paired, gt) < enough) {
       if (gt > 1 && workgroups(paired, 1) >= enough) {
@@ -1111,10 +1136,15 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
     }
     // one workgroup per compute unit is one wavefront per SIMD, which waits for every one of its own steps: then
     // rather eight wavefronts a workgroup, half of them on the other heads (measured at 2,048 tokens: 69 against 77 us)
-    if (can_stage && workgroups(paired, gt) >= enough && workgroups(paired, gt) < 2 * enough && gt >= 2 && gt == gt_best) {
+    // (up to one and a quarter: six prompts of 512 tokens, 384 pairs, 35.6 us as they are and 40.7 with eight wavefronts)
+    if (can_stage && workgroups(paired, gt) >= enough && workgroups(paired, gt) <= enough * 5 / 4 && gt >= 2 && gt == gt_best) {
       gt /= 2;
       hw = 2;
     }
+    // pairs in rounds that are not full: unpaired, if that gives workgroups enough to balance out
+    // (prompts of up to 512 tokens are over too soon for rounds to form: twelve of 512 tokens 60.3 us in pairs, 64.7 without)
+    if (paired && tiles > 8 && !full_rounds(workgroups(1, gt, hw), hw == 2 ? enough : 2 * enough) && workgroups(0, gt, hw) >= spread)
+      paired = 0;
   }
   // keys staged in LDS for pages of 8 keys or more; pages of 4 go to the kernel that reads them itself
   bool staged = can_stage;
