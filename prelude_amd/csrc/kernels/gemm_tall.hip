@@ -232,28 +232,32 @@ using namespace pa;
 // The workgroup's shape the launcher takes for a product of m rows by an [n, k] weight in `slices` slices:
 // out[0] = tiles of 16 rows of X a workgroup (4 or 8), out[1] = tiles of 16 rows of W a wavefront (2 or 3).
 //
-// Measured over the four shapes at the widths of 4B, 8B and 32B models (129 to 1,024 rows); the shapes lie within a
-// tenth or two of one another, and which is ahead follows how the weight's tiles and the rows divide:
-//   - up to 192 rows, tiles of 64 rows (128 would be half empty) and 8 tiles of W a workgroup;
-//   - beyond, narrow weights (up to 3,072 rows: the o and down projections of a 2,560 wide model) keep tiles of
-//     64 rows, which give them workgroups enough, with 12 tiles of W; weights whose tiles divide by 32 but not by
-//     12 without a rest worth mentioning (4,096 rows) take 128 x 128; everything else 128 rows x 12 tiles, the
-//     shape that moves the fewest bytes into the compute units.
-// With the loop's products and LDS traffic taken out the loads alone take four fifths of the kernel's time (a
-// [19456, 2560] weight at 256 rows: 53 us as 64 x 128 tiles, which move 600 MB, 37 us as 128 x 192 tiles, which move
-// 330 MB; the kernel 55 and 47), at any depth of the ring: some 9 to 11 TB/s into all compute units together, of
-// which a tenth comes from memory (the L2 counters: every byte of W once) and the rest from L2.
+// The kernel's time follows the bytes its workgroups pull in (with the loop's products and LDS traffic taken out the
+// loads alone take four fifths of it: a [19456, 2560] weight at 256 rows 53 us as 64 x 128 tiles, which move 600 MB,
+// 37 us as 128 x 192 tiles, which move 330 MB; the kernel 55 and 47; some 9 to 11 TB/s into all compute units
+// together, of which a tenth comes from memory, every byte of W once, and the rest from L2), and a compute unit
+// pulls at one rate with one workgroup on it and at 1.4 times that with two (the same product at 512 rows, twice
+// the workgroups: 70 us).  So a shape is priced at the bytes a step of one workgroup brings in, times what the
+// fullest compute unit has to work off: 1 for one workgroup, 1.43 for two at once, and so on in rounds of two; the
+// cheapest shape is taken.  Measured over the four shapes at the widths of 0.6B to 32B models, 129 to 512 rows, the
+// shape so chosen is the fastest or within a twentieth of it: small weights keep 64 x 128 at every number of rows
+// ([6144, 1024] at 256 rows 11.7 us against 21.5 as 128 x 192), 384 rows of a large one take 128 x 128 ([19456, 2560]
+// 54.8 against 68.8, [5120, 17408] in four slices 87.5 against 113.8), 256 and 512 rows 128 x 192.
+static double tall_price(int mt, int nt, int m, int tiles, int slices) {
+  const long row_tiles = (m + 16 * mt - 1) / (16 * mt), col_groups = (tiles + kTallWaves * nt - 1) / (kTallWaves * nt);
+  const long on_the_fullest = (row_tiles * col_groups * slices + 255) / 256;
+  const double rounds = 1.43 * (double)(on_the_fullest / 2) + (double)(on_the_fullest % 2);
+  return (16.0 * mt * 128.0 + 2048.0 * kTallWaves * nt) * rounds;
+}
+
 extern "C" void pa_gemm_tall_shape(int m, int n, int k, int slices, int* out) {
   (void)k;
   const int tiles = (n + 15) / 16;
-  if (m <= 192) {
-    out[0] = 4, out[1] = 2;
-  } else if (slices > 1 && n <= 3072) {
-    out[0] = 4, out[1] = 3;
-  } else if (slices > 1 && tiles % 32 == 0 && tiles % 12 != 0 && n <= 4096) {
-    out[0] = 8, out[1] = 2;
-  } else {
-    out[0] = 8, out[1] = 3;
+  static const int shapes[4][2] = {{8, 3}, {8, 2}, {4, 3}, {4, 2}};   // at equal price the larger tile
+  double best = 0.0;
+  for (int i = 0; i < 4; ++i) {
+    const double price = tall_price(shapes[i][0], shapes[i][1], m, tiles, slices < 1 ? 1 : slices);
+    if (i == 0 || price < best) best = price, out[0] = shapes[i][0], out[1] = shapes[i][1];
   }
 }
 

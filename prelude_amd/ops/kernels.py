@@ -398,7 +398,10 @@ MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns,
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
 MID_SLICED_LONG_K = 8192
-MID_SLICED_SHORT_ROWS = 24     # ... and up to here small weights with shorter rows stay with the streaming kernel
+MID_SLICED_SHORT_ROWS = 24     # ... and up to here small weights with shorter rows stay with the streaming kernel:
+MID_SLICED_SHORT_K = 4096      #     rows of up to this many columns,
+MID_SLICED_SHORT_ELEMENTS = 1 << 24   # weights of up to this many elements
+MID_SLICED_MIN_ROWS_LONG = 8   # rows of TILED_LONG_ROWS columns or more: in slices from here on
 # A reader that wants a tensor gets the slices too, added by a kernel of their own, where the pair is still ahead of
 # the library: large weights ([10240, 5120] inside a captured step: 24.2 to 26.9 us at 24 to 64 rows against 28.4 to
 # 32.4, 33.7 and 38.6 at 96 and 128 rows against 36.1 and 40.4; [6144, 4096] and [6144, 2560] are within a
@@ -493,7 +496,7 @@ def gemm_tall(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = 
 TALL_MAX_ROWS = 256
 TALL_SLICED_MIN_N = 4096       # outputs at least this wide go to it in slices for the norm ...
 TALL_HUGE_MAX_ROWS = 576       # ... and weights of TALL_HUGE_ELEMENTS up to this many rows
-TALL_HUGE_ELEMENTS = 100 << 20
+TALL_HUGE_ELEMENTS = 80 << 20        # [5120, 17408] at 384 and 512 rows: 127 and 134 us against the library's 141 and 175
 TALL_GATED_MAX_K = 4096
 TALL_PRODUCTS = 3              # ``set_tall_products``: which of these products ``gemm_tall`` takes (measurements):
 #                                1 in slices for a reader of slices, 2 the gated one
@@ -570,16 +573,26 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     # the other way round), from 17 rows on everywhere
     sliced = (MID_PRODUCTS and slices_ok and tiles is not None and k % 8 == 0 and n % 4 == 0 and m <= GEMM_MID_MAX_ROWS
               and out_dtype in (None, torch.bfloat16)
-              and (m > SKINNY_MAX_ROWS or (m >= MID_SLICED_MIN_ROWS and k >= MID_SLICED_LONG_K))
+              and (m > SKINNY_MAX_ROWS or (m >= MID_SLICED_MIN_ROWS and k >= MID_SLICED_LONG_K)
+                   # rows of 16,384 columns and more from 8 rows on ([5120, 17408] with the norm behind it 40.0
+                   # against 42.6 us at 8 rows, [5120, 25600] 54.3 against 57.9; level at 4 rows)
+                   or (m >= MID_SLICED_MIN_ROWS_LONG and k >= TILED_LONG_ROWS))
               # just beyond 16 rows a small weight with short rows is still the streaming kernel's (inside a captured
               # step, with the norm that reads it: [4096, 4096] 13.3 and 14.4 us at 17 and 24 rows against 16.8 in
-              # slices, [2560, 4096] 12.5 and 13.7 against 13.3 and 13.9; from 32 rows on the slices are ahead)
-              and not (m <= MID_SLICED_SHORT_ROWS and k < MID_SLICED_LONG_K and _tiled_beyond_16(m, n, k)))
+              # slices, [2560, 4096] 12.5 and 13.7 against 13.3 and 13.9; from 32 rows on the slices are ahead; a
+              # [5120, 5120] weight is ahead in slices already, 17.5 against 21.2 us at 24 rows)
+              and not (m <= MID_SLICED_SHORT_ROWS and k <= MID_SLICED_SHORT_K and n * k <= MID_SLICED_SHORT_ELEMENTS
+                       and _tiled_beyond_16(m, n, k)))
     if sliced:
         s = gemm_mid_slices(n, k)
         if s >= MID_MIN_SLICES:
             return gemm_mid(x, tiles, bias, slices=s)
     if m <= SKINNY_MAX_ROWS and k % 8 == 0:
+        # a large weight whose reader wants a tensor, 9 to 16 rows: [10240, 5120] 22.5 us against the streaming
+        # kernel's 27.5 at 12 rows (22.9 against 22.3 at 8); [7168, 5120] is the streaming kernel's (15.4 against 20.8)
+        if (MID_PRODUCTS and tiles is not None and m >= MID_SLICED_MIN_ROWS and bias is None and n % 4 == 0
+                and out_dtype in (None, torch.bfloat16) and n * k >= MID_SUMMED_MIN_ELEMENTS and k < TILED_LONG_ROWS):
+            return gemm_mid(x, tiles)
         return gemm_skinny(x, tiles if tiles is not None and m <= 16 else w, bias, out_dtype)
     if (MID_PRODUCTS and tiles is not None and bias is None and k % 8 == 0 and n % 4 == 0 and m <= GEMM_MID_MAX_ROWS
             and out_dtype in (None, torch.bfloat16) and n * k >= MID_SUMMED_MIN_ELEMENTS and k < TILED_LONG_ROWS):
@@ -633,6 +646,14 @@ GATED_MID_MIN_ROWS = 8         # ... for rows shorter than GATED_TILED_LONG_K co
 GATED_TILED_ROWS = 24          # ... and 32 for rows of GATED_TILED_LONG_K columns or more
 GATED_TILED_LONG_K = 4096
 GATED_TILED_ELEMENTS = 1 << 27
+# ... a [34816, 5120] weight too, up to 96 rows (63.4 against the streaming kernel's 70.7 us at 16 rows, 65.3 against
+# the library's 79.3 at 20, 75.0 against 85.8 at 48, 95.9 against 97.1 at 96; 116.9 against 101.6 at 128), while
+# [51200, 5120] is the library's from 12 rows on
+GATED_LARGE_ELEMENTS = 200 << 20
+GATED_LARGE_MAX_ROWS = 96
+# ... and below this size the streaming kernel keeps 8 rows ([12288, 2048] 10.8 against 12.1 us, [6144, 1024] 4.8
+# against 5.5; from 12 rows on the product with X in LDS is level or ahead)
+GATED_SMALL_ELEMENTS = 40 << 20
 
 
 def _gated_tiled(m: int, n: int, k: int) -> bool:
@@ -647,13 +668,19 @@ def linear_gated(x: torch.Tensor, w, activation: str = "silu") -> torch.Tensor:
     if x.dtype == torch.bfloat16 and k % 8 == 0:
         tiles = w.tiles if isinstance(w, LinearWeight) else None
         if m <= SKINNY_MAX_ROWS:
-            if (MID_PRODUCTS and tiles is not None and tiles.n * k <= GATED_TILED_ELEMENTS
-                    and m >= (GATED_MID_MIN_ROWS if k < GATED_TILED_LONG_K else 1)):
+            first = 1 if k >= GATED_TILED_LONG_K else GATED_MID_MIN_ROWS
+            if tiles is not None and tiles.n * k < GATED_SMALL_ELEMENTS:
+                first = GATED_MID_MIN_ROWS + 1
+            elif tiles is not None and tiles.n * k > GATED_TILED_ELEMENTS:
+                first = MID_SLICED_MIN_ROWS
+            if MID_PRODUCTS and tiles is not None and tiles.n * k <= GATED_LARGE_ELEMENTS and m >= first:
                 return gemm_mid(x, tiles, silu_mul_epilogue=True, activation=activation)
             if isinstance(w, LinearWeight):
                 w = tiles if tiles is not None and m <= 16 else w.rows
             return gemm_skinny(x, w, silu_mul_epilogue=True, activation=activation)
-        if MID_PRODUCTS and tiles is not None and m <= GEMM_MID_MAX_ROWS and tiles.n * k <= GATED_TILED_ELEMENTS:
+        if MID_PRODUCTS and tiles is not None and (
+                (m <= GEMM_MID_MAX_ROWS and tiles.n * k <= GATED_TILED_ELEMENTS)
+                or (m <= GATED_LARGE_MAX_ROWS and tiles.n * k <= GATED_LARGE_ELEMENTS)):
             return gemm_mid(x, tiles, silu_mul_epilogue=True, activation=activation)
         if tiles is not None and _gated_tiled(m, tiles.n, k):
             return gemm_skinny(x, tiles, silu_mul_epilogue=True, activation=activation)
