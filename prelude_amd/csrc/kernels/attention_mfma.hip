@@ -974,11 +974,13 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
                   float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_shift, int window, float scale,
                   float softcap, int split_keys, int max_splits, const FusedQkv& fq) {
   const int qtiles = (nh / nkv + 15) / 16;
-  // Up to 1,536 workgroups (what the chip holds at once, below) each XCD gets a contiguous stretch of them; measured
-  // in the decode step of a 4B model: batch 8 at 4,096 keys +0.9 %, batch 9 to 12 +0.8 to 1.2 %, batch 2 at 16,384
-  // +0.3 %, while larger grids do better dealt out plainly (batch 64 at 4,096: +3.5 %, batch 16 to 32: equal)
+  // Grids of 513 to 4,096 workgroups are dealt out so that each XCD gets a contiguous stretch of them; measured in
+  // the decode step of a 4B model: batch 8 at 4,096 keys +0.9 %, batch 9 to 12 +0.8 to 1.2 %, and the kernel alone
+  // (32 heads over 8, in a graph, us contiguous / plain): 768 workgroups 25.8 / 26.1, 1,536 42.7 / 44.5, 2,048
+  // 54.5 / 56.5, 4,096 99.8 / 101.7; larger and smaller grids do better dealt out plainly (8,192: 194.1 / 191.9,
+  // 16,384: 372.6 / 359.8; 512: 21.3 / 20.4, 256: 13.9 / 13.4, 128: 11.5 / 11.2)
   const long total = (long)nkv * qtiles * max_splits * nseq;
-  const int contiguous = total <= 1536;
+  const int contiguous = total > 512 && total <= 4096;
   dim3 grid(nkv * qtiles, max_splits, nseq);
   if (contiguous) grid = dim3((unsigned)total, 1, 1);
   // Twelve wavefronts fit a compute unit (three a SIMD by their registers): three workgroups of four, 768 on the
@@ -988,11 +990,11 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   // measured 1 to 2 % slower with two.  With two wavefronts a split's steps are added in another order (wavefront w
   // takes the steps w, w + 2, .. instead of w, w + 4, ..), so a token's sums can differ in their last bits between
   // steps whose grids fall on either side of these limits; what else is in the batch changes nothing beyond that.
-  // A grid of at most one workgroup a compute unit (one sequence of 4,096 keys: 128) runs with eight, a step of
-  // 32 keys each: batch 1 of a 4B model 2.518 -> 2.499 ms a step, batch 2 (256 workgroups) level; with eight up to
-  // 512 workgroups batch 3 and 4 lose 4 %.
+  // A grid of less than one workgroup a compute unit (one sequence of 4,096 keys: 128) runs with eight, a step of
+  // 32 keys each: batch 1 of a 4B model 2.518 -> 2.499 ms a step; 256 workgroups are level or better off with four
+  // (13.4 against 13.7 us), and with eight up to 512 workgroups batch 3 and 4 lose 4 %.
   const bool two_wavefronts = total > 768 && total <= 1536;
-  const bool eight_wavefronts = total <= 256 && nh / nkv <= 8 && split_keys == 256;
+  const bool eight_wavefronts = total <= 192 && nh / nkv <= 8 && split_keys == 256;
   if (eight_wavefronts) {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 8>), grid, dim3(8 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
