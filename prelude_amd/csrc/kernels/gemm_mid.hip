@@ -254,6 +254,9 @@ inline int mid_waves(int n, int slices) {
   int best = 4;
   double best_busy = 0.0;
   for (int wn : order) {
+    // three wavefronts are for small weights: every workgroup stages all of X, and a wide weight has many
+    // ([34816, 5120] with the gated epilogue at 64 rows: 86.5 us with three, 75.2 with five)
+    if (wn == 3 && tiles >= 1024) continue;
     const long groups = (long)((tiles + wn - 1) / wn) * slices;
     const long rounds = (groups + 255) / 256;
     const double busy = (double)tiles * slices / (double)(rounds * 256 * wn);
@@ -297,13 +300,21 @@ int launch_mid_wn(hipStream_t st, const void* x, const void* w, const float* bia
 using namespace pa;
 
 // How many slices of K pa_gemm_mid cuts a product into when its reader takes slices: as many as give every
-// compute unit a workgroup or two, each slice at least eight steps of 64 columns, eight at most.  Follows the
-// weight's shape alone.
+// compute unit a workgroup or two, each slice at least eight steps of 64 columns; four at most, eight for long rows
+// of a narrow weight.  Every slice is another 32-bit copy of the output that the product writes and the norm behind it
+// reads, with few workgroups: with the norm behind it, [2560, 4096] at 16 / 32 / 64 / 128 rows takes 10.7 / 11.6 /
+// 13.0 / 17.8 us in four slices and 12.0 / 13.4 / 15.7 / 19.3 in eight, [4096, 4096] 14.6 / 15.0 / 18.4 / 22.5 and
+// 16.7 / 17.4 / 20.3 / 26.2, [4096, 12288] 24.9 / 25.5 / 29.8 / 41.8 and 27.7 / 27.9 / 33.2 / 43.1; [2560, 9728] is
+// level or better in eight (18.2 / 18.8 / 21.0 / 27.5 against 17.8 / 19.6 / 21.3 / 30.0).  In the decode step
+// (context 2,048, same box, eight slices at most against this): 4B shape batch 32 / 64 4.61 / 6.64 against 4.58 /
+// 6.59 ms, 8B shape batch 32 / 64 / 128 6.05 / 7.95 / 12.54 against 5.89 / 7.90 / 12.39.  Follows the weight's
+// shape alone.
 extern "C" int pa_gemm_mid_slices(int n, int k) {
   if (n <= 0 || k <= 0) return 1;
   const int blocks = ((n + 15) / 16 + 4) / 5, steps = (k + 63) / 64;
+  const int most = (blocks * 4 < 160 && steps >= 128) ? 8 : 4;
   int s = 1;
-  while (s < 8 && blocks * s < 256 && steps / (2 * s) >= 8) s *= 2;
+  while (s < most && blocks * s < 256 && steps / (2 * s) >= 8) s *= 2;
   return s;
 }
 
