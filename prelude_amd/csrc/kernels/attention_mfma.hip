@@ -1077,7 +1077,11 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // four heads' state in 256) -- unless that leaves compute units without a workgroup: a short prompt is better
   // off unpaired and with a head per wavefront.  Measured at head_dim 128: one prompt of 512 tokens takes 16 us
   // as 256 workgroups and 26 us as 64.
-  const int gt_best = (HD <= 64 && group % 4 == 0) ? 4 : (group % 2 == 0 ? 2 : 1);
+  // (four heads a wavefront, which heads of up to 64 wide have registers for, measured slower than two at every
+  // size but 8,192 tokens, where it is level: 32 heads over 8 of 64 at 2,048 tokens 66 us against 45 and 36 with
+  // two and one; the kernel stays for callers that ask for it)
+  const int gt_best = group % 2 == 0 ? 2 : 1;
+  const int gt_most = (HD <= 64 && group % 4 == 0) ? 4 : gt_best;   // what a caller's own cut may ask for
   const long tiles = (max_q_len + 63) / 64;
   const bool can_stage = page_shift >= 3;
   auto workgroups = [&](int p, int g_, int h_ = 1) {
@@ -1112,11 +1116,15 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
     hw = 2;
   } else if (wide_ok && tiles > 8 && !level && workgroups(0, gt_best, 2) >= spread) {
     paired = 0, hw = 2;
-  } else if (level && workgroups(0, gt_best, wide_ok ? 2 : 1) >= enough) {
+  } else if (level && workgroups(0, gt_best, wide_ok ? 2 : 1) >= (wide_ok ? enough : 2 * enough)) {
+    // (workgroups of four wavefronts want two on a compute unit: 16 heads over 8, 2,048 tokens behind 6,144, as 256
+    // of them 274 us, as 256 of eight wavefronts with a head each 166)
     paired = 0;   // 2,048 tokens behind 6,144: 297 against 342 us
     hw = wide_ok ? 2 : 1;
   } else if (level && can_stage && group % 2 == 0 && workgroups(0, 1, 2) >= enough) {
     paired = 0, gt = 1, hw = 2;   // 1,024 tokens behind 7,168: 205 against 293 us
+  } else if (!wide_ok && gt_best >= 2 && tiles > 8 && full_rounds(workgroups(1, gt_best, 1), 2 * enough)) {
+    // whole rounds of pairs of four wavefronts, two heads each (16 heads over 8 at 8,192 tokens: 307 against 332 us)
   } else if (half_ok && tiles > 8 && full_rounds(workgroups(1, gt_half, 2), enough)) {
     gt = gt_half, hw = 2;         // 2,048 tokens: 256 pairs of eight wavefronts, a head each
   } else if (half_ok && tiles > 8 && workgroups(0, gt_half, 2) >= spread) {
@@ -1153,8 +1161,8 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // a caller's own cut (tests and measurements), where it is one the kernels have
   if (want.paired >= 0) paired = want.paired != 0 && tiles >= 2;
   if (want.heads >= 0) {
-    PA_REQUIRE((want.heads == 1 || want.heads == 2 || want.heads == 4) && want.heads <= gt_best,
-               "attn_prefill: %d heads a wavefront, this shape takes up to %d (1, 2 or 4)", want.heads, gt_best);
+    PA_REQUIRE((want.heads == 1 || want.heads == 2 || want.heads == 4) && want.heads <= gt_most,
+               "attn_prefill: %d heads a wavefront, this shape takes up to %d (1, 2 or 4)", want.heads, gt_most);
     gt = want.heads;
     if (want.groups < 0) hw = 1;
   }
@@ -1169,7 +1177,7 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
     staged = want.staged != 0;
   }
   PA_REQUIRE(staged || hw == 1, "attn_prefill: two head groups a workgroup only with staged keys");
-  PA_REQUIRE(gt <= gt_best, "attn_prefill: %d heads a wavefront, head_dim %d takes up to %d", gt, HD, gt_best);
+  PA_REQUIRE(gt <= gt_most, "attn_prefill: %d heads a wavefront, head_dim %d takes up to %d", gt, HD, gt_most);
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
                                    max_q_len, nh, nkv, page_shift, window, scale, softcap, paired, hw, staged)
