@@ -124,6 +124,8 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, const float* __restrict_
 // The same with 16-byte loads and every element held in registers between the
 // two passes: one read of x and the residual, one write of each output.
 // NV vectors per thread; the block has ceil(hidden / VEC / NV) threads rounded up to a wavefront.
+constexpr int kSlicesAtOnce = 8;
+
 template <typename T, int NV>
 __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, const float* __restrict__ parts, int slices,
                                    size_t slice_stride, T* residual, const float* __restrict__ w,
@@ -149,9 +151,17 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, const float* __restr
 #pragma unroll
         for (int e = 0; e < VEC; e += 4) {
           float4 a = *reinterpret_cast<const float4*>(pr + (size_t)v * VEC + e);
-          for (int p = 1; p < slices; ++p) {
-            const float4 b = *reinterpret_cast<const float4*>(pr + (size_t)p * slice_stride + (size_t)v * VEC + e);
-            a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+          // up to eight slices are asked for together and then added (one trip to memory instead of one a slice)
+          float4 b[kSlicesAtOnce - 1];
+#pragma unroll
+          for (int p = 1; p < kSlicesAtOnce; ++p)
+            if (p < slices) b[p - 1] = *reinterpret_cast<const float4*>(pr + (size_t)p * slice_stride + (size_t)v * VEC + e);
+#pragma unroll
+          for (int p = 1; p < kSlicesAtOnce; ++p)
+            if (p < slices) a.x += b[p - 1].x, a.y += b[p - 1].y, a.z += b[p - 1].z, a.w += b[p - 1].w;
+          for (int p = kSlicesAtOnce; p < slices; ++p) {
+            const float4 c = *reinterpret_cast<const float4*>(pr + (size_t)p * slice_stride + (size_t)v * VEC + e);
+            a.x += c.x, a.y += c.y, a.z += c.z, a.w += c.w;
           }
           s[j][e] = a.x, s[j][e + 1] = a.y, s[j][e + 2] = a.z, s[j][e + 3] = a.w;
         }

@@ -212,7 +212,15 @@ __global__ void sum_slices_kernel(const float* __restrict__ parts, T* __restrict
   if (i >= total) return;
   if (i + 3 < total) {
     float4 s = *reinterpret_cast<const float4*>(parts + i);
-    for (int p = 1; p < slices; ++p) {
+    // up to eight slices are asked for together and then added in their order
+    float4 b[7];
+#pragma unroll
+    for (int p = 1; p < 8; ++p)
+      if (p < slices) b[p - 1] = *reinterpret_cast<const float4*>(parts + (size_t)p * total + i);
+#pragma unroll
+    for (int p = 1; p < 8; ++p)
+      if (p < slices) s.x += b[p - 1].x, s.y += b[p - 1].y, s.z += b[p - 1].z, s.w += b[p - 1].w;
+    for (int p = 8; p < slices; ++p) {
       const float4 v = *reinterpret_cast<const float4*>(parts + (size_t)p * total + i);
       s.x += v.x, s.y += v.y, s.z += v.z, s.w += v.w;
     }
