@@ -321,6 +321,48 @@ def test_gemm_tall_refuses_and_is_dispatched(gpu):
     close(K().linear_silu_mul(xg, lg), pm.silu(g[:, 0::2]) * g[:, 1::2], torch.bfloat16)
 
 
+def test_dispatch_of_large_weights(gpu):
+    """Where the dispatcher sends the products of very large weights at few rows, each against the product in 32-bit
+    on the CPU: a weight of 40 M elements whose reader wants a tensor at 9 to 16 rows (the product with X in LDS,
+    uncut), rows of 16,384 columns for a reader of slices from 8 rows on, and the gated product of a weight between
+    128 M and 200 M elements up to 96 rows (X in LDS, activation in the epilogue) and beyond (the library)."""
+    g = torch.Generator().manual_seed(11)
+    def weight(n, k):
+        return (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16)
+    def rows(m, k):
+        return torch.randn(m, k, generator=g).to(torch.bfloat16)
+    # a reader of tensors, 12 rows
+    w = weight(10240, 4096)
+    lw = K().LinearWeight(w.to(gpu), K().pack_tiles(w.to(gpu)))
+    x = rows(12, 4096)
+    got = K().linear(x.to(gpu), lw)
+    assert isinstance(got, torch.Tensor) and torch.equal(got, K().gemm_mid(x.to(gpu), lw.tiles))
+    close(got, x.float() @ w.float().T, torch.bfloat16)
+    del lw
+    # long rows, a reader of slices, 8 rows
+    w = weight(2560, 16384)
+    lw = K().LinearWeight(w.to(gpu), K().pack_tiles(w.to(gpu)))
+    x = rows(8, 16384)
+    got = K().linear(x.to(gpu), lw, slices_ok=True)
+    assert isinstance(got, K().SliceSums)
+    close(K().as_tensor(got), x.float() @ w.float().T, torch.bfloat16)
+    assert isinstance(K().linear(x[:7].contiguous().to(gpu), lw, slices_ok=True), torch.Tensor)
+    del lw
+    # the gated product of a very large weight
+    w = weight(26624, 5120)
+    lw = K().LinearWeight(w.to(gpu), K().pack_tiles(w.to(gpu)))
+    for m in (20, 96, 100):
+        x = rows(m, 5120)
+        ref = x.float() @ w.float().T
+        want = pm.silu(ref[:, 0::2].double()) * ref[:, 1::2].double()
+        got = K().linear_gated(x.to(gpu), lw)
+        if m <= 96:
+            assert torch.equal(got, K().gemm_mid(x.to(gpu), lw.tiles, silu_mul_epilogue=True))
+            close(got, want, torch.bfloat16)
+        else:   # gate and up rounded to bfloat16 by the library before the activation
+            close(got, want, torch.bfloat16, bf16=1.25e-2)
+
+
 def test_gemm_mid_refuses_and_is_dispatched(gpu):
     from prelude_amd._native import NativeError
     w = rnd(2560, 4096, dtype=torch.bfloat16, seed=1, scale=0.05).to(gpu)
