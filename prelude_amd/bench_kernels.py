@@ -1,6 +1,6 @@
 """Times single kernels against their rooflines on one MI355X.
 
-    python -m prelude_amd.bench_kernels [stream] [gemm] [tall] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
+    python -m prelude_amd.bench_kernels [stream] [gemm] [tall] [dispatch] [cuts] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
 
 Each line gives the kernel's time (device events around repeated launches,
 operands rotated over copies larger than the caches where the kernel streams
@@ -20,8 +20,11 @@ from .ops import kernels as K
 HBM_PEAK = 8.0e12
 MFMA_PEAK = 2.5e15
 SHAPES = {   # hidden, intermediate, heads, kv heads, head_dim, vocabulary
+    "0.6b": (1024, 3072, 16, 8, 128, 151936),
+    "1.7b": (2048, 6144, 16, 8, 128, 151936),
     "4b": (2560, 9728, 32, 8, 128, 151936),
     "8b": (4096, 12288, 32, 8, 128, 151936),
+    "14b": (5120, 17408, 40, 8, 128, 151936),
     "32b": (5120, 25600, 64, 8, 128, 151936),
 }
 
@@ -128,6 +131,125 @@ def bench_tall(dev, shape) -> None:
         del rows, tiles
 
 
+def graph_time(fns, iters: int = 10) -> float:
+    """Microseconds per call of the chain ``fns`` (one call per operand copy), replayed from a captured graph: what a
+    kernel costs inside a step, where no launch waits for the host."""
+    for f in fns:
+        f()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for f in fns:
+            f()
+    g.replay()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        g.replay()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters / len(fns) * 1e3
+
+
+def bench_dispatch(dev, shape) -> None:
+    """Every product of the shape at 1 to 512 rows as ``ops.kernels.linear`` / ``linear_gated`` dispatch it against
+    every kernel forced, each with its reader behind it (the residual add + norm for o and down, which takes a
+    product's slices as they are), inside a graph, weights rotated so that they come from memory.  A line ends in
+    ``<<<`` where the dispatcher's choice is more than a twentieth behind the best kernel."""
+    h, inter, nh, nkv, hd, _ = shape
+    prods = {"qkv": ((nh + 2 * nkv) * hd, h, "tensor"), "o": (h, nh * hd, "norm"), "gate_up": (2 * inter, h, "gated"),
+             "down": (h, inter, "norm")}
+    for pname, (n, k, kind) in prods.items():
+        copies = max(3, min(12, int(700e6 // (n * k * 2))))
+        rows = [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        lws = [K.LinearWeight(r, K.pack_tiles(r)) for r in rows]
+        gain = torch.ones(n, device=dev)
+        for m in (1, 4, 8, 12, 16, 20, 24, 32, 48, 64, 96, 128, 160, 192, 256, 384, 512):
+            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            res = torch.randn(m, n, device=dev, dtype=torch.bfloat16)
+            norm = lambda y: K.rmsnorm(y, gain, 1e-6, residual=res)
+            cands = {}
+            if kind == "tensor":
+                cands["dispatched"] = lambda w: K.linear(x, w)
+                if m <= 64:
+                    cands["skinny"] = lambda w: K.gemm_skinny(x, w.tiles)
+                if m <= 128:
+                    cands["mid"] = lambda w: K.gemm_mid(x, w.tiles)
+                    s = K.gemm_mid_slices(n, k)
+                    if s > 1:
+                        cands["mid sliced + sum"] = lambda w: K.gemm_mid(x, w.tiles, slices=s).materialize()
+                cands["library"] = lambda w: K.gemm_library(x, w.rows)
+                if m > 16:
+                    cands["tall"] = lambda w: K.gemm_tall(x, w.tiles)
+            elif kind == "norm":
+                cands["dispatched"] = lambda w: norm(K.linear(x, w, slices_ok=True))
+                if m <= 64:
+                    cands["skinny"] = lambda w: norm(K.gemm_skinny(x, w.tiles))
+                if m <= 128:
+                    s = K.gemm_mid_slices(n, k)
+                    if s > 1:
+                        cands["mid sliced"] = lambda w: norm(K.gemm_mid(x, w.tiles, slices=s))
+                    cands["mid"] = lambda w: norm(K.gemm_mid(x, w.tiles))
+                cands["library"] = lambda w: norm(K.gemm_library(x, w.rows))
+                if m > 16:
+                    s4 = K._tall_slices(k)
+                    if s4 > 1:
+                        cands["tall sliced"] = lambda w: norm(K.gemm_tall(x, w.tiles, slices=s4))
+                    cands["tall"] = lambda w: norm(K.gemm_tall(x, w.tiles))
+            else:
+                cands["dispatched"] = lambda w: K.linear_gated(x, w, "silu")
+                if m <= 64:
+                    cands["skinny"] = lambda w: K.gemm_skinny(x, w.tiles, silu_mul_epilogue=True)
+                if m <= 128:
+                    cands["mid"] = lambda w: K.gemm_mid(x, w.tiles, silu_mul_epilogue=True)
+                cands["library"] = lambda w: K.silu_mul(K.gemm_library(x, w.rows))
+                if m > 16:
+                    cands["tall"] = lambda w: K.gemm_tall(x, w.tiles, silu_mul_epilogue=True)
+            t = {c: graph_time([(lambda w=w, f=f: f(w)) for w in lws]) for c, f in cands.items()}
+            d = t.pop("dispatched")
+            best = min(t, key=t.get)
+            print(f"{pname:8s} [{n:6d} x {k:6d}] M={m:4d}: dispatched {d:7.1f} us  best {best:16s} {t[best]:7.1f}   " +
+                  "  ".join(f"{c} {v:.1f}" for c, v in t.items()) + ("  <<<" if d > 1.05 * t[best] + 0.3 else ""), flush=True)
+        del rows, lws
+
+
+def bench_cuts(dev, shape, page: int = 16) -> None:
+    """The prefill attention as its launcher cuts the work against every cut forced (tiles paired or not, 1 or 2
+    heads a wavefront, 1 or 2 head groups a workgroup), over prompts of 256 to 8,192 tokens, several prompts a
+    step and portions behind long contexts; every cut gives the same bits."""
+    _, _, nh, nkv, hd, _ = shape
+    sizes = [(1, t, t) for t in (256, 512, 1024, 1536, 2048, 3072, 4096, 6144, 8192)]
+    sizes += [(n, 512, 512) for n in (2, 4, 8, 16)] + [(2, 2048, 2048), (1, 512, 4096), (1, 2048, 8192)]
+    for nseq, t, ctx in sizes:
+        pages = nseq * ctx // page
+        kc = torch.randn(pages, nkv, page, hd, device=dev, dtype=torch.bfloat16)
+        vc = torch.randn(pages, nkv, hd, page, device=dev, dtype=torch.bfloat16)
+        table = torch.randperm(pages, device=dev).to(torch.int32).view(nseq, ctx // page)
+        q = torch.randn(nseq * t, nh, hd, device=dev, dtype=torch.bfloat16)
+        seqs = torch.arange(nseq, device=dev, dtype=torch.int32)
+        cu = torch.arange(0, (nseq + 1) * t, t, device=dev, dtype=torch.int32)
+        lens = torch.full((nseq,), ctx, device=dev, dtype=torch.int32)
+        out = torch.empty_like(q)
+        scale = 1 / math.sqrt(hd)
+        run = lambda cut: timeit(lambda i: K.attention_prefill(q, kc, vc, table, seqs, cu, lens, out, t, 0, scale,
+                                                               min_prefix=ctx - t, cut=cut), 1, iters=15)
+        for _ in range(3):
+            run(None)
+        res = {}
+        for heads, groups in ((1, 1), (1, 2), (2, 1), (2, 2)):
+            for paired in (0, 1):
+                try:
+                    res[f"{heads} heads x {groups}{' paired' if paired else ''}"] = run((paired, heads, groups, 1))
+                except Exception:   # a cut this shape does not have
+                    pass
+        us = min(run(None), run(None))
+        best = min(res, key=res.get)
+        flops = 2.0 * nseq * nh * hd * t * (2 * ctx - t)
+        print(f"prefill attention {nseq:2d} x {t:5d} tokens, context {ctx:5d}: launcher {us:7.1f} us ({flops / us / 1e6 / MFMA_PEAK * 1e12:.2f} of peak)  "
+              f"best cut {best} {res[best]:7.1f}  ratio {us / res[best]:.3f}", flush=True)
+
+
 def bench_decode(dev, shape, page: int = 16) -> None:
     _, _, nh, nkv, hd, _ = shape
     for batch, ctx in ((1, 4096), (8, 512), (8, 4096), (8, 32768), (64, 4096)):
@@ -200,7 +322,7 @@ def bench_sampling(dev, shape) -> None:
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
-    ap.add_argument("what", nargs="*", help="stream, gemm, tall, decode, prefill, elementwise, sampling (default: all)")
+    ap.add_argument("what", nargs="*", help="stream, gemm, tall, decode, prefill, elementwise, sampling (default: all these); dispatch, cuts (sweeps, on request)")
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -212,7 +334,7 @@ def main() -> int:
     print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
           f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
     for name in todo:
-        {"stream": bench_stream, "gemm": bench_gemm, "tall": bench_tall, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
+        {"stream": bench_stream, "gemm": bench_gemm, "tall": bench_tall, "dispatch": bench_dispatch, "cuts": bench_cuts, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
          "sampling": bench_sampling}[name](dev, shape)
     return 0
 

@@ -398,9 +398,6 @@ MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns,
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
 MID_SLICED_LONG_K = 8192
-MID_SLICED_SHORT_ROWS = 24     # ... and up to here small weights with shorter rows stay with the streaming kernel:
-MID_SLICED_SHORT_K = 4096      #     rows of up to this many columns,
-MID_SLICED_SHORT_ELEMENTS = 1 << 24   # weights of up to this many elements
 MID_SLICED_MIN_ROWS_LONG = 8   # rows of TILED_LONG_ROWS columns or more: in slices from here on
 # A reader that wants a tensor gets the slices too, added by a kernel of their own, where the pair is still ahead of
 # the library: large weights ([10240, 5120] inside a captured step: 24.2 to 26.9 us at 24 to 64 rows against 28.4 to
@@ -576,13 +573,11 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
               and (m > SKINNY_MAX_ROWS or (m >= MID_SLICED_MIN_ROWS and k >= MID_SLICED_LONG_K)
                    # rows of 16,384 columns and more from 8 rows on ([5120, 17408] with the norm behind it 40.0
                    # against 42.6 us at 8 rows, [5120, 25600] 54.3 against 57.9; level at 4 rows)
-                   or (m >= MID_SLICED_MIN_ROWS_LONG and k >= TILED_LONG_ROWS))
-              # just beyond 16 rows a small weight with short rows is still the streaming kernel's (inside a captured
-              # step, with the norm that reads it: [4096, 4096] 13.3 and 14.4 us at 17 and 24 rows against 16.8 in
-              # slices, [2560, 4096] 12.5 and 13.7 against 13.3 and 13.9; from 32 rows on the slices are ahead; a
-              # [5120, 5120] weight is ahead in slices already, 17.5 against 21.2 us at 24 rows)
-              and not (m <= MID_SLICED_SHORT_ROWS and k <= MID_SLICED_SHORT_K and n * k <= MID_SLICED_SHORT_ELEMENTS
-                       and _tiled_beyond_16(m, n, k)))
+                   or (m >= MID_SLICED_MIN_ROWS_LONG and k >= TILED_LONG_ROWS)))
+    # (with four slices at most this holds just beyond 16 rows too, where eight slices lost to the streaming kernel:
+    # with the norm that reads it, at 20 and 24 rows, [2560, 4096] 11.3 and 11.4 us against 12.2 and 13.0, [2048, 2048]
+    # 8.7 against 9.0 and 9.2, [5120, 5120] 17.6 and 17.5 against 20.2 and 21.2; [4096, 4096] 14.6 and 14.9 against
+    # 13.9 and 14.7 is the one shape the other way round)
     if sliced:
         s = gemm_mid_slices(n, k)
         if s >= MID_MIN_SLICES:
