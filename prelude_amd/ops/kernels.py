@@ -397,7 +397,7 @@ MID_WIDE_MAX_M = 64            # ... for rows of up to MID_WIDE_SHORT_K columns,
 #                                7,640 tok/s.  The step decides.)
 MID_WIDE_SHORT_K = 4096
 MID_SLICED_MIN_ROWS = 9        # ... for rows of MID_SLICED_LONG_K columns or more; 17 otherwise
-MID_SLICED_LONG_K = 8192
+MID_SLICED_LONG_K = 5120
 MID_SLICED_MIN_ROWS_LONG = 8   # rows of TILED_LONG_ROWS columns or more: in slices from here on
 # A reader that wants a tensor gets the slices too, added by a kernel of their own, where the pair is still ahead of
 # the library: large weights ([10240, 5120] inside a captured step: 24.2 to 26.9 us at 24 to 64 rows against 28.4 to
