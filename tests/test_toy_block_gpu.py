@@ -1,8 +1,9 @@
 """Another arrangement of a layer's parts and another norm, asked for from outside the package without editing a
 file of it: a block that runs its mixer and its feed-forward side by side on one normed input (x + mixer(n(x)) +
 ffn(n(x))) next to a layer of the framework's own pre-norm arrangement, and a norm that subtracts the mean and has a
-bias (in the second layer and as the model's final norm, which norms the wanted rows only).  The mixer and the
-feed-forward in both layers are the framework's own; a toy architecture, against its plain form; no model of
+bias (in the second layer and as the model's final norm, which norms the wanted rows only); an embedding that scales
+its rows by the square root of the width, and a head that bends its logits to cap * tanh(logit / cap).  The mixer
+and the feed-forward in both layers are the framework's own; a toy architecture, against its plain form; no model of
 anyone's.
 """
 import dataclasses
@@ -15,13 +16,44 @@ import plain_model as pm
 
 pytestmark = pytest.mark.gpu
 HD = 64
+LOGIT_CAP = 3.0
 
 
 def register_toy_block():
     from prelude_amd.config.registry import Architecture, register_architecture
     from prelude_amd.models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
     from prelude_amd.ops import kernels as K
-    from prelude_amd.parts import NORM, VECTOR, Block, Norm, TensorReq, register_part
+    from prelude_amd.parts import MATRIX, NORM, VECTOR, Block, Norm, Part, TensorReq, register_part
+
+    @register_part("embedding", "toy_scaled_embedding")
+    class ScaledEmbedding(Part):
+        def __init__(self, vocab_size, hidden_size):
+            self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+
+        def tensors(self):
+            return {"weight": TensorReq((self.vocab_size, self.hidden_size), MATRIX)}
+
+        def load(self, tensors, dtype, device):
+            self.weight = tensors["weight"]
+
+        def forward(self, token_ids):
+            rows = K.embed_gather(token_ids, self.weight)
+            return (rows.float() * math.sqrt(self.hidden_size)).to(rows.dtype)
+
+    @register_part("head", "toy_capped_head")
+    class CappedHead(Part):
+        def __init__(self, vocab_size, hidden_size, cap):
+            self.vocab_size, self.hidden_size, self.cap = int(vocab_size), int(hidden_size), float(cap)
+
+        def tensors(self):
+            return {"weight": TensorReq((self.vocab_size, self.hidden_size), MATRIX)}
+
+        def load(self, tensors, dtype, device):
+            self.weight = K.prepare_weight(tensors["weight"])
+
+        def forward(self, hidden_rows):
+            logits = K.linear(hidden_rows, self.weight, out_dtype=torch.float32)
+            return self.cap * torch.tanh(logits / self.cap)
 
     @register_part("norm", "toy_centered_norm")
     class CenteredNorm(Norm):
@@ -98,9 +130,10 @@ def register_toy_block():
         first = LayerSpec("prenorm", {"input_norm": rms("l0.n1"), "post_mixer_norm": rms("l0.n2"), "mixer": attn(0), "ffn": ffn(0)})
         second = LayerSpec("toy_side_by_side", {"norm": centered("l1.n"), "mixer": attn(1), "ffn": ffn(1)})
         return ModelSpec("ToyBlockForCausalLM", c.vocab_size, c.hidden_size, c.max_positions, (0,),
-                         PartSpec("token_embedding", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "emb"}),
+                         PartSpec("toy_scaled_embedding", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "emb"}),
                          [first, second], [RunSpec(0), RunSpec(1), RunSpec(0)], centered("final"),
-                         PartSpec("linear_head", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size), {"weight": "head"}),
+                         PartSpec("toy_capped_head", dict(vocab_size=c.vocab_size, hidden_size=c.hidden_size, cap=LOGIT_CAP),
+                                  {"weight": "head"}),
                          {"rope": PartSpec("rope", dict(rotary_dim=HD, max_positions=c.max_positions, theta=10000.0))})
 
     register_architecture(Architecture("toy_block", ("ToyBlock",), ("toy_block",),
@@ -135,7 +168,7 @@ def plain(raw, w, toks, norm=centered_norm, side_by_side=True):
     def prenorm(x):
         x = x + attn(pm.rms_norm(x, w["l0.n1"], eps), "l0.attn.")
         return x + ffn(pm.rms_norm(x, w["l0.n2"], eps), "l0.ffn.")
-    x = prenorm(w["emb"][toks])
+    x = prenorm(w["emb"][toks] * math.sqrt(raw["hidden_size"]))
     h = norm(x, w["l1.n.w"], w["l1.n.b"], eps)
     if side_by_side:
         x = x + attn(h, "l1.attn.") + ffn(h, "l1.ffn.")
@@ -143,7 +176,7 @@ def plain(raw, w, toks, norm=centered_norm, side_by_side=True):
         x = x + attn(h, "l1.attn.")
         x = x + ffn(norm(x, w["l1.n.w"], w["l1.n.b"], eps), "l1.ffn.")
     x = prenorm(x)
-    return norm(x, w["final.w"], w["final.b"], eps) @ w["head"].T
+    return LOGIT_CAP * torch.tanh(norm(x, w["final.w"], w["final.b"], eps) @ w["head"].T / LOGIT_CAP)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
