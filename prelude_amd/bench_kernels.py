@@ -215,12 +215,13 @@ def bench_dispatch(dev, shape) -> None:
 
 
 def bench_cuts(dev, shape, page: int = 16) -> None:
-    """The prefill attention as its launcher cuts the work against every cut forced (tiles paired or not, 1 or 2
-    heads a wavefront, 1 or 2 head groups a workgroup), over prompts of 256 to 8,192 tokens, several prompts a
-    step and portions behind long contexts; every cut gives the same bits."""
+    """The prefill attention as its launcher cuts the work against every cut forced (tiles paired, unpaired, or
+    unpaired with the tiles slowest over the grid; 1 or 2 heads a wavefront, 1 or 2 head groups a workgroup), over
+    prompts of 256 to 8,192 tokens, several prompts a step and portions behind long contexts; every cut gives the
+    same bits."""
     _, _, nh, nkv, hd, _ = shape
     sizes = [(1, t, t) for t in (256, 512, 1024, 1536, 2048, 3072, 4096, 6144, 8192)]
-    sizes += [(n, 512, 512) for n in (2, 4, 8, 16)] + [(2, 2048, 2048), (1, 512, 4096), (1, 2048, 8192)]
+    sizes += [(n, 512, 512) for n in (2, 3, 4, 6, 8, 16)] + [(3, 1024, 1024), (2, 2048, 2048), (3, 2048, 2048), (1, 512, 4096), (1, 2048, 8192)]
     for nseq, t, ctx in sizes:
         pages = nseq * ctx // page
         kc = torch.randn(pages, nkv, page, hd, device=dev, dtype=torch.bfloat16)
@@ -238,9 +239,9 @@ def bench_cuts(dev, shape, page: int = 16) -> None:
             run(None)
         res = {}
         for heads, groups in ((1, 1), (1, 2), (2, 1), (2, 2)):
-            for paired in (0, 1):
+            for paired in (0, 1, 2):
                 try:
-                    res[f"{heads} heads x {groups}{' paired' if paired else ''}"] = run((paired, heads, groups, 1))
+                    res[f"{heads} heads x {groups}{('', ' paired', ' tiles slowest')[paired]}"] = run((paired, heads, groups, 1))
                 except Exception:   # a cut this shape does not have
                     pass
         us = min(run(None), run(None))

@@ -950,13 +950,17 @@ __global__ __launch_bounds__(256 * HW, 2) void attn_prefill_lds_kernel(
   const int group = nh / nkv;
   const int hgroups = group / (GT * HW);
   const int kvh = blockIdx.x / hgroups, hg = blockIdx.x % hgroups;   // head groups fastest over the grid
-  const int seq = seq_ids[blockIdx.z];
+  // paired 2: unpaired, and the tiles (not the sequences) slowest over the grid, so that the long tiles of every
+  // sequence are handed out before any short one
+  const bool tile_slowest = paired == 2;
+  const int seq = seq_ids[tile_slowest ? blockIdx.y : blockIdx.z];
+  const int at = tile_slowest ? (int)blockIdx.z : (int)blockIdx.y;
   const int row0 = cu_q[seq];
   const int q_len = cu_q[seq + 1] - row0;
   const int ctx = context_lens[seq];
   const int tiles = (q_len + 63) / 64;
-  const int first = paired ? (int)blockIdx.y : tiles - 1 - (int)blockIdx.y;
-  const int second = paired ? tiles - 1 - (int)blockIdx.y : first;
+  const int first = paired == 1 ? at : tiles - 1 - at;
+  const int second = paired == 1 ? tiles - 1 - at : first;
   if (first > second || first < 0) return;   // the same for the whole workgroup
   const int* table = block_table + (size_t)seq * table_stride;
   const int head0 = kvh * group + hg * GT * HW;
@@ -1027,7 +1031,8 @@ int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const v
                           int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale,
                           float softcap, int paired) {
   const int tiles = (max_q_len + 63) / 64;
-  dim3 grid(nkv * (nh / nkv / (GT * HW)), paired ? (tiles + 1) / 2 : tiles, nseq);
+  dim3 grid(nkv * (nh / nkv / (GT * HW)), paired == 1 ? (tiles + 1) / 2 : tiles, nseq);
+  if (paired == 2) grid = dim3(grid.x, nseq, tiles);
   // the two buffers are more than the 64 KB a kernel may declare: asked for at launch, allowed once per kernel
   static const hipError_t allowed =
       hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_lds_kernel<HD, GT, HW>),
@@ -1046,7 +1051,8 @@ int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void*
                       int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, float softcap,
                       int paired, int hw, bool staged) {
   const int tiles = (max_q_len + 63) / 64;
-  dim3 grid(nkv * (nh / nkv / GT), paired ? (tiles + 1) / 2 : tiles, nseq);
+  if (!staged && paired == 2) paired = 0;   // the kernel that reads the cache itself has the one order
+  dim3 grid(nkv * (nh / nkv / GT), paired == 1 ? (tiles + 1) / 2 : tiles, nseq);
   if (staged) {
     if (hw == 2)
       return launch_prefill_staged<HD, GT, 2>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
@@ -1108,7 +1114,34 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
     return (w >= slots && (w % slots == 0 || w >= 4 * slots)) || (tiles <= 16 && 4 * w >= 3 * slots && w <= slots);
   };
   const long spread = enough * 3 / 2;
-  if (wide_ok && tiles > 8 && full_rounds(workgroups(1, gt_best, 2), enough)) {
+  // Two to six prompts: within a launch the workgroups are handed out sequence by sequence, so unpaired the last
+  // prompt's long tiles start late; with the tiles slowest over the grid (paired 2) every prompt's long tiles
+  // come first, and unpaired is ahead of pairs wherever the pairs are not exactly whole rounds (32 heads over 8 of
+  // 128, us: three prompts of 512 tokens 20.0 against 22.1 in pairs and 23.2 sequence by sequence, six of 512 32.1
+  // against 35.0, three of 1,024 44.6 against 49.9, three of 2,048 131.6 against 147.1; 40 heads over 8, two of 512
+  // 17.7 against 23.8).  With many prompts the interleaving costs more in the L2 than the order gains (sixteen of
+  // 512: 80.9 against 70.5).
+  const bool few = can_stage && !level && nseq >= 2 && nseq <= 6 && tiles >= 2;
+  auto whole = [&](long w, long slots) { return w >= slots && w % slots == 0; };
+  if (few) {
+    // the kinds of workgroup from the most heads down; of each, pairs if they are whole rounds, else unpaired if
+    // there are workgroups enough to balance out
+    if (wide_ok && whole(workgroups(1, gt_best, 2), enough)) {
+      hw = 2;
+    } else if (wide_ok && workgroups(0, gt_best, 2) >= spread) {
+      paired = 2, hw = 2;
+    } else if (whole(workgroups(1, gt_best, 1), 2 * enough)) {
+      hw = 1;
+    } else if (gt_best >= 2 && workgroups(0, gt_best, 1) >= 2 * spread) {
+      paired = 2, hw = 1;
+    } else if (half_ok && whole(workgroups(1, gt_half, 2), enough)) {
+      gt = gt_half, hw = 2;
+    } else if (half_ok && workgroups(0, gt_half, 2) >= spread) {
+      paired = 2, gt = gt_half, hw = 2;
+    } else {
+      paired = 2, gt = gt_half, hw = 1;
+    }
+  } else if (wide_ok && tiles > 8 && full_rounds(workgroups(1, gt_best, 2), enough)) {
     // the most work per staged key that still gives every compute unit a workgroup (measured at head_dim 128,
     // 32 heads over 8: 4,096 tokens 171 against 186 us, 8,192 tokens 624 against 648); not for many short prompts,
     // whose workgroups are over after a few blocks (16 prompts of 512 tokens: 66 against 70 us with four
@@ -1159,7 +1192,7 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   // keys staged in LDS for pages of 8 keys or more; pages of 4 go to the kernel that reads them itself
   bool staged = can_stage;
   // a caller's own cut (tests and measurements), where it is one the kernels have
-  if (want.paired >= 0) paired = want.paired != 0 && tiles >= 2;
+  if (want.paired >= 0) paired = want.paired == 2 ? 2 : (want.paired != 0 && tiles >= 2);
   if (want.heads >= 0) {
     PA_REQUIRE((want.heads == 1 || want.heads == 2 || want.heads == 4) && want.heads <= gt_most,
                "attn_prefill: %d heads a wavefront, this shape takes up to %d (1, 2 or 4)", want.heads, gt_most);

@@ -897,15 +897,16 @@ def test_mfma_attention_first_keys_far_below_zero(gpu, hd, page, window):
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(8, 2, 128, 16, 0), (8, 1, 64, 32, 0), (4, 1, 96, 8, 150), (16, 2, 32, 64, 0),
                                                    (8, 2, 128, 128, 0), (4, 2, 64, 256, 100)])
 def test_prefill_attention_every_cut(gpu, nh, nkv, hd, page, window):
-    """The launcher cuts a prefill by the size of the step (tiles in pairs, 1, 2 or 4 heads a wavefront, one or two
-    head groups a workgroup, keys staged in LDS or not); small cases would only ever see one cut, so each is
-    asked for here, on portions that start inside a context, end inside a tile and share a step."""
+    """The launcher cuts a prefill by the size of the step (tiles in pairs, unpaired sequence by sequence or unpaired
+    with the tiles slowest over the grid; 1, 2 or 4 heads a wavefront, one or two head groups a workgroup, keys
+    staged in LDS or not); small cases would only ever see one cut, so each is asked for here, on portions that
+    start inside a context, end inside a tile and share a step."""
     seqs = [(333, 333), (500, 70), (1, 1), (129, 128), (64, 64), (700, 450)]
     group = nh // nkv
     most = 4 if hd <= 64 and group % 4 == 0 else 2
     base = None
     for staged in (1, 0):
-        for paired in (1, 0):
+        for paired in (1, 0, 2):
             for heads in (1, 2, 4):
                 for groups in (1, 2):
                     if heads > most or (groups == 2 and (not staged or group % (2 * heads))):
@@ -929,6 +930,20 @@ def test_prefill_attention_far_into_its_context(gpu, nh, nkv, hd, page):
         close(out, ref, torch.bfloat16)
         fixed, _ = paged_case(gpu, torch.bfloat16, nh, nkv, hd, page, seqs, 0, seed=11, kernel="mfma", cut=(1, 1, 1, 1))
         assert torch.equal(out, fixed)
+
+
+def test_prefill_attention_of_a_few_prompts(gpu):
+    """Two to six prompts a step take a branch of their own (pairs only in whole rounds, else unpaired with every
+    prompt's long tiles first): sizes that reach each of its cuts, prompts of unequal length among them."""
+    for seqs in ([(512, 512)] * 3, [(512, 512)] * 4, [(500, 500), (130, 130), (512, 512), (64, 64), (333, 333), (1, 1)],
+                 [(1024, 1024)] * 2, [(1024, 1024), (700, 700), (1000, 1000)], [(2048, 2048)] * 2):
+        out, ref = paged_case(gpu, torch.bfloat16, 32, 8, 128, 16, seqs, 0, seed=13, kernel="mfma")
+        close(out, ref, torch.bfloat16)
+        fixed, _ = paged_case(gpu, torch.bfloat16, 32, 8, 128, 16, seqs, 0, seed=13, kernel="mfma", cut=(1, 1, 1, 1))
+        assert torch.equal(out, fixed)
+    for nh, nkv in ((40, 8), (16, 8)):
+        out, ref = paged_case(gpu, torch.bfloat16, nh, nkv, 128, 16, [(512, 512), (300, 300), (512, 512)], 0, seed=14, kernel="mfma")
+        close(out, ref, torch.bfloat16)
 
 
 def test_prefill_attention_refuses_a_cut_the_shape_does_not_take(gpu):
