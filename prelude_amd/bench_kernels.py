@@ -1,6 +1,6 @@
 """Times single kernels against their rooflines on one MI355X.
 
-    python -m prelude_amd.bench_kernels [stream] [gemm] [tall] [dispatch] [cuts] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
+    python -m prelude_amd.bench_kernels [stream] [gemm] [tall] [dispatch] [normed] [cuts] [decode] [prefill] [elementwise] [sampling] [--shape 4b|8b|32b]
 
 Each line gives the kernel's time (device events around repeated launches,
 operands rotated over copies larger than the caches where the kernel streams
@@ -214,6 +214,26 @@ def bench_dispatch(dev, shape) -> None:
         del rows, lws
 
 
+def bench_normed(dev, shape) -> None:
+    """The residual add + RMSNorm and the gated product behind it at 1 to 16 rows: the two kernels apart (the product
+    as ``linear_gated`` dispatches it) against the one kernel that does both, inside a graph, weights from memory."""
+    h, inter = shape[0], shape[1]
+    n, k = 2 * inter, h
+    copies = max(3, min(12, int(700e6 // (n * k * 2))))
+    rows = [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+    lws = [K.LinearWeight(r, K.pack_tiles(r)) for r in rows]
+    gain = torch.ones(k, device=dev)
+    for m in (1, 2, 4, 6, 8, 12, 16):
+        x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+        res = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+        apart = graph_time([(lambda w=w: K.linear_gated(K.rmsnorm(x, gain, 1e-6, residual=res), w, "silu")) for w in lws])
+        if not K.gated_after_norm_supported(x, res, lws[0]):
+            print(f"norm + gate_up [{n:6d} x {k:6d}] M={m:4d}: apart {apart:7.1f} us  (the one kernel does not take this)", flush=True)
+            continue
+        fused = graph_time([(lambda w=w: K.linear_gated_after_norm(x, res, gain, 1e-6, w, "silu")) for w in lws])
+        print(f"norm + gate_up [{n:6d} x {k:6d}] M={m:4d}: apart {apart:7.1f} us  in one kernel {fused:7.1f} us", flush=True)
+
+
 def bench_cuts(dev, shape, page: int = 16) -> None:
     """The prefill attention as its launcher cuts the work against every cut forced (tiles paired, unpaired, or
     unpaired with the tiles slowest over the grid; 1 or 2 heads a wavefront, 1 or 2 head groups a workgroup), over
@@ -323,7 +343,7 @@ def bench_sampling(dev, shape) -> None:
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
-    ap.add_argument("what", nargs="*", help="stream, gemm, tall, decode, prefill, elementwise, sampling (default: all these); dispatch, cuts (sweeps, on request)")
+    ap.add_argument("what", nargs="*", help="stream, gemm, tall, decode, prefill, elementwise, sampling (default: all these); dispatch, normed, cuts (sweeps, on request)")
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES))
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -335,7 +355,7 @@ def main() -> int:
     print(f"Qwen3-{args.shape.upper()} shapes: hidden {shape[0]}, intermediate {shape[1]}, {shape[2]} heads, "
           f"{shape[3]} KV heads, head_dim {shape[4]}, vocabulary {shape[5]}")
     for name in todo:
-        {"stream": bench_stream, "gemm": bench_gemm, "tall": bench_tall, "dispatch": bench_dispatch, "cuts": bench_cuts, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
+        {"stream": bench_stream, "gemm": bench_gemm, "tall": bench_tall, "dispatch": bench_dispatch, "normed": bench_normed, "cuts": bench_cuts, "decode": bench_decode, "prefill": bench_prefill, "elementwise": bench_elementwise,
          "sampling": bench_sampling}[name](dev, shape)
     return 0
 

@@ -70,6 +70,10 @@ int pa_gemm_mid_slices(int n, int k);
 long pa_gemm_mid_parts(int m, int n, int slices);
 int pa_gemm_mid(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
                 float* parts, int m, int n, int k, long ldx, long ldc, int slices, int waves);
+// pa_gemm_mid's gated product of up to 16 rows with the residual add and RMSNorm in front of it, done as X is staged:
+// res_out = x + res (another buffer than res), c = act(gate) * up of rmsnorm(x + res; gain, eps) W^T.
+int pa_gemm_mid_normed(void* stream, int epilogue, const void* x, const void* res, const float* gain, float eps,
+                       void* res_out, const void* w, void* c, int m, int n, int k, long ldx, long ldc, int waves);
 // C = X W^T for any number of rows from the weight in tiles, the output tiled both ways (gemm_tall.hip): 16 mt rows
 // of X by 64 nt rows of W a workgroup (mt, nt = 0, 0: the launcher's choice, what pa_gemm_tall_shape puts into
 // out[0], out[1]).  epilogue 0: C (+ bias) in bfloat16; 1: C[m, n/2] = silu(gate) * up.  slices > 1 (epilogue 0): parts

@@ -43,15 +43,27 @@ __device__ __forceinline__ MidFrag mid_load_w(const bf16* tile, int step, int la
 
 enum MidEpilogue : int { kMidPlain = 0, kMidSiluMul = 1, kMidSlices = 2 };
 
+// The residual add and RMSNorm in front of the product, done as X is staged (NORM kernels): X is `x` + `res`, summed
+// in 32-bit; the sum rounded once is the new residual (`res_out`, another buffer than `res`: every workgroup reads
+// `res`, the first one writes `res_out`), the sum times the norm's gain is what goes to LDS, and the row's scale
+// rsqrt(mean of squares + eps), which is the same for all its columns, is applied to the finished sums of products.
+// Every workgroup sees all of K (no slices), so each forms the rows' sums of squares itself, in a fixed order.
+struct MidNorm {
+  const bf16* res;
+  const float* gain;
+  bf16* res_out;
+  float eps;
+};
+
 // MT tiles of 16 rows of X; KC columns of X a chunk (a multiple of 64): KC / 64 steps between two barriers; WN
 // wavefronts a workgroup, a tile of 16 rows of W each.
-template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI>
+template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI, bool NORM = false>
 __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __restrict__ x,
                                                                        const bf16* __restrict__ w,
                                                                        const float* __restrict__ bias,
                                                                        TC* __restrict__ c, float* __restrict__ parts,
                                                                        int m, int n, int k, long ldx, long ldc,
-                                                                       int steps_per_slice, int act) {
+                                                                       int steps_per_slice, int act, MidNorm nm = MidNorm{}) {
   constexpr int SPC = KC / 64;                  // steps a chunk
   constexpr int CPR = DEPTH / SPC;              // chunks the ring of W steps spans
   static_assert(DEPTH % SPC == 0 && CPR >= 1, "the ring holds whole chunks");
@@ -64,6 +76,8 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
   constexpr bool EVEN = ROWS * PPR % THREADS == 0;               // else the last piece of the later threads is none
   extern __shared__ __align__(16) unsigned char mid_lds[];
   bf16 (*xs)[ROWS][ROW] = reinterpret_cast<bf16 (*)[ROWS][ROW]>(mid_lds);   // two buffers
+  // NORM: behind them a row's sums of squares, one per piece of a chunk's row (each from one thread)
+  float (*ssl)[PPR] = reinterpret_cast<float (*)[PPR]>(mid_lds + 2 * sizeof(bf16) * ROWS * ROW);
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
@@ -93,21 +107,60 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
   // loads than the step at hand needs anyway (loads come back in the order they were asked for: one wait for a
   // whole chunk's pieces at the chunk's end would drain the ring of weight steps each time).
   bf16x8 staged[PIECES];
+  bf16x8 staged_r[NORM ? PIECES : 1];      // NORM: the residual's piece, the gain's eight columns, where they belong
+  float4 staged_g[NORM ? PIECES : 1][2];
+  int staged_at[NORM ? PIECES : 1];
+  float ssp[NORM ? PIECES : 1];            // this thread's share of its rows' sums of squares
+  if constexpr (NORM) {
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) ssp[j] = 0.f;
+  }
   auto stage_load = [&](int chunk, int q0, int q1) {
     const int k0 = (s_begin + chunk * SPC) * 64;
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
       if (j < q0 * PIECES / SPC || j >= q1 * PIECES / SPC) continue;
       const int at = k0 + col[j];
-      staged[j] = *reinterpret_cast<const bf16x8*>(src[j] + (at + 8 <= k ? at : 0));
+      const int from = at + 8 <= k ? at : 0;
+      staged[j] = *reinterpret_cast<const bf16x8*>(src[j] + from);
+      if constexpr (NORM) {
+        staged_r[j] = *reinterpret_cast<const bf16x8*>(nm.res + (src[j] - x) + from);
+        staged_g[j][0] = *reinterpret_cast<const float4*>(nm.gain + from);
+        staged_g[j][1] = *reinterpret_cast<const float4*>(nm.gain + from + 4);
+        staged_at[j] = at + 8 <= k ? at : -1;
+      }
     }
   };
-  auto stage_store = [&](int buf, int q0, int q1) {
+  // `fresh`: the chunk is stored for the first time (the last chunk is staged again while the ring of W steps runs
+  // out: its squares must count once, and the new residual is written once)
+  auto stage_store = [&](int buf, int q0, int q1, bool fresh = true) {
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
       if (j < q0 * PIECES / SPC || j >= q1 * PIECES / SPC) continue;
       const int p = threadIdx.x + j * THREADS;
-      if (EVEN || j + 1 < PIECES || p < ROWS * PPR) *reinterpret_cast<bf16x8*>(&xs[buf][p / PPR][col[j]]) = staged[j];
+      if (!(EVEN || j + 1 < PIECES || p < ROWS * PPR)) continue;
+      if constexpr (NORM) {
+        const int row = p / PPR;
+        const float gn[8] = {staged_g[j][0].x, staged_g[j][0].y, staged_g[j][0].z, staged_g[j][0].w,
+                             staged_g[j][1].x, staged_g[j][1].y, staged_g[j][1].z, staged_g[j][1].w};
+        bf16x8 sum, scaled;
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float s = to_f32(staged[j][i]) + to_f32(staged_r[j][i]);
+          sq += s * s;
+          sum[i] = from_f32<bf16>(s);
+          scaled[i] = from_f32<bf16>(s * gn[i]);
+        }
+        const bool counts = fresh && row < m && staged_at[j] >= 0;
+        if (counts) {
+          ssp[j] += sq;
+          if (blockIdx.x == 0) *reinterpret_cast<bf16x8*>(nm.res_out + (size_t)row * ldx + staged_at[j]) = sum;
+        }
+        *reinterpret_cast<bf16x8*>(&xs[buf][row][col[j]]) = scaled;
+      } else {
+        *reinterpret_cast<bf16x8*>(&xs[buf][p / PPR][col[j]]) = staged[j];
+      }
     }
   };
 
@@ -149,7 +202,7 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
         MidFrag wc = wbuf[u * SPC + ss];
         // the step that takes this slot of the ring next; past the slice's end the last step again, never used
         wbuf[u * SPC + ss] = mid_load_w(wtile, s + DEPTH < s_end ? s + DEPTH : last, lane);
-        stage_store(buf ^ 1, ss, ss + 1);
+        stage_store(buf ^ 1, ss, ss + 1, ch + 1 < nchunks);
         stage_load(ahead, ss, ss + 1);
         if (ss + 1 < SPC) load_x(buf, ss + 1, xf[(ss + 1) & 1]);   // the next step's, under this step's products
         if (s >= s_end) {   // a step past the slice's end counts nothing: zeros for W, and no branch around the products
@@ -165,6 +218,22 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
       __syncthreads();
     }
   }
+  float inv[NORM ? MT : 1];
+  if constexpr (NORM) {
+    // a row's squares: one sum per piece of a chunk's row and thread, added in the pieces' order
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int p = threadIdx.x + j * THREADS;
+      if (EVEN || j + 1 < PIECES || p < ROWS * PPR) ssl[p / PPR][p % PPR] = ssp[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float total = 0.f;
+      for (int i = 0; i < PPR; ++i) total += ssl[16 * t + r][i];
+      inv[t] = rsqrtf(total / (float)k + nm.eps);
+    }
+  }
   if (!n_ok) return;
   // lane (g, r) holds four consecutive n of token 16 t + r
   const int nb = 16 * tile + 4 * g;
@@ -172,6 +241,10 @@ __global__ __launch_bounds__(WN* kWave, 2) void gemm_mid_kernel(const bf16* __re
   for (int t = 0; t < MT; ++t) {
     const int mi = 16 * t + r;
     if (mi >= m) continue;
+    if constexpr (NORM) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[t][i] *= inv[t];
+    }
     if (EPI == kMidSlices) {
       float* dst = parts + ((size_t)blockIdx.y * m + mi) * n + nb;
       if (nb + 3 < n && n % 4 == 0) {
@@ -234,18 +307,18 @@ __global__ void sum_slices_kernel(const float* __restrict__ parts, T* __restrict
   }
 }
 
-template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI>
+template <int MT, int KC, int DEPTH, int WN, typename TC, int EPI, bool NORM = false>
 int launch_mid(hipStream_t st, const void* x, const void* w, const float* bias, void* c, float* parts, int m, int n, int k,
-               long ldx, long ldc, int slices, int act) {
+               long ldx, long ldc, int slices, int act, MidNorm nm = MidNorm{}) {
   const int tiles = (n + 15) / 16, steps = (k + 63) / 64;
   const int sps = (steps + slices - 1) / slices;
-  constexpr size_t lds = 2 * (size_t)(16 * MT) * (KC + 8) * sizeof(bf16);
-  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI>),
+  constexpr size_t lds = 2 * (size_t)(16 * MT) * (KC + 8) * sizeof(bf16) + (NORM ? (size_t)(16 * MT) * (KC / 8) * sizeof(float) : 0);
+  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI, NORM>),
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (allowed != hipSuccess) return pa::fail("gemm_mid: %zu bytes of LDS refused: %s", lds, hipGetErrorString(allowed));
   dim3 grid((tiles + WN - 1) / WN, (steps + sps - 1) / sps);
-  hipLaunchKernelGGL((gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI>), grid, dim3(WN * kWave), lds, st, (const bf16*)x,
-                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps, act);
+  hipLaunchKernelGGL((gemm_mid_kernel<MT, KC, DEPTH, WN, TC, EPI, NORM>), grid, dim3(WN * kWave), lds, st, (const bf16*)x,
+                     (const bf16*)w, bias, (TC*)c, parts, m, n, k, ldx, ldc, sps, act, nm);
   return check_launch("gemm_mid");
 }
 
@@ -324,6 +397,37 @@ extern "C" int pa_gemm_mid_slices(int n, int k) {
   int s = 1;
   while (s < most && blocks * s < 256 && steps / (2 * s) >= 8) s *= 2;
   return s;
+}
+
+// The gated product of up to 16 rows with the residual add and RMSNorm in front of it (see MidNorm):
+// res_out[m, k] = x + res (rounded once), c[m, n/2] = act(gate) * up of rmsnorm(x + res; gain, eps) W^T.  x, res and
+// res_out have the row stride ldx; res_out must be another buffer than res and x.  epilogue 1 + a as in pa_gemm_mid.
+extern "C" int pa_gemm_mid_normed(void* stream, int epilogue, const void* x, const void* res, const float* gain, float eps,
+                                  void* res_out, const void* w, void* c, int m, int n, int k, long ldx, long ldc,
+                                  int waves) {
+  if (m == 0 || n == 0) return 0;
+  PA_REQUIRE(m > 0 && m <= 16 && n > 0 && k > 0, "gemm_mid_normed: bad sizes m=%d (up to 16) n=%d k=%d", m, n, k);
+  PA_REQUIRE(k % 8 == 0 && ldx % 8 == 0 && ldx >= k, "gemm_mid_normed: k=%d and the row stride %ld must be multiples of 8, the stride at least k",
+             k, ldx);
+  PA_REQUIRE(x && res && gain && res_out && w && c, "gemm_mid_normed: an operand is missing");
+  PA_REQUIRE(res_out != res && res_out != x, "gemm_mid_normed: the new residual needs a buffer of its own");
+  PA_REQUIRE(epilogue >= 1 && epilogue <= kActCount && n % 2 == 0, "gemm_mid_normed: a gated epilogue (1 + activation) and an even n");
+  PA_REQUIRE(ldc >= n / 2, "gemm_mid_normed: output row stride %ld is too small", ldc);
+  PA_REQUIRE(waves == 0 || waves == 3 || waves == 4 || waves == 5 || waves == 6 || waves == 8,
+             "gemm_mid_normed: %d wavefronts a workgroup (3, 4, 5, 6, 8, or 0 to let the launcher choose)", waves);
+  hipStream_t st = (hipStream_t)stream;
+  const MidNorm nm{(const bf16*)res, gain, (bf16*)res_out, eps};
+  const int act = epilogue - 1;
+#define PA_NORMED(WN) \
+  return launch_mid<1, 256, 4, WN, bf16, kMidSiluMul, true>(st, x, w, nullptr, c, nullptr, m, n, k, ldx, ldc, 1, act, nm)
+  switch (waves ? waves : mid_waves(n, 1)) {
+    case 3: PA_NORMED(3);
+    case 5: PA_NORMED(5);
+    case 6: PA_NORMED(6);
+    case 8: PA_NORMED(8);
+    default: PA_NORMED(4);
+  }
+#undef PA_NORMED
 }
 
 // Floats of `parts` a product of m rows cut into `slices` needs.

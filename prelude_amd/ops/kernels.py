@@ -685,6 +685,52 @@ def linear_gated(x: torch.Tensor, w, activation: str = "silu") -> torch.Tensor:
     return silu_mul(linear(x, w), activation)
 
 
+# The residual add and RMSNorm in front of the gated product, inside that product (``gemm_mid`` stages X through LDS
+# once per workgroup, and there are a few hundred workgroups, so adding the residual and multiplying by the gain as
+# it stages costs little; the row's scale is applied to the finished sums): one kernel less in a decode step's layer.
+# For up to 16 rows whose mixer output comes as a tensor, and weights of 40 M to 200 M elements: measured against
+# the two kernels apart it gains 1.3 to 3 us at [19456, 2560], 2.3 to 3.8 us at [24576, 4096], 2.5 us up to 8 rows
+# at [34816, 5120] (nothing at 12 rows, and it loses 1.5 us at 16), and loses 0.3 to 1.6 us at [6144, 1024] and
+# [12288, 2048], where the streaming kernel is the better product.
+NORMED_GATED = True              # ``set_normed_gated``: off runs the norm and the product apart (measurements)
+NORMED_GATED_MAX_ROWS = 16
+NORMED_GATED_MAX_ROWS_LARGE = 12   # ... for weights of more than GATED_TILED_ELEMENTS elements
+
+
+def set_normed_gated(on: bool) -> None:
+    global NORMED_GATED
+    NORMED_GATED = bool(on)
+
+
+def gated_after_norm_supported(x, residual, w, activation: str = "silu") -> bool:
+    """Whether ``linear_gated_after_norm`` takes these operands (else: the norm, then ``linear_gated``)."""
+    if not (NORMED_GATED and MID_PRODUCTS and isinstance(x, torch.Tensor) and isinstance(residual, torch.Tensor)
+            and isinstance(w, LinearWeight) and w.tiles is not None and activation in GATE_ACTIVATIONS):
+        return False
+    m, k = x.shape
+    return (x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 and residual.shape == x.shape and x.is_contiguous()
+            and residual.is_contiguous() and k % 8 == 0 and w.tiles.n % 2 == 0
+            and GATED_SMALL_ELEMENTS <= w.tiles.n * k <= GATED_LARGE_ELEMENTS
+            and 1 <= m <= (NORMED_GATED_MAX_ROWS if w.tiles.n * k <= GATED_TILED_ELEMENTS else NORMED_GATED_MAX_ROWS_LARGE))
+
+
+def linear_gated_after_norm(x: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor, eps: float, w,
+                            activation: str = "silu", waves: int = 0):
+    """(residual + x rounded once, act(h Wg^T) * (h Wu^T)) for h = rmsnorm(residual + x; gain, eps): the residual add,
+    the norm and the gated product in one kernel.  The new residual is a tensor of its own."""
+    _dev(x, residual, gain, w.tiles.data)
+    _f32(gain, "gain")
+    m, k = x.shape
+    n = w.tiles.n
+    if gain.shape != (k,) or w.tiles.k != k:
+        raise NativeError(f"linear_gated_after_norm: x {tuple(x.shape)} / gain {tuple(gain.shape)} / w {w.tiles.shape}")
+    res_out = torch.empty_like(residual)
+    out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    check(kernels().pa_gemm_mid_normed(_stream(), 1 + gate_activation_code(activation), _ptr(x), _ptr(residual), _ptr(gain),
+                                       float(eps), _ptr(res_out), _ptr(w.tiles.data), _ptr(out), m, n, k, k, n // 2, int(waves)))
+    return res_out, out
+
+
 def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
     """``linear_gated`` with SiLU, the reference's own feed-forward (crates/prelude-core/src/models/qwen3.rs:429-447)."""
     return linear_gated(x, w, "silu")

@@ -202,12 +202,27 @@ class FeedForward(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_after_norm(self, x, residual, norm: "Norm"):
+        """(new residual, forward(norm of residual + x)): what a block asks for behind a mixer.  A feed-forward whose
+        first kernel can take the add and the norm in (it learns the norm's kind from ``norm.as_rms()``) does so
+        here; this is the plain order."""
+        if not norm.TAKES_SLICE_SUMS:
+            from ..ops.kernels import as_tensor
+            x = as_tensor(x)
+        residual, h = norm.forward_residual(x, residual)
+        return residual, self.forward(h)
+
 
 class Norm(Part):
     # True for a norm whose three methods also take a product that was left as partial sums of slices of its
     # inner size (``ops.kernels.SliceSums``) in place of ``x``, adding the slices as it loads them; a block
     # hands other norms the finished tensor.
     TAKES_SLICE_SUMS = False
+
+    def as_rms(self):
+        """(gain, eps) if this norm is exactly y = x * rsqrt(mean(x^2) + eps) * gain over the whole row with the
+        sum taken of the unrounded residual + x, else None: a kernel that follows may then do the norm itself."""
+        return None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError

@@ -27,8 +27,5 @@ class PreNormBlock(Block):
             hidden = K.as_tensor(hidden)
         residual, h = self.input_norm.forward_residual(hidden, residual)
         h = self.mixer.forward(h, step, cache, write_cache)
-        if not self.post_mixer_norm.TAKES_SLICE_SUMS:
-            h = K.as_tensor(h)
-        residual, h = self.post_mixer_norm.forward_residual(h, residual)
-        h = self.ffn.forward(h)
+        residual, h = self.ffn.forward_after_norm(h, residual, self.post_mixer_norm)
         return h, residual

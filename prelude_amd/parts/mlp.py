@@ -44,3 +44,11 @@ class GatedMLP(FeedForward):
 
     def forward(self, x):
         return K.linear(K.linear_gated(x, self.gate_up, self.activation), self.down, slices_ok=True)
+
+    def forward_after_norm(self, x, residual, norm):
+        # a few rows behind an RMS norm: the add and the norm ride in the gated product's staging of X
+        rms = norm.as_rms() if residual is not None else None
+        if rms is None or not K.gated_after_norm_supported(x, residual, self.gate_up, self.activation):
+            return super().forward_after_norm(x, residual, norm)
+        residual, h = K.linear_gated_after_norm(x, residual, rms[0], rms[1], self.gate_up, self.activation)
+        return residual, K.linear(h, self.down, slices_ok=True)

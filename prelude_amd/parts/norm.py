@@ -32,6 +32,9 @@ class RMSNorm(Norm):
     def load(self, tensors, dtype, device):
         self.weight = tensors["weight"]
 
+    def as_rms(self):
+        return self.weight, self.eps
+
     def forward(self, x):
         return K.rmsnorm(x, self.weight, self.eps)
 

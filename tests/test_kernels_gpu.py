@@ -230,6 +230,57 @@ def test_gemm_mid(gpu, m, n, k, slices):
             assert torch.equal(K().gemm_mid(xd, tiles, bd, slices=slices, waves=waves).parts, ss.parts), f"{waves} wavefronts, slices"
 
 
+@pytest.mark.parametrize("m,n,k,eps", [(8, 19456, 2560, 1e-6), (1, 64, 64, 1e-5), (16, 200, 4096, 1e-6), (5, 330, 1000, 3e-4),
+                                       (13, 36, 72, 1e-6), (9, 1288, 520, 1e-2), (3, 6144, 1024, 1e-6), (16, 512, 256, 1e-6)])
+def test_gated_product_behind_its_norm(gpu, m, n, k, eps):
+    """Residual add, RMSNorm and gated product in one kernel: the new residual is the sum rounded once, the norm is
+    taken of the unrounded sum, and the product is that of the two kernels apart."""
+    x, res = rnd(m, k, dtype=torch.bfloat16, scale=0.7), rnd(m, k, dtype=torch.bfloat16, seed=5, scale=3.0)
+    res[m - 1] *= 40.0          # a row far larger than the others: every row has a scale of its own
+    gain = 1 + 0.3 * rnd(k, seed=3)
+    w = rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05)
+    total = x.double() + res.double()
+    h = pm.rms_norm(total, gain.double(), eps)
+    g = h @ w.double().T
+    ref = pm.silu(g[:, 0::2]) * g[:, 1::2]
+    lw = K().LinearWeight(w.to(gpu), K().pack_tiles(w.to(gpu)))
+    xd, resd, gd = x.to(gpu), res.to(gpu), gain.to(gpu)
+    # the block takes it where it measured faster than the two kernels apart: weights of 40 M elements and more
+    assert K().gated_after_norm_supported(xd, resd, lw) == (n * k >= 40 << 20)
+    new_res, y = K().linear_gated_after_norm(xd, resd, gd, eps, lw)
+    assert torch.equal(resd.cpu(), res) and torch.equal(xd.cpu(), x)          # the inputs stay as they were
+    assert torch.equal(new_res.cpu(), (x.float() + res.float()).to(torch.bfloat16))
+    close(y, ref, torch.bfloat16, bf16=1.25e-2)
+    # beside the two kernels apart: the same residual, a product within rounding of it
+    apart_res = resd.clone()
+    apart = K().linear_gated(K().rmsnorm(xd, gd, eps, residual=apart_res), lw)
+    assert torch.equal(apart_res, new_res)
+    close(y, apart.double().cpu(), torch.bfloat16, bf16=1.25e-2)
+    # a row's result depends neither on the other rows nor on how many wavefronts share a workgroup
+    one_res, one = K().linear_gated_after_norm(xd[m - 1:].contiguous(), resd[m - 1:].contiguous(), gd, eps, lw)
+    assert torch.equal(one[0], y[m - 1]) and torch.equal(one_res[0], new_res[m - 1])
+    for waves in (3, 4, 5, 6, 8):
+        r2, y2 = K().linear_gated_after_norm(xd, resd, gd, eps, lw, waves=waves)
+        assert torch.equal(y2, y) and torch.equal(r2, new_res), f"{waves} wavefronts"
+    # what lies behind the rows is not the kernel's to read: NaN there must not show
+    behind_x = torch.full((m + 8, k), float("nan"), dtype=torch.bfloat16, device=gpu)
+    behind_r = torch.full((m + 8, k), float("nan"), dtype=torch.bfloat16, device=gpu)
+    behind_x[:m], behind_r[:m] = xd, resd
+    r3, y3 = K().linear_gated_after_norm(behind_x[:m], behind_r[:m], gd, eps, lw)
+    assert torch.equal(y3, y) and torch.equal(r3, new_res)
+    # the other activation, and what it does not take
+    import torch.nn.functional as F
+    _, y4 = K().linear_gated_after_norm(xd, resd, gd, eps, lw, "gelu_tanh")
+    close(y4, F.gelu(g[:, 0::2], approximate="tanh") * g[:, 1::2], torch.bfloat16, bf16=1.25e-2)
+    assert not K().gated_after_norm_supported(torch.zeros(17, k, dtype=torch.bfloat16, device=gpu),
+                                              torch.zeros(17, k, dtype=torch.bfloat16, device=gpu), lw)
+    assert not K().gated_after_norm_supported(xd.float(), resd.float(), lw)
+    from prelude_amd._native import NativeError
+    with pytest.raises(NativeError, match="buffer of its own"):
+        K().check(K().kernels().pa_gemm_mid_normed(None, 1, xd.data_ptr(), resd.data_ptr(), gd.data_ptr(), eps, resd.data_ptr(),
+                                                   lw.tiles.data.data_ptr(), y.data_ptr(), m, n, k, k, n // 2, 0))
+
+
 @pytest.mark.parametrize("m,n,k,slices", [(129, 2560, 4096, 4), (300, 331, 1000, 1), (256, 200, 4096, 2), (513, 2560, 2560, 1),
                                           (192, 6144, 2560, 4), (1030, 72, 640, 1), (260, 1000, 2560, 1), (140, 36, 72, 1),
                                           (576, 2560, 9728, 4), (2, 64, 64, 1)])

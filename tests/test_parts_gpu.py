@@ -76,6 +76,45 @@ def test_gated_mlp_part(gpu, dtype):
         build_part("ffn", "gated_mlp", dict(hidden_size=8, intermediate_size=8, activation="relu"))
 
 
+@pytest.mark.parametrize("hidden,inter,rows,one_kernel", [(72, 200, 9, False), (2560, 8200, 5, True), (2560, 8200, 17, False)])
+def test_gated_mlp_behind_a_norm(gpu, hidden, inter, rows, one_kernel):
+    """What a block asks of its feed-forward behind the mixer: (residual + x, forward(norm(residual + x))).  At
+    small sizes and at more than 16 rows that is the norm's kernel and then the feed-forward's; a few rows at the
+    widths of real models take the add and the norm into the gated product.  Both against the plain functions."""
+    from prelude_amd.ops import kernels as K
+    from prelude_amd.parts import build_part
+    m = build_part("ffn", "gated_mlp", dict(hidden_size=hidden, intermediate_size=inter))
+    norm = build_part("norm", "rms_norm", dict(size=hidden, eps=1e-5))
+    w = {"gate_proj.weight": rnd(inter, hidden, seed=1, scale=0.03), "up_proj.weight": rnd(inter, hidden, seed=2, scale=0.03),
+         "down_proj.weight": rnd(hidden, inter, seed=3, scale=0.03)}
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    gain = 1 + 0.2 * rnd(hidden, seed=4)
+    m.load({k: v.to(gpu) for k, v in w.items()}, torch.bfloat16, gpu)
+    norm.load({"weight": gain.to(gpu)}, torch.bfloat16, gpu)
+    x, res = rnd(rows, hidden, seed=5).to(torch.bfloat16), rnd(rows, hidden, seed=6, scale=4.0).to(torch.bfloat16)
+    xd, resd = x.to(gpu), res.to(gpu)
+    assert K.gated_after_norm_supported(xd, resd, m.gate_up) == one_kernel
+    new_res, y = m.forward_after_norm(xd, resd, norm)
+    total = x.double() + res.double()
+    ref = pm.swiglu(pm.rms_norm(total, gain.double(), 1e-5), *(w[k].double() for k in ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
+    assert torch.equal(new_res.cpu(), (x.float() + res.float()).to(torch.bfloat16))
+    y = K.as_tensor(y)
+    assert float((y.double().cpu() - ref).abs().max()) < 2e-2 * max(1.0, float(ref.abs().max()))
+    # a norm that is not that formula is never taken in: the plain order, which asks nothing of the norm but its own methods
+    class Doubled(type(norm)):
+        def as_rms(self):
+            return None
+
+        def forward_residual(self, x, residual):
+            residual, h = super().forward_residual(x, residual)
+            return residual, h * 2
+    other = Doubled(hidden, 1e-5)
+    other.load({"weight": gain.to(gpu)}, torch.bfloat16, gpu)
+    _, y2 = m.forward_after_norm(xd, res.to(gpu), other)
+    ref2 = pm.swiglu(2 * pm.rms_norm(total, gain.double(), 1e-5), *(w[k].double() for k in ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
+    assert float((K.as_tensor(y2).double().cpu() - ref2).abs().max()) < 2e-2 * max(1.0, float(ref2.abs().max()))
+
+
 def test_embedding_and_head_parts(gpu):
     from prelude_amd.parts import build_part
     # crates/prelude-core/tests/modules.rs:245-271: arange(12).reshape(4, 3), ids [2, 0, 3]

@@ -101,6 +101,39 @@ def test_twenty_requests_decode_together(gpu):
     assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
 
 
+def test_the_norm_inside_the_gated_product(gpu, monkeypatch):
+    """Up to 16 rows at these widths the residual add and the norm behind the attention run inside the gated product:
+    eight requests decode together with it and without it, both against the plain implementation, and the
+    kernel is seen to run in the one case and not in the other."""
+    from prelude_amd.ops import kernels as K
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref, _ = wide_model()
+    calls = []
+    inner = K.linear_gated_after_norm
+    monkeypatch.setattr(K, "linear_gated_after_norm", lambda *a, **kw: (calls.append(a[0].shape[0]), inner(*a, **kw))[1])
+    starts = [5 + 9 * i for i in range(8)]
+    try:
+        for on in (True, False):
+            K.set_normed_gated(on)
+            calls.clear()
+            r = TraceRunner(folder, "bfloat16", 8 * 96, page_size=16)
+            for i, s in enumerate(starts):
+                r.step([{"id": f"r{i}", "tokens": toks[:s], "want": []}])
+            seen = len(calls)
+            rows = [[] for _ in starts]
+            for k in range(4):
+                out = r.step([{"id": f"r{i}", "tokens": [toks[s + k]], "want": [0]} for i, s in enumerate(starts)])
+                for i in range(len(starts)):
+                    rows[i].append(out[i:i + 1])
+            for i, s in enumerate(starts):
+                check(np.concatenate(rows[i]), ref[s:s + 4], "bfloat16", f"norm inside the product {on}, request {i}")
+            # (a step replayed from a graph does not come by here again: at least the step that was recorded did)
+            assert (set(calls[seen:]) == {8} and len(calls) - seen >= wide_config()["num_hidden_layers"]) if on else not calls, calls
+            r.step([], [f"r{i}" for i in range(8)])
+    finally:
+        K.set_normed_gated(True)
+
+
 @pytest.mark.parametrize("batch", [33, 64, 100, 128])
 def test_many_requests_decode_together(gpu, batch):
     """Decode steps of 33 to 128 requests at the real widths: the products of 17 to 128 rows (X through LDS, the
