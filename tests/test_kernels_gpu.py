@@ -532,6 +532,18 @@ def test_drawn_products(gpu, seed):
         parts = K().gemm_mid(x3d, tiles, bd, slices=c, waves=waves).parts
         err = float((parts.double().sum(0).cpu() - ref3 - b.double()).abs().max())
         assert err <= tol(torch.float32, ref3, f32=2e-5), f"{what}, rows {m3}, {waves} wavefronts, {c} slices: max error {err:.3e}"
+    # the gated product with the residual add and the norm in front of it, inside it: up to 16 rows
+    m5 = int(rng.choice([1, 8, 15, 16, int(rng.integers(1, 17))]))
+    eps5 = float(rng.choice([1e-6, 1e-5, 1e-3]))
+    x5, res5 = rnd(m5, k, dtype=torch.bfloat16, seed=seed + 9), rnd(m5, k, dtype=torch.bfloat16, seed=seed + 10, scale=float(rng.choice([0.1, 1.0, 30.0])))
+    gain5 = 1 + 0.3 * rnd(k, seed=seed + 11)
+    total5 = x5.double() + res5.double()
+    g5 = pm.rms_norm(total5, gain5.double(), eps5) @ w.double().T
+    new5, y5 = K().linear_gated_after_norm(x5.to(gpu), res5.to(gpu), gain5.to(gpu), eps5, lw, waves=waves)
+    assert torch.equal(new5.cpu(), (x5.float() + res5.float()).to(torch.bfloat16)), f"{what}, rows {m5}: the new residual"
+    want5 = pm.silu(g5[:, 0::2]) * g5[:, 1::2]
+    err = float((y5.double().cpu() - want5).abs().max())
+    assert err <= tol(torch.bfloat16, want5, bf16=1.25e-2), f"{what}, rows {m5}, {waves} wavefronts, norm + SiLU*up: max error {err:.3e}"
     # the product tiled both ways, at a drawn number of rows, shape of workgroup, activation and number of slices
     m4 = int(rng.choice([1, 129, 192, 256, 257, int(rng.integers(1, 700))]))
     x4 = rnd(m4, k, dtype=torch.bfloat16, seed=seed + 7)
