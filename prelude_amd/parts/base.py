@@ -8,14 +8,16 @@ tensors it needs (by local name and shape), receives them, and runs.
 Categories and the interface each must have:
 
 ``norm``      ``forward(x)``, ``forward_residual(x, residual) -> (residual, normed)``,
-              ``forward_rows(x, residual, rows)``
+              ``forward_rows(x, residual, rows)``; ``as_rms() -> (gain, eps) | None`` (given by the base class:
+              None) tells a kernel behind it that it may do the plain RMS formula itself
 ``mixer``/``ffn`` may return their last product as ``ops.kernels.SliceSums`` (``linear(..., slices_ok=True)``):
               only a norm reads it, and one that says ``TAKES_SLICE_SUMS`` adds the slices itself
 ``position``  ``prepare(device)``; what it offers (tables) is between it and the mixers that name it
 ``mixer``     ``cache_spec()`` -> a ``PagedCacheSpec`` (``KVCacheSpec`` or a kind of the mixer's own) | a
               ``SlotCacheSpec`` (``StateSpec``) | ``None``;
               ``forward(x, step, cache, write_cache=True)``
-``ffn``       ``forward(x)``
+``ffn``       ``forward(x)``; ``forward_after_norm(x, residual, norm) -> (residual, out)`` (given by the base class:
+              the norm's ``forward_residual``, then ``forward``) is what a block calls behind its mixer
 ``block``     ``forward(hidden, residual, step, cache, write_cache) -> (hidden, residual)``
 ``embedding`` ``forward(token_ids)``
 ``head``      ``forward(hidden_rows) -> float32 logits``
