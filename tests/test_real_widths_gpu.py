@@ -134,6 +134,46 @@ def test_the_norm_inside_the_gated_product(gpu, monkeypatch):
         K.set_normed_gated(True)
 
 
+def test_graph_replays_equal_eager_steps_at_real_widths(gpu):
+    """Decode steps of one, five and twelve requests at these widths (the streaming products, the gated product with
+    the norm inside it, the decode attention on the raw projection) replayed from graphs give the bits of the same
+    steps run directly, with prompt portions between the replays."""
+    from prelude_amd.config import EngineConfig
+    from prelude_amd.engine import Engine, StepEntry
+    folder, toks, _, _ = wide_model()
+
+    def play(hip_graph):
+        eng = Engine.from_model_dir(folder, EngineConfig(dtype="bfloat16", page_size=16, max_cache_tokens=12 * 96,
+                                                         hip_graph=hip_graph))
+        outs, at = [], {}
+
+        def feed(parts):
+            entries = []
+            for r, n in parts:
+                lo = at.get(r, 0)
+                entries.append(StepEntry(r, toks[lo:lo + n], [n - 1]))
+                at[r] = lo + n
+            outs.append(eng.step(entries).cpu())
+        feed([(0, 30)])
+        for _ in range(4):
+            feed([(0, 1)])
+        feed([(r, 10 + 3 * r) for r in range(1, 5)])
+        for _ in range(4):
+            feed([(r, 1) for r in range(5)])
+        feed([(r, 5 + r) for r in range(5, 12)])
+        for _ in range(4):
+            feed([(r, 1) for r in range(12)])
+        for _ in range(2):
+            feed([(0, 1)])
+        return eng, outs
+
+    eager_eng, eager = play(False)
+    graph_eng, graphed = play(True)
+    assert eager_eng._graphs is None and graph_eng._graphs.captures == 3 and graph_eng._graphs.replays >= 11
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.equal(a, b), f"step {i}: the replay differs from the eager step"
+
+
 @pytest.mark.parametrize("batch", [33, 64, 100, 128])
 def test_many_requests_decode_together(gpu, batch):
     """Decode steps of 33 to 128 requests at the real widths: the products of 17 to 128 rows (X through LDS, the
