@@ -54,6 +54,8 @@ _KERNEL_API = {
     "pa_gemm_mid_slices": (I, [I, I]),
     "pa_gemm_mid_parts": (c_long, [I, I, I]),
     "pa_gemm_mid": (I, [P, I, I, P, P, P, P, P, I, I, I, c_long, c_long, I, I]),
+    "pa_gemm_skinny_slices": (I, [I, I]),
+    "pa_gemm_skinny_sliced": (I, [P, P, P, P, P, I, I, I, c_long, I, I]),
     "pa_gemm_mid_normed": (I, [P, I, P, P, P, F, P, P, P, I, I, I, c_long, c_long, I]),
     "pa_sum_slices": (I, [P, I, P, P, I, c_long]),
     "pa_gemm_tall_shape": (None, [I, I, I, I, IP]),

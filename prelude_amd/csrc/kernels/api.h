@@ -58,6 +58,9 @@ int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, cons
 // C[m, n] = X[m, k] W[n, k]^T for m <= 64 in bfloat16 (32-bit accumulation); out_dtype 0 = float32, 1 = bfloat16.
 // epilogue 0: (+ bias[n]); 1: C[m, n/2] = silu(gate) * up for a weight whose rows alternate gate_j, up_j.
 // tiled 1: w is the weight as pa_pack_tiles lays it out.
+int pa_gemm_skinny_slices(int k, int slices);
+int pa_gemm_skinny_sliced(void* stream, const void* x, const void* w, const float* bias, float* parts, int m, int n, int k,
+                          long ldx, int slices, int waves);
 int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const void* x, const void* w, const float* bias, void* c,
                    int m, int n, int k, long ldx, long ldc, int tiled);
 // C[m, n] = X[m, k] W[n, k]^T for m <= 128 from the weight in tiles, X staged through LDS and W streamed by

@@ -92,21 +92,29 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
                                                                    const bf16* __restrict__ w,
                                                                    const float* __restrict__ bias,
                                                                    TC* __restrict__ c, int m, int n, int k, long ldx,
-                                                                   long ldc, int act) {
+                                                                   long ldc, int act, int steps_per_slice) {
   __shared__ float red[WAVES][NT * MT][kWave][4];
   // the wavefront's number as a scalar: what depends on it (the steps it takes, the loop's end) is then uniform
   // for the compiler too, and a branch on it is a branch, not a mask
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int n0 = blockIdx.x * 16 * NT;
-  const int steps = (k + 63) / 64;
+  // grid.y cuts K into slices of steps_per_slice k-steps, each with an output of its own (32-bit, m * ldc apart) for
+  // a reader that adds them; one slice: all of K
+  const int steps_lo = blockIdx.y * steps_per_slice;
+  const int steps_all = (k + 63) / 64;
+  const int steps = steps_lo + steps_per_slice < steps_all ? steps_lo + steps_per_slice : steps_all;
+  if (gridDim.y > 1) {
+    c += (size_t)blockIdx.y * m * ldc;
+    if (blockIdx.y) bias = nullptr;
+  }
 
   bool n_ok[NT];
   const bf16* wrow[NT];
 #pragma unroll
   for (int u = 0; u < NT; ++u) {
     n_ok[u] = TILED ? n0 + 16 * u < n : n0 + 16 * u + r < n;
-    wrow[u] = TILED ? w + (size_t)(n_ok[u] ? n0 / 16 + u : 0) * steps * 1024
+    wrow[u] = TILED ? w + (size_t)(n_ok[u] ? n0 / 16 + u : 0) * steps_all * 1024
                     : w + (size_t)(n_ok[u] ? n0 + 16 * u + r : 0) * k + 16 * g;
   }
   const bf16* xrow[MT];
@@ -130,7 +138,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
   Frag wbuf[DEPTH][NT], xbuf[DEPTH][MT];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
-    const int s = wave + d * WAVES;
+    const int s = steps_lo + wave + d * WAVES;
     const int sc = s < steps ? s : last;
 #pragma unroll
     for (int u = 0; u < NT; ++u)
@@ -139,7 +147,7 @@ __global__ __launch_bounds__(WAVES* kWave) void gemm_skinny_kernel(const bf16* _
     for (int t = 0; t < MT; ++t)
       xbuf[d][t] = TILED ? load_x_always(xrow[t], sc * 64 + 16 * g, k) : load_frag(xrow[t], s * 64, kk, m_ok[t] && s < steps);
   }
-  for (int s0 = wave; s0 < steps; s0 += WAVES * DEPTH) {
+  for (int s0 = steps_lo + wave; s0 < steps; s0 += WAVES * DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       Frag wc[NT], xc[MT];
@@ -267,11 +275,12 @@ constexpr bool skinny_built() {
 
 template <int MT, int NT, int WV, typename TC, int EPI, bool TILED, int DEPTH>
 int launch_skinny_as(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                     long ldx, long ldc, int act) {
+                     long ldx, long ldc, int act, int slices = 1) {
   if constexpr (skinny_built<MT, TILED, NT, WV>()) {
-    dim3 grid(((n + 15) / 16 + NT - 1) / NT);
+    const int steps = (k + 63) / 64, per = (steps + slices - 1) / slices;
+    dim3 grid(((n + 15) / 16 + NT - 1) / NT, (steps + per - 1) / per);
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WV, TC, EPI, TILED, DEPTH>), grid, dim3(WV * kWave), 0, st,
-                       (const bf16*)x, (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc, act);
+                       (const bf16*)x, (const bf16*)w, bias, (TC*)c, m, n, k, ldx, ldc, act, per);
     return check_launch("gemm_skinny");
   } else {
     return pa::fail("gemm_skinny: no kernel for %d row tiles with %d tiles a workgroup on %d wavefronts (%s weight)", MT,
@@ -281,10 +290,12 @@ int launch_skinny_as(hipStream_t st, const void* x, const void* w, const float* 
 
 template <int MT, typename TC, int EPI, bool TILED, int DEPTH>
 int launch_skinny_depth(hipStream_t st, const void* x, const void* w, const float* bias, void* c, int m, int n, int k,
-                        long ldx, long ldc, int act) {
+                        long ldx, long ldc, int act, int slices = 1, int waves_asked = 0) {
   int nt, waves, depth;
   skinny_shape(m, n, k, MT, TILED, &nt, &waves, &depth);
-#define PA_AS(NT, WV) return launch_skinny_as<MT, NT, WV, TC, EPI, TILED, DEPTH>(st, x, w, bias, c, m, n, k, ldx, ldc, act)
+  if (waves_asked) waves = waves_asked, nt = 1;
+#define PA_AS(NT, WV) \
+  return launch_skinny_as<MT, NT, WV, TC, EPI, TILED, DEPTH>(st, x, w, bias, c, m, n, k, ldx, ldc, act, slices)
 #define PA_WAVES(NT)     \
   switch (waves) {       \
     case 16: PA_AS(NT, 16); \
@@ -384,4 +395,27 @@ extern "C" int pa_gemm_skinny(void* stream, int out_dtype, int epilogue, const v
   if (gated && out_dtype == kBF16)
     return launch_skinny_mt<bf16, kSiluMul>(st, x, w, bias, c, m, n, k, ldx, ldc, act, tiled);
   return pa::fail("gemm_skinny: unsupported output type %d with epilogue %d", out_dtype, epilogue);
+}
+
+// pa_gemm_skinny of up to 16 rows of a tiled weight with K cut into `slices` (the last may be shorter; the launch
+// makes ceil(steps / ceil(steps / slices)) of them, which pa_gemm_skinny_slices tells): parts[slice][m][n] in 32-bit,
+// the bias in slice 0, for a reader that adds the slices in their order (the residual add + RMSNorm does).  A narrow
+// weight has too few tiles to give every compute unit a workgroup; its slices do.  waves: 8 or 16 wavefronts a
+// workgroup, 0 for the launcher's choice by the slice's length.
+extern "C" int pa_gemm_skinny_slices(int k, int slices) {
+  const int steps = (k + 63) / 64;
+  if (slices < 1) slices = 1;
+  const int per = (steps + slices - 1) / slices;
+  return (steps + per - 1) / per;
+}
+extern "C" int pa_gemm_skinny_sliced(void* stream, const void* x, const void* w, const float* bias, float* parts, int m,
+                                     int n, int k, long ldx, int slices, int waves) {
+  if (m == 0 || n == 0) return 0;
+  PA_REQUIRE(m > 0 && m <= 16 && n > 0 && k > 0, "gemm_skinny_sliced: bad sizes m=%d (up to 16) n=%d k=%d", m, n, k);
+  PA_REQUIRE(k % 8 == 0 && ldx % 8 == 0 && ldx >= k, "gemm_skinny_sliced: k=%d and the row stride %ld must be multiples of 8, the stride at least k", k, ldx);
+  PA_REQUIRE(slices >= 1 && slices <= (k + 63) / 64, "gemm_skinny_sliced: %d slices of %d steps", slices, (k + 63) / 64);
+  PA_REQUIRE(waves == 0 || waves == 8 || waves == 16, "gemm_skinny_sliced: %d wavefronts a workgroup (8, 16 or 0)", waves);
+  PA_REQUIRE(x && w && parts, "gemm_skinny_sliced: an operand is missing");
+  if (!waves) waves = ((k + 63) / 64 + slices - 1) / slices >= 128 ? 16 : 8;
+  return launch_skinny_depth<1, float, kPlain, true, 1>((hipStream_t)stream, x, w, bias, parts, m, n, k, ldx, n, 0, slices, waves);
 }

@@ -382,6 +382,23 @@ class SliceSums:
         return out
 
 
+def gemm_skinny_sliced(x: torch.Tensor, w: "TiledWeight", bias: Optional[torch.Tensor] = None, slices: int = 2,
+                       waves: int = 0) -> SliceSums:
+    """``gemm_skinny`` of up to 16 rows with K cut into slices, each a workgroup of its own a tile, left as 32-bit
+    partial sums for a reader that adds them: a narrow weight has too few tiles to give every compute unit work."""
+    _dev(x, w.data, bias)
+    _f32(bias, "bias")
+    m, k = x.shape
+    n = w.shape[0]
+    if x.dtype != torch.bfloat16 or w.shape[1] != k or not 1 <= m <= 16 or (bias is not None and bias.shape != (n,)):
+        raise NativeError(f"gemm_skinny_sliced: x {tuple(x.shape)} {x.dtype} / w {w.shape}")
+    made = int(kernels().pa_gemm_skinny_slices(k, int(slices)))
+    parts = torch.empty((made, m, n), dtype=torch.float32, device=x.device)
+    check(kernels().pa_gemm_skinny_sliced(_stream(), _ptr(x), _ptr(w.data), _ptr(bias), _ptr(parts), m, n, k, k, int(slices),
+                                          int(waves)))
+    return SliceSums(parts, torch.bfloat16)
+
+
 GEMM_MID_MAX_ROWS = 128
 # Where ``linear`` takes the product with X staged in LDS (measured at the shapes of 4B, 8B and 32B models, 17 to
 # 128 rows).  Cut into slices, for a reader that adds them, wherever the weight's shape gives two slices or more:
@@ -578,6 +595,10 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     # with the norm that reads it, at 20 and 24 rows, [2560, 4096] 11.3 and 11.4 us against 12.2 and 13.0, [2048, 2048]
     # 8.7 against 9.0 and 9.2, [5120, 5120] 17.6 and 17.5 against 20.2 and 21.2; [4096, 4096] 14.6 and 14.9 against
     # 13.9 and 14.7 is the one shape the other way round)
+    if SKINNY_SLICED and slices_ok and tiles is not None and k % 8 == 0 and n % 4 == 0 and out_dtype in (None, torch.bfloat16):
+        s = _skinny_slices(m, n, k)
+        if s > 1:
+            return gemm_skinny_sliced(x, tiles, bias, slices=s, waves=8)
     if sliced:
         s = gemm_mid_slices(n, k)
         if s >= MID_MIN_SLICES:
@@ -613,6 +634,33 @@ def linear(x: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
     if out_dtype is not None and out_dtype != y.dtype:
         y = to_f32(y)
     return y
+
+
+# A narrow weight has too few tiles of 16 rows to give every compute unit a workgroup of the streaming kernel (160
+# for 2,560 outputs, 64 for 1,024): for a reader of slices K is cut so that there are 256 to 480 workgroups.  Measured
+# with the norm behind it, inside a graph, against what was dispatched before (us): [2560, 9728] in three slices
+# 16.0 -> 14.9 at 6 rows, 16.8 -> 15.0 at 8, 16.5 -> 15.5 at 10, level at 4 and 12 and behind at 1, 2 and 16;
+# [2048, 6144] in two 9.7 -> 8.9 at one row, 10.5 -> 9.5 at 8, 11.0 -> 9.9 at 16; [1024, 3072] in four 7.0 -> 6.5,
+# 7.8 -> 7.0, 8.8 -> 7.3; [1024, 2048] in four 6.5 -> 6.3, 7.2 -> 6.8, 7.8 -> 7.0; nothing for [2048, 2048], [4096, 4096],
+# [5120, 8192], and for [5120, 5120] at 6 to 8 rows only.
+# (most tiles, slices, least k-steps, rows from, rows to)
+SKINNY_SLICED_SHAPES = ((64, 4, 32, 1, 16), (128, 2, 64, 1, 16), (160, 3, 128, 4, 12))
+SKINNY_SLICED = True    # ``set_skinny_sliced``: off sends these products where they went before (measurements)
+
+
+def set_skinny_sliced(on: bool) -> None:
+    global SKINNY_SLICED
+    SKINNY_SLICED = bool(on)
+
+
+def _skinny_slices(m: int, n: int, k: int) -> int:
+    tiles, steps = (n + 15) // 16, (k + 63) // 64
+    if k >= TILED_LONG_ROWS:      # rows this long have rules of their own (MID_SLICED_MIN_ROWS_LONG), measured at their shapes
+        return 1
+    for most_tiles, slices, least_steps, rows_from, rows_to in SKINNY_SLICED_SHAPES:
+        if tiles <= most_tiles:
+            return slices if steps >= least_steps and rows_from <= m <= rows_to else 1
+    return 1
 
 
 def as_tensor(x):

@@ -462,6 +462,72 @@ def test_gemm_mid_refuses_and_is_dispatched(gpu):
     close(K().linear_silu_mul(xg, lg), pm.silu(ref[:, 0::2]) * ref[:, 1::2], torch.bfloat16, bf16=1.25e-2)
 
 
+@pytest.mark.parametrize("m,n,k,slices", [(8, 2560, 9728, 3), (1, 1024, 3072, 4), (16, 1024, 2048, 4), (5, 200, 520, 2),
+                                          (3, 2048, 6144, 2), (12, 331, 1000, 5), (7, 48, 72, 2)])
+def test_gemm_skinny_in_slices(gpu, m, n, k, slices):
+    """The streaming product of up to 16 rows with K cut into slices, a workgroup a tile and slice, left as 32-bit
+    partial sums: their sum against 64-bit, the bias in the first slice, through the norm that adds them."""
+    x, w, b = rnd(m, k, dtype=torch.bfloat16), rnd(n, k, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(n, seed=2)
+    ref = x.double() @ w.double().T
+    xd, bd = x.to(gpu), b.to(gpu)
+    tiles = K().pack_tiles(w.to(gpu))
+    ss = K().gemm_skinny_sliced(xd, tiles, bd, slices=slices)
+    steps = -(-k // 64)
+    made = -(-steps // -(-steps // slices))
+    assert isinstance(ss, K().SliceSums) and tuple(ss.parts.shape) == (made, m, n) and ss.dtype == torch.bfloat16
+    close(ss.parts.double().sum(0), ref + b.double(), torch.float32, f32=2e-5)
+    close(ss.parts[1:].double().sum(0), (x[:, 64 * -(-steps // slices):].double() @ w[:, 64 * -(-steps // slices):].double().T),
+          torch.float32, f32=2e-5)                                   # the bias is in the first slice alone
+    close(ss.materialize(), ref + b.double(), torch.bfloat16)
+    none = K().gemm_skinny_sliced(xd, tiles, slices=slices)
+    close(none.parts.double().sum(0), ref, torch.float32, f32=2e-5)
+    if n % 4 == 0:
+        weight, res = 1 + 0.1 * rnd(n, seed=3), rnd(m, n, dtype=torch.bfloat16, seed=4)
+        resd = res.to(gpu)
+        normed = K().rmsnorm(none, weight.to(gpu), 1e-5, residual=resd)
+        total = none.parts.double().sum(0).cpu() + res.double()
+        close(resd, total, torch.bfloat16)
+        close(normed, pm.rms_norm(total, weight.double(), 1e-5), torch.bfloat16)
+    # a row's sums depend neither on the other rows nor on what lies behind X; eight and sixteen wavefronts are both right
+    one = K().gemm_skinny_sliced(xd[m - 1:].contiguous(), tiles, slices=slices)
+    assert torch.equal(one.parts[:, 0], none.parts[:, m - 1])
+    behind = torch.full((m + 8, k), float("nan"), dtype=torch.bfloat16, device=gpu)
+    behind[:m] = xd
+    assert torch.equal(K().gemm_skinny_sliced(behind[:m], tiles, slices=slices).parts, none.parts)
+    for waves in (8, 16):
+        close(K().gemm_skinny_sliced(xd, tiles, slices=slices, waves=waves).parts.double().sum(0), ref, torch.float32, f32=2e-5)
+    from prelude_amd._native import NativeError
+    with pytest.raises(NativeError, match="gemm_skinny_sliced: x"):
+        K().gemm_skinny_sliced(torch.zeros(17, k, dtype=torch.bfloat16, device=gpu), tiles, slices=slices)
+    with pytest.raises(NativeError, match="slices of"):
+        K().check(K().kernels().pa_gemm_skinny_sliced(None, xd.data_ptr(), tiles.data.data_ptr(), None, none.parts.data_ptr(), m, n, k,
+                                                       k, steps + 1, 0))
+
+
+def test_narrow_weights_go_to_the_streaming_kernel_in_slices(gpu):
+    """linear() for a reader of slices: weights of few tiles are cut so that the chip has workgroups enough, at the
+    rows where that measured faster; the same bits as asked for directly; and not for a reader that wants a tensor."""
+    for (n, k, rows, slices) in ((2560, 9728, (4, 8, 12), 3), (2048, 6144, (1, 16), 2), (1024, 3072, (1, 9, 16), 4), (1024, 2048, (2,), 4)):
+        w = rnd(n, k, dtype=torch.bfloat16, seed=n, scale=0.03).to(gpu)
+        lw = K().LinearWeight(w, K().pack_tiles(w))
+        for m in rows:
+            x = rnd(m, k, dtype=torch.bfloat16, seed=m).to(gpu)
+            got = K().linear(x, lw, slices_ok=True)
+            assert isinstance(got, K().SliceSums) and got.parts.shape[0] == slices, (n, k, m)
+            assert torch.equal(got.parts, K().gemm_skinny_sliced(x, lw.tiles, slices=slices, waves=8).parts)
+            assert isinstance(K().linear(x, lw), torch.Tensor)
+            close(K().as_tensor(got), x.double().cpu() @ w.double().cpu().T, torch.bfloat16)
+    w = rnd(2560, 9728, dtype=torch.bfloat16, seed=1, scale=0.03).to(gpu)
+    lw = K().LinearWeight(w, K().pack_tiles(w))
+    for m in (1, 2, 3):       # behind at so few rows: the kernel uncut
+        assert isinstance(K().linear(rnd(m, 9728, dtype=torch.bfloat16).to(gpu), lw, slices_ok=True), torch.Tensor)
+    K().set_skinny_sliced(False)
+    try:
+        assert isinstance(K().linear(rnd(8, 9728, dtype=torch.bfloat16).to(gpu), lw, slices_ok=True), torch.Tensor)
+    finally:
+        K().set_skinny_sliced(True)
+
+
 @pytest.mark.parametrize("m,n,k", [(30, 24, 16), (4, 76, 24), (16, 48, 40), (1, 32, 8), (39, 2304, 24), (64, 40, 72)])
 def test_gemm_skinny_stays_inside_its_rows(gpu, m, n, k):
     """Rows shorter than a step of 64 columns, or ending inside one: what lies behind a row of X is not the
@@ -544,6 +610,12 @@ def test_drawn_products(gpu, seed):
     want5 = pm.silu(g5[:, 0::2]) * g5[:, 1::2]
     err = float((y5.double().cpu() - want5).abs().max())
     assert err <= tol(torch.bfloat16, want5, bf16=1.25e-2), f"{what}, rows {m5}, {waves} wavefronts, norm + SiLU*up: max error {err:.3e}"
+    # the streaming product of up to 16 rows in slices of K
+    s6 = int(rng.integers(1, min(steps, 6) + 1))
+    parts6 = K().gemm_skinny_sliced(x5.to(gpu), tiles, bd, slices=s6, waves=int(rng.choice([0, 8, 16]))).parts
+    ref6 = x5.double() @ w.double().T + b.double()
+    err = float((parts6.double().sum(0).cpu() - ref6).abs().max())
+    assert err <= tol(torch.float32, ref6, f32=2e-5), f"{what}, rows {m5}, streaming kernel in {s6} slices: max error {err:.3e}"
     # the product tiled both ways, at a drawn number of rows, shape of workgroup, activation and number of slices
     m4 = int(rng.choice([1, 129, 192, 256, 257, int(rng.integers(1, 700))]))
     x4 = rnd(m4, k, dtype=torch.bfloat16, seed=seed + 7)

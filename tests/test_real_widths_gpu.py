@@ -134,6 +134,59 @@ def test_the_norm_inside_the_gated_product(gpu, monkeypatch):
         K.set_normed_gated(True)
 
 
+@functools.lru_cache(maxsize=None)
+def narrow_model():
+    """The widths of a small model (Qwen3-0.6B: hidden 1,024, 16 heads over 8 KV heads of 128, intermediate 3,072), three
+    layers, a small vocabulary: its o and down products have 64 tiles of 16 rows, which the streaming kernel cuts
+    into slices of K for the norm behind them."""
+    from prelude_amd.weights import write_safetensors
+    cfg = dict(wide_config(), vocab_size=4099, eos_token_id=4098, hidden_size=1024, intermediate_size=3072,
+               num_attention_heads=16, num_key_value_heads=8, num_hidden_layers=3, max_window_layers=3)
+    w = pm.random_weights(cfg, seed=12, std=0.03, norm_std=0.02)
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    tmp = tempfile.TemporaryDirectory(prefix="prelude_amd_test_narrow_")
+    _keep.append(tmp)
+    with open(os.path.join(tmp.name, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(tmp.name, "model.safetensors"), w)
+    toks = torch.randint(0, cfg["vocab_size"], (80,), generator=torch.Generator().manual_seed(5)).tolist()
+    return tmp.name, toks, pm.forward(cfg, {k: v.double() for k, v in w.items()}, toks)
+
+
+def test_narrow_widths_decode_with_their_products_in_slices(gpu, monkeypatch):
+    """One request decoded token by token and nine decoding together at a small model's widths, where the last
+    product of the attention and of the feed-forward come as slices of K from the streaming kernel: against the
+    plain implementation, and the kernel is seen to run."""
+    from prelude_amd.ops import kernels as K
+    from prelude_amd.trace import TraceRunner
+    folder, toks, ref = narrow_model()
+    calls = []
+    inner = K.gemm_skinny_sliced
+    monkeypatch.setattr(K, "gemm_skinny_sliced", lambda *a, **kw: (calls.append(a[0].shape[0]), inner(*a, **kw))[1])
+    r = TraceRunner(folder, "bfloat16", 10 * 96, page_size=16)
+    n = len(toks)
+    outs = [r.step([{"id": "d", "tokens": toks[:n - 24], "want": list(range(n - 24))}])]
+    for i in range(n - 24, n):
+        outs.append(r.step([{"id": "d", "tokens": [toks[i]], "want": [0]}]))
+    r.step([], ["d"])
+    check(np.concatenate(outs), ref, "bfloat16", "decoded")
+    assert calls and set(calls) == {1}
+    calls.clear()
+    starts = [4 + 7 * i for i in range(9)]
+    for i, s in enumerate(starts):
+        r.step([{"id": f"r{i}", "tokens": toks[:s], "want": []}])
+    rows = [[] for _ in starts]
+    for k in range(4):
+        out = r.step([{"id": f"r{i}", "tokens": [toks[s + k]], "want": [0]} for i, s in enumerate(starts)])
+        for i in range(len(starts)):
+            rows[i].append(out[i:i + 1])
+    for i, s in enumerate(starts):
+        check(np.concatenate(rows[i]), ref[s:s + 4], "bfloat16", f"request {i} from position {s}")
+    assert 9 in calls
+    r.step([], [f"r{i}" for i in range(9)])
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
 def test_graph_replays_equal_eager_steps_at_real_widths(gpu):
     """Decode steps of one, five and twelve requests at these widths (the streaming products, the gated product with
     the norm inside it, the decode attention on the raw projection) replayed from graphs give the bits of the same
